@@ -1,0 +1,170 @@
+/*
+ * bsa_mi355x.h - C ABI of the MI355X (gfx950) block-sparse attention engine.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream
+ * (passed as void*, 0 = the null stream).  Nothing here allocates device
+ * memory, synchronises with the host or keeps mutable global state besides a
+ * thread-local error string; callers own every buffer.  All functions return
+ * BSA_OK (0) or a negative bsa_status; bsa_last_error() describes the last
+ * failure on the calling thread.  Arguments are validated on the host before
+ * anything is launched, so a bad call never reaches the GPU.
+ *
+ * Layouts.  "THW order" is the reference's token order, S = (T, H, W)
+ * row-major.  "Blocked order" is (Nt, Nh, Nw, t, h, w): consecutive runs of
+ * t*h*w slots form one 3-D chunk.  When a grid axis is not a multiple of its
+ * chunk axis it is padded at the high end; padded slots hold zeros and are
+ * flagged invalid in a per-64-slot bit mask ("tile validity", bit s of word i
+ * covers slot 64*i+s).
+ *
+ * Reference interfaces replaced (paths relative to the reference checkout,
+ * bsa = longcat_video/block_sparse_attention/bsa_interface.py,
+ * vmask = longcat_video/block_sparse_attention/flash_attn_bsa_varlen_mask.py):
+ * cited per function below.
+ */
+#ifndef BSA_MI355X_H
+#define BSA_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum bsa_status {
+    BSA_OK = 0,
+    BSA_ERR_BAD_ARG = -1,        /* null pointer, non-positive size, misalignment */
+    BSA_ERR_UNSUPPORTED = -2,    /* dtype / head_dim / chunk size not built */
+    BSA_ERR_SHAPE = -3,          /* sizes inconsistent with each other */
+    BSA_ERR_WORKSPACE = -4,      /* workspace smaller than bsa_workspace_bytes() */
+    BSA_ERR_HIP = -5             /* a HIP call failed; text in bsa_last_error() */
+} bsa_status;
+
+typedef enum bsa_dtype {
+    BSA_BF16 = 0,
+    BSA_F16 = 1,
+    BSA_F32 = 2
+} bsa_dtype;
+
+/* Library version, major*10000 + minor*100 + patch. */
+int bsa_version(void);
+
+/* Text of the last error raised on this thread ("" if none). */
+const char* bsa_last_error(void);
+
+/* Number of KV blocks kept per query block: int((1 - sparsity) * n_kv_blocks)
+ * in IEEE doubles with truncation.  Replaces bsa:214. */
+int bsa_num_selected(double sparsity, int n_kv_blocks);
+
+/* Padded slot count of a (T,H,W) grid cut into (t,h,w) chunks. */
+int64_t bsa_padded_tokens(int T, int H, int W, int t, int h, int w);
+
+/*
+ * R1.  THW order -> blocked order, zero-filling padded slots.
+ * Replaces rearrange_THW_to_3d_block, bsa:600-604 (called bsa:650-652).
+ *   src          [B, Hn, T*H*W, D], element strides src_strides = {B, Hn, S};
+ *                the D axis must be contiguous and every row 16-byte aligned
+ *   dst          [B, Hn, S_padded, D] contiguous
+ *   pooled       optional [B, Hn, n_blocks, D] in `dtype`: per-chunk mean over
+ *                all t*h*w slots (zeros included), fp32 sum, one rounding;
+ *                the same result as bsa_mean_pool on dst (bsa:168-178)
+ *   tile_valid   optional [S_padded/64] uint64 tile validity (needs t*h*w % 64 == 0)
+ */
+int bsa_permute_thw_to_blocks(const void* src, const int64_t src_strides[3], void* dst,
+                              void* pooled, uint64_t* tile_valid,
+                              int B, int Hn, int T, int H, int W, int t, int h, int w,
+                              int D, int dtype, void* stream);
+
+/*
+ * R7.  Blocked order -> THW order, dropping padded slots.
+ * Replaces rearrange_3d_block_to_THW, bsa:606-610 (called bsa:659).
+ *   src [B, Hn, S_padded, D] contiguous; dst [B, Hn, T*H*W, D] with element
+ *   strides dst_strides = {B, Hn, S} (so the caller may point it at a
+ *   [B, S, Hn, D] buffer and skip the transpose of attention.py:140-141).
+ */
+int bsa_unpermute_blocks_to_thw(const void* src, void* dst, const int64_t dst_strides[3],
+                                int B, int Hn, int T, int H, int W, int t, int h, int w,
+                                int D, int dtype, void* stream);
+
+/*
+ * R2.  Block mean pooling.  Replaces mean_pooling_compression, bsa:168-178.
+ *   x [B, Hn, S, D] contiguous; out [B, Hn, ceil(S/block), D] in `dtype`.
+ *   A ragged last block is summed over its real rows and still divided by
+ *   `block` (the reference zero-pads first, bsa:175-177).
+ */
+int bsa_mean_pool(const void* x, void* out, int B, int Hn, int64_t S, int block, int D,
+                  int dtype, void* stream);
+
+/*
+ * R3 + R4.  Pooled scores and top-k selection.
+ * Replaces cal_score (bsa:180-184) and get_select_indices_topk_from_score
+ * (bsa:212-224).
+ *   q_cmp [B, Hn, nbq, D], k_cmp [B, Hn, nbk, D] contiguous, `dtype`
+ *   score = q_cmp . k_cmp^T, fp32 accumulate, rounded once to `dtype`, unscaled
+ *   idx_out   int32 [B, Hn, nbq, k_sel]: the k_sel best blocks of every row in
+ *             descending score order, ties broken towards the lowest index
+ *   lens_out  int32 [B, Hn, nbq], every entry k_sel (bsa:217-222)
+ *   score_out optional [B, Hn, nbq, nbk] in `dtype`
+ * Limits: D == 128, 0 <= k_sel <= nbk <= 4096, k_sel <= 1024.
+ * NaN scores order above +inf, as torch.topk orders them.
+ */
+int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32_t* lens_out,
+                   void* score_out, int B, int Hn, int nbq, int nbk, int D, int k_sel,
+                   int dtype, void* stream);
+
+/* R4 alone, from a caller-supplied score tensor [B, Hn, nbq, nbk] in `dtype`. */
+int bsa_topk_from_score(const void* score, int32_t* idx_out, int32_t* lens_out,
+                        int B, int Hn, int nbq, int nbk, int k_sel, int dtype, void* stream);
+
+/*
+ * R5 + R6.  Block-sparse flash-attention forward over blocked-order tensors.
+ * Replaces attn_fwd_bsa_varlen_triton (bsa:290-341) and the kernel
+ * _attn_fwd_bsa_varlen_align (vmask:172-285).
+ *   q [B, Hn, Sq, D], k/v [B, Hn, Sk, D], o [B, Hn, Sq, D] contiguous
+ *   idx  int32 [B, Hn, Sq/bs_q, idx_stride]; lens int32 [B, Hn, Sq/bs_q];
+ *        row m attends to KV blocks idx[..., m, 0 .. lens[..., m])
+ *   tile_valid optional [Sk/64] uint64: keys whose bit is 0 get -inf logits
+ *   lse  optional fp32 [B, Hn, Sq], natural-log sum-exp (bsa:338-339)
+ *   o = softmax(q k^T * sm_scale) v restricted to the listed blocks; logits are
+ *   fp32, the scale is applied after the dot as sm_scale*log2(e), probabilities
+ *   are rounded to `dtype` for the P V product while the row sum stays fp32.
+ *   An empty list gives o = 0, lse = -inf.
+ * Limits: D == 128; bs_q, bs_k multiples of 64; Sq % bs_q == 0, Sk % bs_k == 0.
+ */
+int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, const int32_t* lens,
+            const uint64_t* tile_valid, void* o, float* lse,
+            int B, int Hn, int64_t Sq, int64_t Sk, int D, int bs_q, int bs_k, int idx_stride,
+            float sm_scale, int dtype, void* stream);
+
+/*
+ * R9.  The whole operator on THW-order tensors: permute q,k,v (+pool), score,
+ * top-k, attention, unpermute.  Replaces flash_attn_bsa_3d, bsa:612-660, and
+ * _attention_bsa.forward, bsa:535-568 (cdf_threshold = None).
+ *   q [B, Hn, Tq*Hq*Wq, D] with element strides q_strides = {B, Hn, S}; same
+ *   for k, v; o likewise with o_strides.  k_sel from bsa_num_selected() on the
+ *   padded KV block count.  workspace: bsa_workspace_bytes() bytes, 256-byte
+ *   aligned.  idx_out/lens_out/score_out are optional copies for inspection
+ *   (shapes as in bsa_score_topk).
+ */
+typedef struct bsa_3d_params {
+    int B, Hn, D, dtype;
+    int Tq, Hq, Wq, Tk, Hk, Wk;      /* latent grids */
+    int tq, hq, wq, tk, hk, wk;      /* chunk shapes */
+    int k_sel;
+    float sm_scale;
+} bsa_3d_params;
+
+size_t bsa_workspace_bytes(const bsa_3d_params* p);
+
+int bsa_fwd_3d(const bsa_3d_params* p,
+               const void* q, const int64_t q_strides[3],
+               const void* k, const int64_t k_strides[3],
+               const void* v, const int64_t v_strides[3],
+               void* o, const int64_t o_strides[3],
+               void* workspace, size_t workspace_bytes,
+               int32_t* idx_out, int32_t* lens_out, void* score_out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BSA_MI355X_H */

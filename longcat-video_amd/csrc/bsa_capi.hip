@@ -1,0 +1,276 @@
+// C ABI of the engine: argument validation, workspace carving, kernel
+// sequencing.  Nothing here allocates device memory or waits for the GPU.
+#include "bsa_common.h"
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+
+namespace bsa {
+
+static thread_local char g_err[512] = "";
+
+int set_error(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+namespace {
+
+inline int hip_fail(hipError_t e, const char* what) {
+    return set_error(BSA_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Row pitch rules shared by the data-movement kernels: rows are moved in
+// 16-byte pieces by groups of lanes whose count divides the workgroup.
+int check_row(int D, int dtype) {
+    const int es = dtype_size(dtype);
+    if (es == 0) return set_error(BSA_ERR_UNSUPPORTED, "unknown dtype %d", dtype);
+    if (D <= 0) return set_error(BSA_ERR_BAD_ARG, "head dim %d must be positive", D);
+    const int bytes = D * es;
+    if (bytes % 16 != 0) return set_error(BSA_ERR_UNSUPPORTED, "row of %d bytes is not a multiple of 16", bytes);
+    const int cpr = bytes / 16;
+    if (cpr > 256 || (256 % cpr) != 0)
+        return set_error(BSA_ERR_UNSUPPORTED, "head dim %d: row pieces (%d) must divide 256", D, cpr);
+    return BSA_OK;
+}
+
+int check_grid(int B, int Hn, int T, int H, int W, int t, int h, int w) {
+    if (B <= 0 || Hn <= 0 || T <= 0 || H <= 0 || W <= 0 || t <= 0 || h <= 0 || w <= 0)
+        return set_error(BSA_ERR_BAD_ARG, "sizes must be positive (B=%d heads=%d grid=%dx%dx%d chunk=%dx%dx%d)",
+                         B, Hn, T, H, W, t, h, w);
+    if ((int64_t)B * Hn > 65535) return set_error(BSA_ERR_UNSUPPORTED, "B*heads = %lld exceeds 65535", (long long)B * Hn);
+    return BSA_OK;
+}
+
+int check_strides(const int64_t s[3], int D, int dtype, const char* name) {
+    if (s == nullptr) return set_error(BSA_ERR_BAD_ARG, "%s strides are null", name);
+    const int es = dtype_size(dtype);
+    for (int i = 0; i < 3; ++i) {
+        if (s[i] < 0) return set_error(BSA_ERR_BAD_ARG, "%s stride %d is negative", name, i);
+        if ((s[i] * es) % 16 != 0)
+            return set_error(BSA_ERR_BAD_ARG, "%s stride %d (%lld elements) breaks 16-byte row alignment", name, i, (long long)s[i]);
+    }
+    if (s[2] < D) return set_error(BSA_ERR_BAD_ARG, "%s token stride %lld is smaller than head dim %d", name, (long long)s[2], D);
+    return BSA_OK;
+}
+
+}  // namespace
+}  // namespace bsa
+
+using namespace bsa;
+
+#define BSA_TRY(expr)                   \
+    do {                                \
+        const int rc_ = (expr);         \
+        if (rc_ != BSA_OK) return rc_;  \
+    } while (0)
+
+extern "C" {
+
+int bsa_version(void) { return 100; }
+
+const char* bsa_last_error(void) { return g_err; }
+
+int bsa_num_selected(double sparsity, int n_kv_blocks) {
+    return (int)((1.0 - sparsity) * (double)n_kv_blocks);
+}
+
+int64_t bsa_padded_tokens(int T, int H, int W, int t, int h, int w) {
+    if (T <= 0 || H <= 0 || W <= 0 || t <= 0 || h <= 0 || w <= 0) return -1;
+    const Grid3 g = make_grid(T, H, W, t, h, w);
+    return (int64_t)g.blocks() * g.chunk();
+}
+
+int bsa_permute_thw_to_blocks(const void* src, const int64_t src_strides[3], void* dst, void* pooled,
+                              uint64_t* tile_valid, int B, int Hn, int T, int H, int W, int t, int h,
+                              int w, int D, int dtype, void* stream) {
+    if (!src || !dst) return set_error(BSA_ERR_BAD_ARG, "permute: src/dst is null");
+    BSA_TRY(check_row(D, dtype));
+    BSA_TRY(check_grid(B, Hn, T, H, W, t, h, w));
+    BSA_TRY(check_strides(src_strides, D, dtype, "src"));
+    if (!aligned16(src) || !aligned16(dst)) return set_error(BSA_ERR_BAD_ARG, "permute: pointers must be 16-byte aligned");
+    const Grid3 g = make_grid(T, H, W, t, h, w);
+    if (tile_valid && g.chunk() % 64 != 0)
+        return set_error(BSA_ERR_UNSUPPORTED, "tile validity needs a chunk of a multiple of 64 tokens, got %d", g.chunk());
+    const hipError_t e = launch_permute(src, src_strides, dst, pooled, tile_valid, B, Hn, g, D, dtype, (hipStream_t)stream);
+    return e == hipSuccess ? BSA_OK : hip_fail(e, "permute launch");
+}
+
+int bsa_unpermute_blocks_to_thw(const void* src, void* dst, const int64_t dst_strides[3], int B, int Hn,
+                                int T, int H, int W, int t, int h, int w, int D, int dtype, void* stream) {
+    if (!src || !dst) return set_error(BSA_ERR_BAD_ARG, "unpermute: src/dst is null");
+    BSA_TRY(check_row(D, dtype));
+    BSA_TRY(check_grid(B, Hn, T, H, W, t, h, w));
+    BSA_TRY(check_strides(dst_strides, D, dtype, "dst"));
+    if (!aligned16(src) || !aligned16(dst)) return set_error(BSA_ERR_BAD_ARG, "unpermute: pointers must be 16-byte aligned");
+    const Grid3 g = make_grid(T, H, W, t, h, w);
+    const hipError_t e = launch_unpermute(src, dst, dst_strides, B, Hn, g, D, dtype, (hipStream_t)stream);
+    return e == hipSuccess ? BSA_OK : hip_fail(e, "unpermute launch");
+}
+
+int bsa_mean_pool(const void* x, void* out, int B, int Hn, int64_t S, int block, int D, int dtype, void* stream) {
+    if (!x || !out) return set_error(BSA_ERR_BAD_ARG, "mean_pool: x/out is null");
+    BSA_TRY(check_row(D, dtype));
+    if (B <= 0 || Hn <= 0 || S <= 0 || block <= 0)
+        return set_error(BSA_ERR_BAD_ARG, "mean_pool: sizes must be positive (B=%d heads=%d S=%lld block=%d)", B, Hn, (long long)S, block);
+    if ((int64_t)B * Hn > 65535) return set_error(BSA_ERR_UNSUPPORTED, "B*heads exceeds 65535");
+    if (!aligned16(x)) return set_error(BSA_ERR_BAD_ARG, "mean_pool: x must be 16-byte aligned");
+    const hipError_t e = launch_mean_pool(x, out, B, Hn, S, block, D, dtype, (hipStream_t)stream);
+    return e == hipSuccess ? BSA_OK : hip_fail(e, "mean_pool launch");
+}
+
+static int check_topk(int B, int Hn, int nbq, int nbk, int k_sel, int dtype) {
+    if (dtype_size(dtype) == 0) return set_error(BSA_ERR_UNSUPPORTED, "unknown dtype %d", dtype);
+    if (B <= 0 || Hn <= 0 || nbq <= 0 || nbk <= 0)
+        return set_error(BSA_ERR_BAD_ARG, "top-k: sizes must be positive (B=%d heads=%d nbq=%d nbk=%d)", B, Hn, nbq, nbk);
+    if (k_sel < 0 || k_sel > nbk) return set_error(BSA_ERR_SHAPE, "top-k: k_sel=%d outside [0, %d]", k_sel, nbk);
+    if (nbk > 4096) return set_error(BSA_ERR_UNSUPPORTED, "top-k: %d KV blocks exceed the limit of 4096", nbk);
+    if (k_sel > 1024) return set_error(BSA_ERR_UNSUPPORTED, "top-k: k_sel=%d exceeds the limit of 1024", k_sel);
+    return BSA_OK;
+}
+
+int bsa_topk_from_score(const void* score, int32_t* idx_out, int32_t* lens_out, int B, int Hn, int nbq,
+                        int nbk, int k_sel, int dtype, void* stream) {
+    if (!score || !idx_out || !lens_out) return set_error(BSA_ERR_BAD_ARG, "top-k: null pointer");
+    BSA_TRY(check_topk(B, Hn, nbq, nbk, k_sel, dtype));
+    const hipError_t e = launch_topk(score, idx_out, lens_out, (int64_t)B * Hn * nbq, nbk, k_sel, dtype, (hipStream_t)stream);
+    return e == hipSuccess ? BSA_OK : hip_fail(e, "top-k launch");
+}
+
+int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32_t* lens_out, void* score_out,
+                   int B, int Hn, int nbq, int nbk, int D, int k_sel, int dtype, void* stream) {
+    if (!q_cmp || !k_cmp || !idx_out || !lens_out) return set_error(BSA_ERR_BAD_ARG, "score_topk: null pointer");
+    if (!score_out) return set_error(BSA_ERR_BAD_ARG, "score_topk: a score buffer of B*heads*nbq*nbk elements is required");
+    BSA_TRY(check_topk(B, Hn, nbq, nbk, k_sel, dtype));
+    if (D <= 0 || D % 16 != 0 || D > 256) return set_error(BSA_ERR_UNSUPPORTED, "score: head dim %d must be a multiple of 16, at most 256", D);
+    if ((int64_t)B * Hn > 65535) return set_error(BSA_ERR_UNSUPPORTED, "B*heads exceeds 65535");
+    if (!aligned16(q_cmp) || !aligned16(k_cmp)) return set_error(BSA_ERR_BAD_ARG, "score: pooled tensors must be 16-byte aligned");
+    hipError_t e = launch_score(q_cmp, k_cmp, score_out, B * Hn, nbq, nbk, D, dtype, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "score launch");
+    e = launch_topk(score_out, idx_out, lens_out, (int64_t)B * Hn * nbq, nbk, k_sel, dtype, (hipStream_t)stream);
+    return e == hipSuccess ? BSA_OK : hip_fail(e, "top-k launch");
+}
+
+int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, const int32_t* lens,
+            const uint64_t* tile_valid, void* o, float* lse, int B, int Hn, int64_t Sq, int64_t Sk, int D,
+            int bs_q, int bs_k, int idx_stride, float sm_scale, int dtype, void* stream) {
+    if (!q || !k || !v || !idx || !lens || !o) return set_error(BSA_ERR_BAD_ARG, "fwd: null pointer");
+    if (dtype_size(dtype) == 0) return set_error(BSA_ERR_UNSUPPORTED, "unknown dtype %d", dtype);
+    if (D != 128) return set_error(BSA_ERR_UNSUPPORTED, "fwd: head dim %d is not built (only 128)", D);
+    if (B <= 0 || Hn <= 0 || Sq <= 0 || Sk <= 0 || idx_stride < 0)
+        return set_error(BSA_ERR_BAD_ARG, "fwd: sizes must be positive (B=%d heads=%d Sq=%lld Sk=%lld)", B, Hn, (long long)Sq, (long long)Sk);
+    if ((int64_t)B * Hn > 65535) return set_error(BSA_ERR_UNSUPPORTED, "B*heads exceeds 65535");
+    if (bs_q <= 0 || bs_k <= 0 || bs_q % 64 != 0 || bs_k % 64 != 0)
+        return set_error(BSA_ERR_UNSUPPORTED, "fwd: chunk sizes %d/%d must be multiples of 64", bs_q, bs_k);
+    if (Sq % bs_q != 0 || Sk % bs_k != 0)
+        return set_error(BSA_ERR_SHAPE, "fwd: Sq=%lld / Sk=%lld are not multiples of the chunk sizes %d / %d", (long long)Sq, (long long)Sk, bs_q, bs_k);
+    if (!(sm_scale > 0.f) || !std::isfinite(sm_scale)) return set_error(BSA_ERR_BAD_ARG, "fwd: sm_scale must be positive and finite");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
+        return set_error(BSA_ERR_BAD_ARG, "fwd: q/k/v/o must be 16-byte aligned");
+    const hipError_t e = launch_fwd(q, k, v, idx, lens, tile_valid, o, lse, B, Hn, Sq, Sk, bs_q, bs_k, idx_stride,
+                                    sm_scale, dtype, (hipStream_t)stream);
+    return e == hipSuccess ? BSA_OK : hip_fail(e, "fwd launch");
+}
+
+// ---- whole operator -------------------------------------------------------
+namespace {
+struct Plan {
+    Grid3 gq, gk;
+    int64_t Sqp, Skp;
+    int nbq, nbk, es;
+    size_t off_qp, off_kp, off_vp, off_op, off_qc, off_kc, off_score, off_idx, off_lens, off_valid, total;
+};
+inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+int make_plan(const bsa_3d_params* p, Plan* pl) {
+    if (!p) return set_error(BSA_ERR_BAD_ARG, "params are null");
+    BSA_TRY(check_row(p->D, p->dtype));
+    BSA_TRY(check_grid(p->B, p->Hn, p->Tq, p->Hq, p->Wq, p->tq, p->hq, p->wq));
+    BSA_TRY(check_grid(p->B, p->Hn, p->Tk, p->Hk, p->Wk, p->tk, p->hk, p->wk));
+    if (p->D != 128) return set_error(BSA_ERR_UNSUPPORTED, "head dim %d is not built (only 128)", p->D);
+    pl->gq = make_grid(p->Tq, p->Hq, p->Wq, p->tq, p->hq, p->wq);
+    pl->gk = make_grid(p->Tk, p->Hk, p->Wk, p->tk, p->hk, p->wk);
+    if (pl->gq.chunk() % 64 != 0 || pl->gk.chunk() % 64 != 0)
+        return set_error(BSA_ERR_UNSUPPORTED, "chunk sizes %d/%d must be multiples of 64 tokens", pl->gq.chunk(), pl->gk.chunk());
+    pl->nbq = pl->gq.blocks();
+    pl->nbk = pl->gk.blocks();
+    BSA_TRY(check_topk(p->B, p->Hn, pl->nbq, pl->nbk, p->k_sel, p->dtype));
+    if (!(p->sm_scale > 0.f) || !std::isfinite(p->sm_scale)) return set_error(BSA_ERR_BAD_ARG, "sm_scale must be positive and finite");
+    pl->Sqp = (int64_t)pl->nbq * pl->gq.chunk();
+    pl->Skp = (int64_t)pl->nbk * pl->gk.chunk();
+    pl->es = dtype_size(p->dtype);
+    const size_t bh = (size_t)p->B * p->Hn;
+    size_t off = 0;
+    auto take = [&](size_t bytes) { const size_t o = off; off += up256(bytes); return o; };
+    pl->off_qp = take(bh * pl->Sqp * p->D * pl->es);
+    pl->off_kp = take(bh * pl->Skp * p->D * pl->es);
+    pl->off_vp = take(bh * pl->Skp * p->D * pl->es);
+    pl->off_op = take(bh * pl->Sqp * p->D * pl->es);
+    pl->off_qc = take(bh * pl->nbq * p->D * pl->es);
+    pl->off_kc = take(bh * pl->nbk * p->D * pl->es);
+    pl->off_score = take(bh * pl->nbq * (size_t)pl->nbk * pl->es);
+    pl->off_idx = take(bh * pl->nbq * (size_t)(p->k_sel > 0 ? p->k_sel : 1) * sizeof(int32_t));
+    pl->off_lens = take(bh * pl->nbq * sizeof(int32_t));
+    pl->off_valid = take((size_t)(pl->Skp / 64) * sizeof(uint64_t));
+    pl->total = off;
+    return BSA_OK;
+}
+}  // namespace
+
+size_t bsa_workspace_bytes(const bsa_3d_params* p) {
+    Plan pl;
+    if (make_plan(p, &pl) != BSA_OK) return 0;
+    return pl.total;
+}
+
+int bsa_fwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3], const void* k,
+               const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
+               const int64_t o_strides[3], void* workspace, size_t workspace_bytes, int32_t* idx_out,
+               int32_t* lens_out, void* score_out, void* stream) {
+    Plan pl;
+    BSA_TRY(make_plan(p, &pl));
+    if (!q || !k || !v || !o || !workspace) return set_error(BSA_ERR_BAD_ARG, "fwd_3d: null pointer");
+    if (workspace_bytes < pl.total)
+        return set_error(BSA_ERR_WORKSPACE, "fwd_3d: workspace of %zu bytes is smaller than the %zu required", workspace_bytes, pl.total);
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return set_error(BSA_ERR_BAD_ARG, "fwd_3d: workspace must be 256-byte aligned");
+    BSA_TRY(check_strides(q_strides, p->D, p->dtype, "q"));
+    BSA_TRY(check_strides(k_strides, p->D, p->dtype, "k"));
+    BSA_TRY(check_strides(v_strides, p->D, p->dtype, "v"));
+    BSA_TRY(check_strides(o_strides, p->D, p->dtype, "o"));
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
+        return set_error(BSA_ERR_BAD_ARG, "fwd_3d: q/k/v/o must be 16-byte aligned");
+
+    char* ws = static_cast<char*>(workspace);
+    void* qp = ws + pl.off_qp; void* kp = ws + pl.off_kp; void* vp = ws + pl.off_vp; void* op = ws + pl.off_op;
+    void* qc = ws + pl.off_qc; void* kc = ws + pl.off_kc; void* score = ws + pl.off_score;
+    int32_t* idx = reinterpret_cast<int32_t*>(ws + pl.off_idx);
+    int32_t* lens = reinterpret_cast<int32_t*>(ws + pl.off_lens);
+    uint64_t* valid = reinterpret_cast<uint64_t*>(ws + pl.off_valid);
+    const bool padded_k = (p->Tk % p->tk) || (p->Hk % p->hk) || (p->Wk % p->wk);
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e;
+#define BSA_HIP(call, what) do { e = (call); if (e != hipSuccess) return hip_fail(e, what); } while (0)
+    BSA_HIP(launch_permute(q, q_strides, qp, qc, nullptr, p->B, p->Hn, pl.gq, p->D, p->dtype, st), "permute q");
+    BSA_HIP(launch_permute(k, k_strides, kp, kc, padded_k ? valid : nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st), "permute k");
+    BSA_HIP(launch_permute(v, v_strides, vp, nullptr, nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st), "permute v");
+    BSA_HIP(launch_score(qc, kc, score, p->B * p->Hn, pl.nbq, pl.nbk, p->D, p->dtype, st), "score");
+    BSA_HIP(launch_topk(score, idx, lens, (int64_t)p->B * p->Hn * pl.nbq, pl.nbk, p->k_sel, p->dtype, st), "top-k");
+    BSA_HIP(launch_fwd(qp, kp, vp, idx, lens, padded_k ? valid : nullptr, op, nullptr, p->B, p->Hn, pl.Sqp, pl.Skp,
+                       pl.gq.chunk(), pl.gk.chunk(), p->k_sel, p->sm_scale, p->dtype, st), "attention");
+    BSA_HIP(launch_unpermute(op, o, o_strides, p->B, p->Hn, pl.gq, p->D, p->dtype, st), "unpermute");
+    const size_t bh = (size_t)p->B * p->Hn;
+    if (idx_out && p->k_sel > 0)
+        BSA_HIP(hipMemcpyAsync(idx_out, idx, bh * pl.nbq * p->k_sel * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy idx");
+    if (lens_out) BSA_HIP(hipMemcpyAsync(lens_out, lens, bh * pl.nbq * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy lens");
+    if (score_out) BSA_HIP(hipMemcpyAsync(score_out, score, bh * pl.nbq * (size_t)pl.nbk * pl.es, hipMemcpyDeviceToDevice, st), "copy score");
+#undef BSA_HIP
+    return BSA_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,191 @@
+// 3-D chunk permute / unpermute and block mean pooling (HBM-bound kernels).
+//
+// One workgroup moves one chunk (t*h*w slots of D elements).  Rows are moved
+// as 16-byte pieces: the D/EPV lanes that share a row read one contiguous row
+// (256 B for D=128 bf16) and consecutive row groups walk the w-run, so both
+// the gather from THW order and the store to blocked order are coalesced.
+// The pooled mean is accumulated on the fly from the registers that already
+// hold the row, so q and k are read from HBM once for permute + pool.
+#include "bsa_common.h"
+
+namespace bsa {
+namespace {
+
+constexpr int kThreads = 256;
+
+template <typename T> struct Piece { static constexpr int EPV = 16 / sizeof(T); };
+
+template <typename T>
+__device__ inline void accumulate(float* acc, const uint4& v) {
+    constexpr int EPV = Piece<T>::EPV;
+    const T* e = reinterpret_cast<const T*>(&v);
+#pragma unroll
+    for (int i = 0; i < EPV; ++i) acc[i] += (float)e[i];
+}
+
+// Sum the per-row-group partials in a fixed order (row group ascending) and
+// store mean = sum * (1/bs) rounded once to T.
+template <typename T>
+__device__ inline void finish_pool(float* acc, float* red, T* out_row, int cpr, int c, int rg,
+                                   int RG, float inv_bs) {
+    constexpr int EPV = Piece<T>::EPV;
+    const int D = cpr * EPV;
+#pragma unroll
+    for (int i = 0; i < EPV; ++i) red[rg * D + c * EPV + i] = acc[i];
+    __syncthreads();
+    for (int d = threadIdx.x; d < D; d += kThreads) {
+        float s = 0.f;
+        for (int g = 0; g < RG; ++g) s += red[g * D + d];
+        out_row[d] = (T)(s * inv_bs);
+    }
+}
+
+template <typename T, bool POOL>
+__global__ __launch_bounds__(kThreads) void permute_kernel(
+    const T* __restrict__ src, int64_t sB, int64_t sH, int64_t sS, T* __restrict__ dst,
+    T* __restrict__ pooled, uint64_t* __restrict__ tile_valid, Grid3 g, int Hn, int D) {
+    extern __shared__ float red[];
+    constexpr int EPV = Piece<T>::EPV;
+    const int blk = blockIdx.x;
+    const int bh = blockIdx.y;
+    const int b = bh / Hn, hd = bh % Hn;
+    const int nw = blk % g.Nw, nh = (blk / g.Nw) % g.Nh, nt = blk / (g.Nw * g.Nh);
+    const int bs = g.chunk();
+    const int nb = g.blocks();
+    const int cpr = D / EPV;
+    const int c = threadIdx.x % cpr, rg = threadIdx.x / cpr, RG = kThreads / cpr;
+    const T* sbase = src + (int64_t)b * sB + (int64_t)hd * sH;
+    T* dbase = dst + ((int64_t)bh * nb + blk) * bs * D;
+    float acc[EPV];
+#pragma unroll
+    for (int i = 0; i < EPV; ++i) acc[i] = 0.f;
+
+    for (int r = rg; r < bs; r += RG) {
+        const int wi = r % g.w, hi = (r / g.w) % g.h, ti = r / (g.w * g.h);
+        const int tt = nt * g.t + ti, hh = nh * g.h + hi, ww = nw * g.w + wi;
+        uint4 val = make_uint4(0, 0, 0, 0);
+        if (tt < g.T && hh < g.H && ww < g.W) {
+            const int64_t s = ((int64_t)tt * g.H + hh) * g.W + ww;
+            val = *reinterpret_cast<const uint4*>(sbase + s * sS + c * EPV);
+        }
+        *reinterpret_cast<uint4*>(dbase + (int64_t)r * D + c * EPV) = val;
+        if (POOL) accumulate<T>(acc, val);
+    }
+    if (tile_valid != nullptr && bh == 0) {
+        // bit s of word i <=> slot 64*i+s of the blocked order holds a real token
+        for (int r0 = (threadIdx.x / 64) * 64; r0 < bs; r0 += kThreads) {
+            const int r = r0 + (threadIdx.x & 63);
+            const int wi = r % g.w, hi = (r / g.w) % g.h, ti = r / (g.w * g.h);
+            const bool ok = nt * g.t + ti < g.T && nh * g.h + hi < g.H && nw * g.w + wi < g.W;
+            const uint64_t m = __ballot(ok);
+            if ((threadIdx.x & 63) == 0) tile_valid[((int64_t)blk * bs + r0) / 64] = m;
+        }
+    }
+    if (POOL)
+        finish_pool<T>(acc, red, pooled + ((int64_t)bh * nb + blk) * D, cpr, c, rg, RG, 1.0f / bs);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void unpermute_kernel(
+    const T* __restrict__ src, T* __restrict__ dst, int64_t sB, int64_t sH, int64_t sS, Grid3 g,
+    int Hn, int D) {
+    constexpr int EPV = Piece<T>::EPV;
+    const int blk = blockIdx.x;
+    const int bh = blockIdx.y;
+    const int b = bh / Hn, hd = bh % Hn;
+    const int nw = blk % g.Nw, nh = (blk / g.Nw) % g.Nh, nt = blk / (g.Nw * g.Nh);
+    const int bs = g.chunk();
+    const int nb = g.blocks();
+    const int cpr = D / EPV;
+    const int c = threadIdx.x % cpr, rg = threadIdx.x / cpr, RG = kThreads / cpr;
+    const T* sbase = src + ((int64_t)bh * nb + blk) * bs * D;
+    T* dbase = dst + (int64_t)b * sB + (int64_t)hd * sH;
+    for (int r = rg; r < bs; r += RG) {
+        const int wi = r % g.w, hi = (r / g.w) % g.h, ti = r / (g.w * g.h);
+        const int tt = nt * g.t + ti, hh = nh * g.h + hi, ww = nw * g.w + wi;
+        if (tt < g.T && hh < g.H && ww < g.W) {
+            const int64_t s = ((int64_t)tt * g.H + hh) * g.W + ww;
+            *reinterpret_cast<uint4*>(dbase + s * sS + c * EPV) =
+                *reinterpret_cast<const uint4*>(sbase + (int64_t)r * D + c * EPV);
+        }
+    }
+}
+
+// Mean over consecutive `block`-row groups of a contiguous [BH, S, D] tensor.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void mean_pool_kernel(const T* __restrict__ x,
+                                                            T* __restrict__ out, int64_t S,
+                                                            int block, int nb, int D) {
+    extern __shared__ float red[];
+    constexpr int EPV = Piece<T>::EPV;
+    const int blk = blockIdx.x;
+    const int bh = blockIdx.y;
+    const int cpr = D / EPV;
+    const int c = threadIdx.x % cpr, rg = threadIdx.x / cpr, RG = kThreads / cpr;
+    const T* base = x + (int64_t)bh * S * D;
+    float acc[EPV];
+#pragma unroll
+    for (int i = 0; i < EPV; ++i) acc[i] = 0.f;
+    for (int r = rg; r < block; r += RG) {
+        const int64_t s = (int64_t)blk * block + r;
+        if (s < S) accumulate<T>(acc, *reinterpret_cast<const uint4*>(base + s * D + c * EPV));
+    }
+    finish_pool<T>(acc, red, out + ((int64_t)bh * nb + blk) * D, cpr, c, rg, RG, 1.0f / block);
+}
+
+inline size_t red_bytes(int D, int esize) {
+    const int cpr = D / (16 / esize);
+    return (size_t)(kThreads / cpr) * D * sizeof(float);
+}
+
+}  // namespace
+
+hipError_t launch_permute(const void* src, const int64_t st3[3], void* dst, void* pooled,
+                          uint64_t* tile_valid, int B, int Hn, const Grid3& g, int D, int dtype,
+                          hipStream_t st) {
+    dim3 grid(g.blocks(), B * Hn), block(kThreads);
+    const size_t smem = pooled ? red_bytes(D, dtype_size(dtype)) : 0;
+#define BSA_LAUNCH(T)                                                                          \
+    if (pooled)                                                                                \
+        hipLaunchKernelGGL((permute_kernel<T, true>), grid, block, smem, st, (const T*)src,     \
+                           st3[0], st3[1], st3[2], (T*)dst, (T*)pooled, tile_valid, g, Hn, D);  \
+    else                                                                                       \
+        hipLaunchKernelGGL((permute_kernel<T, false>), grid, block, smem, st, (const T*)src,    \
+                           st3[0], st3[1], st3[2], (T*)dst, (T*)pooled, tile_valid, g, Hn, D);
+    if (dtype == BSA_BF16) { BSA_LAUNCH(__bf16) }
+    else if (dtype == BSA_F16) { BSA_LAUNCH(_Float16) }
+    else { BSA_LAUNCH(float) }
+#undef BSA_LAUNCH
+    return hipGetLastError();
+}
+
+hipError_t launch_unpermute(const void* src, void* dst, const int64_t st3[3], int B, int Hn,
+                            const Grid3& g, int D, int dtype, hipStream_t st) {
+    dim3 grid(g.blocks(), B * Hn), block(kThreads);
+    if (dtype == BSA_F32)
+        hipLaunchKernelGGL((unpermute_kernel<float>), grid, block, 0, st, (const float*)src,
+                           (float*)dst, st3[0], st3[1], st3[2], g, Hn, D);
+    else  // 16-bit types move as raw bits
+        hipLaunchKernelGGL((unpermute_kernel<uint16_t>), grid, block, 0, st, (const uint16_t*)src,
+                           (uint16_t*)dst, st3[0], st3[1], st3[2], g, Hn, D);
+    return hipGetLastError();
+}
+
+hipError_t launch_mean_pool(const void* x, void* out, int B, int Hn, int64_t S, int block, int D,
+                            int dtype, hipStream_t st) {
+    const int nb = (int)((S + block - 1) / block);
+    dim3 grid(nb, B * Hn), blk(kThreads);
+    const size_t smem = red_bytes(D, dtype_size(dtype));
+    if (dtype == BSA_BF16)
+        hipLaunchKernelGGL((mean_pool_kernel<__bf16>), grid, blk, smem, st, (const __bf16*)x,
+                           (__bf16*)out, S, block, nb, D);
+    else if (dtype == BSA_F16)
+        hipLaunchKernelGGL((mean_pool_kernel<_Float16>), grid, blk, smem, st, (const _Float16*)x,
+                           (_Float16*)out, S, block, nb, D);
+    else
+        hipLaunchKernelGGL((mean_pool_kernel<float>), grid, blk, smem, st, (const float*)x,
+                           (float*)out, S, block, nb, D);
+    return hipGetLastError();
+}
+
+}  // namespace bsa

@@ -1,0 +1,321 @@
+"""Host side of the block-sparse attention operator.
+
+Mirrors the call surface of the reference module
+``longcat_video/block_sparse_attention/bsa_interface.py`` (names, argument
+order and meaning, error types) so that ``Attention._process_attn``
+(longcat_video/modules/attention.py:58-67) can call it unchanged.  Every
+function here only validates, allocates torch tensors and calls the C-ABI of
+the gfx950 engine; there is no eager or CPU implementation behind it.
+
+Differences from the reference, all supersets:
+  * grids that are not chunk multiples are padded at the high end (zeros,
+    padded keys masked, padded query rows dropped) instead of raising; pass
+    ``allow_padding=False`` for the reference's AssertionError
+    (bsa_interface.py:639-640);
+  * block indices are int32 inside the engine; the helpers that the reference
+    returns int64 from (torch.topk) convert on the way out;
+  * forward only: inputs that require grad are rejected while grad mode is on;
+  * ``cdf_threshold`` other than None raises NotImplementedError.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from .. import _capi
+
+_DTYPES = {torch.bfloat16: _capi.BSA_BF16, torch.float16: _capi.BSA_F16, torch.float32: _capi.BSA_F32}
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise NotImplementedError("dtype %s is not supported (bf16, fp16, fp32)" % t.dtype)
+
+
+def _need_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("the block-sparse attention engine runs on the GPU only; got a %s tensor" % t.device)
+
+
+def _no_grad(*tensors: torch.Tensor) -> None:
+    if torch.is_grad_enabled() and any(t.requires_grad for t in tensors):
+        raise RuntimeError("block-sparse attention is forward-only here; call it under torch.no_grad()")
+
+
+def _stream(t: torch.Tensor) -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> C.c_void_p:
+    return C.c_void_p(None if t is None else t.data_ptr())
+
+
+def _rows_ok(t: torch.Tensor) -> torch.Tensor:
+    """[B,H,S,D] with a contiguous, 16-byte aligned D axis; anything else is copied."""
+    es = t.element_size()
+    ok = t.stride(3) == 1 and t.data_ptr() % 16 == 0 and all((t.stride(i) * es) % 16 == 0 for i in range(3))
+    return t if ok else t.contiguous()
+
+
+def num_selected(sparsity: float, n_kv_blocks: int) -> int:
+    """bsa_interface.py:214: ``int((1 - sparsity) * n_blocks)`` in Python doubles."""
+    return int((1 - sparsity) * n_kv_blocks)
+
+
+# ---------------------------------------------------------------------------
+# R1 / R7: 3-D chunk permute and its inverse
+# ---------------------------------------------------------------------------
+def _permute(x, latent_shape, chunk, want_pooled=False, want_valid=False):
+    _need_gpu(x)
+    B, H, S, D = x.shape
+    T, Hh, W = (int(v) for v in latent_shape)
+    t, h, w = (int(v) for v in chunk)
+    assert T * Hh * W == S, "latent shape %s does not match %d tokens" % ((T, Hh, W), S)
+    x = _rows_ok(x)
+    lib = _capi.load()
+    Sp = lib.bsa_padded_tokens(T, Hh, W, t, h, w)
+    nb = Sp // (t * h * w)
+    out = torch.empty(B, H, Sp, D, dtype=x.dtype, device=x.device)
+    pooled = torch.empty(B, H, nb, D, dtype=x.dtype, device=x.device) if want_pooled else None
+    valid = torch.empty(Sp // 64, dtype=torch.int64, device=x.device) if want_valid else None
+    with torch.cuda.device(x.device):
+        _capi.check(lib.bsa_permute_thw_to_blocks(
+            _ptr(x), _capi.strides3(x.stride()[:3]), _ptr(out), _ptr(pooled), _ptr(valid),
+            B, H, T, Hh, W, t, h, w, D, _code(x), _stream(x)), "permute")
+    return out, pooled, valid
+
+
+def rearrange_THW_to_3d_block(x, Nt, Nh, Nw, t, h, w, D=None, latent_shape=None):
+    """bsa_interface.py:600-604.  ``latent_shape`` (T,H,W) may be given when the
+    grid is not a chunk multiple; it defaults to (Nt*t, Nh*h, Nw*w)."""
+    if latent_shape is None:
+        latent_shape = (Nt * t, Nh * h, Nw * w)
+    return _permute(x, latent_shape, (t, h, w))[0]
+
+
+def rearrange_3d_block_to_THW(x, Nt, Nh, Nw, t, h, w, D=None, latent_shape=None):
+    """bsa_interface.py:606-610; padded slots are dropped."""
+    _need_gpu(x)
+    if latent_shape is None:
+        latent_shape = (Nt * t, Nh * h, Nw * w)
+    T, Hh, W = (int(v) for v in latent_shape)
+    B, H, Sp, Dd = x.shape
+    assert Sp == Nt * Nh * Nw * t * h * w, "blocked tensor has %d slots, expected %d" % (Sp, Nt * Nh * Nw * t * h * w)
+    x = x.contiguous()
+    out = torch.empty(B, H, T * Hh * W, Dd, dtype=x.dtype, device=x.device)
+    lib = _capi.load()
+    with torch.cuda.device(x.device):
+        _capi.check(lib.bsa_unpermute_blocks_to_thw(
+            _ptr(x), _ptr(out), _capi.strides3(out.stride()[:3]), B, H, T, Hh, W, t, h, w, Dd, _code(x),
+            _stream(x)), "unpermute")
+    return out
+
+
+# ---------------------------------------------------------------------------
+# R2 - R4: gating
+# ---------------------------------------------------------------------------
+def mean_pooling_compression(x: torch.Tensor, block_size: int) -> torch.Tensor:
+    """bsa_interface.py:168-178."""
+    _need_gpu(x)
+    B, H, S, D = x.shape
+    x = x.contiguous()
+    nb = math.ceil(S / block_size)
+    out = torch.empty(B, H, nb, D, dtype=x.dtype, device=x.device)
+    lib = _capi.load()
+    with torch.cuda.device(x.device):
+        _capi.check(lib.bsa_mean_pool(_ptr(x), _ptr(out), B, H, S, int(block_size), D, _code(x), _stream(x)), "mean_pool")
+    return out
+
+
+def _score_topk(q_cmp, k_cmp, k_sel):
+    _need_gpu(q_cmp, k_cmp)
+    B, H, nbq, D = q_cmp.shape
+    nbk = k_cmp.shape[2]
+    assert k_cmp.shape[0] == B and k_cmp.shape[1] == H and k_cmp.shape[3] == D
+    q_cmp, k_cmp = q_cmp.contiguous(), k_cmp.contiguous()
+    score = torch.empty(B, H, nbq, nbk, dtype=q_cmp.dtype, device=q_cmp.device)
+    idx = torch.empty(B * H * nbq * max(k_sel, 1), dtype=torch.int32, device=q_cmp.device)
+    idx = idx[: B * H * nbq * k_sel].view(B, H, nbq, k_sel)     # never a null pointer, even for k_sel == 0
+    lens = torch.empty(B, H, nbq, dtype=torch.int32, device=q_cmp.device)
+    lib = _capi.load()
+    with torch.cuda.device(q_cmp.device):
+        _capi.check(lib.bsa_score_topk(_ptr(q_cmp), _ptr(k_cmp), _ptr(idx), _ptr(lens), _ptr(score),
+                                       B, H, nbq, nbk, D, k_sel, _code(q_cmp), _stream(q_cmp)), "score_topk")
+    return idx, lens, score
+
+
+def cal_score(q: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
+    """bsa_interface.py:180-184: unscaled ``q @ k^T`` in the input dtype."""
+    return _score_topk(q, k, 0)[2]
+
+
+def get_select_indices_topk_from_score(score: torch.Tensor, sparsity: float):
+    """bsa_interface.py:212-224.  Indices int64, descending score, ties towards
+    the lowest index; lens int32, all ``num_selected``."""
+    _need_gpu(score)
+    B, H, nbq, nbk = score.shape
+    k_sel = num_selected(sparsity, nbk)
+    score = score.contiguous()
+    idx = torch.empty(B * H * nbq * max(k_sel, 1), dtype=torch.int32, device=score.device)
+    idx = idx[: B * H * nbq * k_sel].view(B, H, nbq, k_sel)
+    lens = torch.empty(B, H, nbq, dtype=torch.int32, device=score.device)
+    lib = _capi.load()
+    with torch.cuda.device(score.device):
+        _capi.check(lib.bsa_topk_from_score(_ptr(score), _ptr(idx), _ptr(lens), B, H, nbq, nbk, k_sel,
+                                            _code(score), _stream(score)), "topk")
+    return idx.long(), lens
+
+
+def get_select_indices_topk(q: torch.Tensor, k: torch.Tensor, sparsity: float):
+    """bsa_interface.py:206-210."""
+    idx, lens, _ = _score_topk(q, k, num_selected(sparsity, k.shape[2]))
+    return idx.long(), lens
+
+
+def get_select_indices(q, k, sparsity, cdf_threshold):
+    """bsa_interface.py:268-277."""
+    if sparsity is not None and cdf_threshold is None:
+        return get_select_indices_topk(q, k, sparsity)
+    if sparsity is None and cdf_threshold is None:
+        raise ValueError
+    raise NotImplementedError("CDF-threshold selection is not built; pass cdf_threshold=None")
+
+
+# ---------------------------------------------------------------------------
+# R5 / R6: the attention kernel on blocked-order tensors
+# ---------------------------------------------------------------------------
+def attn_fwd_bsa_varlen(q, k, v, sm_scale, block_indices, block_indices_lens, chunk_size_q, chunk_size_k,
+                        sparsity=None, tile_valid: Optional[torch.Tensor] = None):
+    """bsa_interface.py:290-341 (attn_fwd_bsa_varlen_triton).  Returns ``(o, lse)``
+    with ``lse`` the natural-log sum-exp, fp32 [B,H,S]."""
+    _need_gpu(q, k, v, block_indices, block_indices_lens)
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    assert k.shape == v.shape and k.shape[0] == B and k.shape[1] == H and k.shape[3] == D
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    idx = block_indices.to(torch.int32).contiguous()
+    lens = block_indices_lens.to(torch.int32).contiguous()
+    assert idx.shape[:3] == (B, H, Sq // chunk_size_q) and lens.shape == idx.shape[:3]
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device)
+    lib = _capi.load()
+    with torch.cuda.device(q.device):
+        _capi.check(lib.bsa_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(idx), _ptr(lens), _ptr(tile_valid), _ptr(o), _ptr(lse),
+                                B, H, Sq, Sk, D, int(chunk_size_q), int(chunk_size_k), idx.shape[3],
+                                float(sm_scale), _code(q), _stream(q)), "bsa_fwd")
+    return o, lse
+
+
+attn_fwd_bsa_varlen_triton = attn_fwd_bsa_varlen   # the reference's name for the same entry
+
+
+def flash_attn_bsa(q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold, sm_scale,
+                   tile_valid: Optional[torch.Tensor] = None):
+    """bsa_interface.py:535-568, 598 (``_attention_bsa.apply``) on blocked-order
+    tensors: pool, score, top-k, attention.  Returns ``o`` only, like the reference."""
+    _no_grad(q, k, v)
+    D = q.shape[-1]
+    assert D == k.shape[-1] and D == v.shape[-1]
+    assert D in {16, 32, 64, 128, 256}
+    q_cmp = mean_pooling_compression(q, chunk_size_q)
+    k_cmp = mean_pooling_compression(k, chunk_size_k)
+    if sparsity is None and cdf_threshold is None:
+        raise ValueError
+    if cdf_threshold is not None:
+        raise NotImplementedError("CDF-threshold selection is not built; pass cdf_threshold=None")
+    idx, lens, _ = _score_topk(q_cmp, k_cmp, num_selected(sparsity, k_cmp.shape[2]))
+    o, _ = attn_fwd_bsa_varlen(q, k, v, sm_scale, idx, lens, chunk_size_q, chunk_size_k, sparsity, tile_valid)
+    return o
+
+
+# ---------------------------------------------------------------------------
+# R9: the operator
+# ---------------------------------------------------------------------------
+def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k, want_selection=False):
+    _need_gpu(q, k, v)
+    B, H, Sq, D = q.shape
+    Tq, Hq, Wq = (int(x) for x in latent_shape_q)
+    Tk, Hk, Wk = (int(x) for x in latent_shape_k)
+    tq, hq, wq = (int(x) for x in chunk_q)
+    tk, hk, wk = (int(x) for x in chunk_k)
+    lib = _capi.load()
+    q, k, v = _rows_ok(q), _rows_ok(k), _rows_ok(v)
+    nbk = lib.bsa_padded_tokens(Tk, Hk, Wk, tk, hk, wk) // (tk * hk * wk)
+    nbq = lib.bsa_padded_tokens(Tq, Hq, Wq, tq, hq, wq) // (tq * hq * wq)
+    k_sel = num_selected(sparsity, nbk)
+    prm = _capi.Bsa3dParams(B, H, D, _code(q), Tq, Hq, Wq, Tk, Hk, Wk, tq, hq, wq, tk, hk, wk, k_sel,
+                            1.0 / D ** 0.5)
+    need = lib.bsa_workspace_bytes(C.byref(prm))
+    if need == 0:
+        _capi.check(lib.bsa_fwd_3d(C.byref(prm), None, None, None, None, None, None, None, None, None, 0,
+                                   None, None, None, None), "flash_attn_bsa_3d")
+    ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+    o = torch.empty(B, H, Sq, D, dtype=q.dtype, device=q.device)
+    idx = lens = score = None
+    if want_selection:
+        idx = torch.empty(B, H, nbq, k_sel, dtype=torch.int32, device=q.device)
+        lens = torch.empty(B, H, nbq, dtype=torch.int32, device=q.device)
+        score = torch.empty(B, H, nbq, nbk, dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        _capi.check(lib.bsa_fwd_3d(
+            C.byref(prm), _ptr(q), _capi.strides3(q.stride()[:3]), _ptr(k), _capi.strides3(k.stride()[:3]),
+            _ptr(v), _capi.strides3(v.stride()[:3]), _ptr(o), _capi.strides3(o.stride()[:3]),
+            _ptr(ws), need, _ptr(idx), _ptr(lens), _ptr(score), _stream(q)), "flash_attn_bsa_3d")
+    return (o, idx, lens, score) if want_selection else o
+
+
+@torch.library.custom_op("longcat_video_amd::flash_attn_bsa_3d", mutates_args=())
+def _bsa_3d_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, latent_shape_q: Sequence[int],
+               latent_shape_k: Sequence[int], sparsity: float, chunk_3d_shape_q: Sequence[int],
+               chunk_3d_shape_k: Sequence[int]) -> torch.Tensor:
+    return _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_3d_shape_q, chunk_3d_shape_k)
+
+
+@_bsa_3d_op.register_fake
+def _(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_3d_shape_q, chunk_3d_shape_k):
+    return q.new_empty(q.shape)
+
+
+def flash_attn_bsa_3d(
+    q: torch.Tensor,  # [B, H, Sq, D]
+    k: torch.Tensor,  # [B, H, Skv, D]
+    v: torch.Tensor,  # [B, H, Skv, D]
+    latent_shape_q,
+    latent_shape_k,
+    # bsa_params
+    sparsity=0.875,
+    cdf_threshold=None,
+    chunk_3d_shape_q=[4, 4, 8],
+    chunk_3d_shape_k=[4, 4, 8],
+    allow_padding: bool = True,
+) -> torch.Tensor:
+    """Drop-in for bsa_interface.py:612-660.  q [B,H,Sq,D], k/v [B,H,Skv,D] in
+    (T,H,W) token order, any strides with a contiguous D axis; returns a fresh
+    contiguous [B,H,Sq,D] tensor of the same dtype."""
+    _, _, Sq, head_dim_q = q.shape
+    _, _, Sk, head_dim_k = k.shape
+    assert head_dim_q == head_dim_k
+    assert v.shape == k.shape and k.shape[:2] == q.shape[:2] and q.dtype == k.dtype == v.dtype
+    Tq, Hq, Wq = latent_shape_q
+    Tk, Hk, Wk = latent_shape_k
+    assert Tq * Hq * Wq == Sq
+    assert Tk * Hk * Wk == Sk
+    tq, hq, wq = chunk_3d_shape_q
+    tk, hk, wk = chunk_3d_shape_k
+    if not allow_padding:
+        assert Tq % tq == 0 and Hq % hq == 0 and Wq % wq == 0
+        assert Tk % tk == 0 and Hk % hk == 0 and Wk % wk == 0
+    assert head_dim_q in {16, 32, 64, 128, 256}
+    if sparsity is None and cdf_threshold is None:
+        raise ValueError
+    if cdf_threshold is not None:
+        raise NotImplementedError("CDF-threshold selection is not built; pass cdf_threshold=None")
+    _no_grad(q, k, v)
+    return _bsa_3d_op(q, k, v, [int(x) for x in latent_shape_q], [int(x) for x in latent_shape_k],
+                      float(sparsity), [int(x) for x in chunk_3d_shape_q], [int(x) for x in chunk_3d_shape_k])

@@ -1,0 +1,131 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header
+declares, and rejects bad arguments on the host before anything is launched."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from longcat_video_amd import _capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "bsa_mi355x.h")
+FAKE = C.c_void_p(0x10000)          # never dereferenced: validation fails first
+
+
+def declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    return sorted(set(re.findall(r"\b(bsa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _capi.load()
+    names = declared_functions()
+    assert "bsa_fwd_3d" in names and "bsa_permute_thw_to_blocks" in names and len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), "library lacks %s" % n
+        assert n in _capi.SIGNATURES, "binding lacks %s" % n
+    assert sorted(_capi.SIGNATURES) == names
+
+
+def test_version_and_error_string():
+    lib = _capi.load()
+    assert lib.bsa_version() >= 100
+    assert isinstance(_capi.last_error(), str)
+
+
+@pytest.mark.parametrize("sparsity,n", [(0.875, 8), (0.9375, 1440), (0.9, 10), (0.0, 7), (1.0, 7), (0.3, 10), (0.9375, 624)])
+def test_num_selected_matches_python_doubles(sparsity, n):
+    assert _capi.load().bsa_num_selected(sparsity, n) == int((1 - sparsity) * n)
+
+
+def test_padded_tokens():
+    lib = _capi.load()
+    assert lib.bsa_padded_tokens(24, 45, 80, 4, 4, 4) == 92160
+    assert lib.bsa_padded_tokens(24, 30, 52, 4, 4, 4) == 39936
+    assert lib.bsa_padded_tokens(4, 8, 8, 4, 4, 4) == 256
+    assert lib.bsa_padded_tokens(0, 8, 8, 4, 4, 4) == -1
+
+
+def test_permute_rejects_bad_arguments():
+    lib = _capi.load()
+    st = _capi.strides3([256 * 128, 256 * 128, 128])
+    ok_tail = (1, 1, 4, 8, 8, 4, 4, 4, 128, _capi.BSA_BF16, None)
+    assert lib.bsa_permute_thw_to_blocks(None, st, FAKE, None, None, *ok_tail) == _capi.BSA_ERR_BAD_ARG
+    assert "null" in _capi.last_error()
+    assert lib.bsa_permute_thw_to_blocks(FAKE, None, FAKE, None, None, *ok_tail) == _capi.BSA_ERR_BAD_ARG
+    bad_dtype = ok_tail[:9] + (7, None)
+    assert lib.bsa_permute_thw_to_blocks(FAKE, st, FAKE, None, None, *bad_dtype) == _capi.BSA_ERR_UNSUPPORTED
+    odd_d = ok_tail[:8] + (100, _capi.BSA_BF16, None)     # 200-byte rows
+    assert lib.bsa_permute_thw_to_blocks(FAKE, st, FAKE, None, None, *odd_d) == _capi.BSA_ERR_UNSUPPORTED
+    zero = (1, 1, 0, 8, 8, 4, 4, 4, 128, _capi.BSA_BF16, None)
+    assert lib.bsa_permute_thw_to_blocks(FAKE, st, FAKE, None, None, *zero) == _capi.BSA_ERR_BAD_ARG
+    misaligned = C.c_void_p(0x10002)
+    assert lib.bsa_permute_thw_to_blocks(misaligned, st, FAKE, None, None, *ok_tail) == _capi.BSA_ERR_BAD_ARG
+    bad_stride = _capi.strides3([256 * 128, 256 * 128, 100])
+    assert lib.bsa_permute_thw_to_blocks(FAKE, bad_stride, FAKE, None, None, *ok_tail) == _capi.BSA_ERR_BAD_ARG
+    small_chunk = (1, 1, 4, 8, 8, 2, 2, 2, 128, _capi.BSA_BF16, None)   # 8-token chunk: no 64-slot tiles
+    assert lib.bsa_permute_thw_to_blocks(FAKE, st, FAKE, None, FAKE, *small_chunk) == _capi.BSA_ERR_UNSUPPORTED
+
+
+def test_topk_rejects_bad_arguments():
+    lib = _capi.load()
+    assert lib.bsa_topk_from_score(FAKE, FAKE, FAKE, 1, 1, 4, 4, 5, _capi.BSA_BF16, None) == _capi.BSA_ERR_SHAPE
+    assert lib.bsa_topk_from_score(FAKE, FAKE, FAKE, 1, 1, 4, 5000, 5, _capi.BSA_BF16, None) == _capi.BSA_ERR_UNSUPPORTED
+    assert lib.bsa_topk_from_score(FAKE, FAKE, FAKE, 1, 1, 4, 4096, 2000, _capi.BSA_BF16, None) == _capi.BSA_ERR_UNSUPPORTED
+    assert lib.bsa_topk_from_score(None, FAKE, FAKE, 1, 1, 4, 4, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_BAD_ARG
+    assert lib.bsa_score_topk(FAKE, FAKE, FAKE, FAKE, FAKE, 1, 1, 4, 4, 100, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_UNSUPPORTED
+    assert lib.bsa_score_topk(FAKE, FAKE, FAKE, FAKE, None, 1, 1, 4, 4, 128, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_BAD_ARG
+
+
+def test_fwd_rejects_bad_arguments():
+    lib = _capi.load()
+    ptrs = [FAKE] * 5 + [None, FAKE, None]
+
+    def call(B=1, Hn=1, Sq=256, Sk=256, D=128, bs_q=64, bs_k=64, stride=2, scale=0.088, dtype=_capi.BSA_BF16, p=ptrs):
+        return lib.bsa_fwd(*p, B, Hn, Sq, Sk, D, bs_q, bs_k, stride, scale, dtype, None)
+
+    assert call(D=64) == _capi.BSA_ERR_UNSUPPORTED and "128" in _capi.last_error()
+    assert call(bs_q=48) == _capi.BSA_ERR_UNSUPPORTED
+    assert call(Sq=200) == _capi.BSA_ERR_SHAPE
+    assert call(Sk=100) == _capi.BSA_ERR_SHAPE
+    assert call(scale=0.0) == _capi.BSA_ERR_BAD_ARG
+    assert call(scale=float("nan")) == _capi.BSA_ERR_BAD_ARG
+    assert call(dtype=9) == _capi.BSA_ERR_UNSUPPORTED
+    assert call(B=0) == _capi.BSA_ERR_BAD_ARG
+    assert call(p=[None] + ptrs[1:]) == _capi.BSA_ERR_BAD_ARG
+
+
+def test_fwd_3d_plan_and_workspace():
+    lib = _capi.load()
+    prm = _capi.Bsa3dParams(1, 32, 128, _capi.BSA_BF16, 24, 45, 80, 24, 45, 80, 4, 4, 4, 4, 4, 4, 90, 0.0883883)
+    need = lib.bsa_workspace_bytes(C.byref(prm))
+    body = 4 * 32 * 92160 * 128 * 2                  # q, k, v, o in blocked order
+    assert need > body and need < body + 300 * 2 ** 20
+    st = _capi.strides3([32 * 86400 * 128, 86400 * 128, 128])
+    args = (FAKE, st, FAKE, st, FAKE, st, FAKE, st)
+    ws = C.c_void_p(0x100000)
+    assert lib.bsa_fwd_3d(C.byref(prm), *args, ws, need - 1, None, None, None, None) == _capi.BSA_ERR_WORKSPACE
+    assert lib.bsa_fwd_3d(C.byref(prm), *args, C.c_void_p(0x100010), need, None, None, None, None) == _capi.BSA_ERR_BAD_ARG
+    prm.k_sel = 2000
+    assert lib.bsa_workspace_bytes(C.byref(prm)) == 0
+    assert lib.bsa_fwd_3d(C.byref(prm), *args, ws, need, None, None, None, None) == _capi.BSA_ERR_SHAPE
+    prm.k_sel, prm.D = 90, 64
+    assert lib.bsa_fwd_3d(C.byref(prm), *args, ws, need, None, None, None, None) == _capi.BSA_ERR_UNSUPPORTED
+    prm.D, prm.tq = 128, 2                          # 32-token query chunks
+    assert lib.bsa_fwd_3d(C.byref(prm), *args, ws, need, None, None, None, None) == _capi.BSA_ERR_UNSUPPORTED
+    assert lib.bsa_fwd_3d(None, *args, ws, need, None, None, None, None) == _capi.BSA_ERR_BAD_ARG
+
+
+def test_status_to_exception_mapping():
+    lib = _capi.load()
+    rc = lib.bsa_topk_from_score(FAKE, FAKE, FAKE, 1, 1, 4, 4, 5, _capi.BSA_BF16, None)
+    with pytest.raises(AssertionError):
+        _capi.check(rc)
+    rc = lib.bsa_topk_from_score(None, FAKE, FAKE, 1, 1, 4, 4, 2, _capi.BSA_BF16, None)
+    with pytest.raises(ValueError):
+        _capi.check(rc)
+    rc = lib.bsa_topk_from_score(FAKE, FAKE, FAKE, 1, 1, 4, 5000, 5, _capi.BSA_BF16, None)
+    with pytest.raises(NotImplementedError):
+        _capi.check(rc)
+    _capi.check(0)

@@ -1,0 +1,57 @@
+"""Pins the oracle's glue functions (R11): RMSNorm and 3-D RoPE."""
+import math
+
+import torch
+
+from oracle import bsa_oracle as O
+
+
+def test_rms_norm_unit_rms_and_weight():
+    x = torch.randn(2, 3, 5, 128, generator=torch.Generator().manual_seed(0)) * 7
+    y = O.rms_norm_fp32(x, torch.ones(128))
+    assert torch.allclose(y.pow(2).mean(-1), torch.ones(2, 3, 5), atol=1e-4)
+    w = torch.linspace(0.5, 2, 128)
+    assert torch.allclose(O.rms_norm_fp32(x, w), y * w)
+    yb = O.rms_norm_fp32(x.bfloat16(), torch.ones(128, dtype=torch.bfloat16))
+    assert yb.dtype == torch.bfloat16
+
+
+def test_rope_axis_split_and_frequencies():
+    ang = O.rope_3d_angles((3, 4, 5), 128)
+    assert ang.shape == (60, 128)
+    # dims: t = 128 - 4*21 = 44, h = w = 42
+    tok = lambda t, h, w: (t * 4 + h) * 5 + w
+    a = ang[tok(2, 3, 4)]
+    for i in range(22):
+        assert math.isclose(a[2 * i].item(), 2 * 10000 ** (-2 * i / 44), rel_tol=1e-5)
+        assert a[2 * i].item() == a[2 * i + 1].item()
+    for i in range(21):
+        assert math.isclose(a[44 + 2 * i].item(), 3 * 10000 ** (-2 * i / 42), rel_tol=1e-5)
+        assert math.isclose(a[86 + 2 * i].item(), 4 * 10000 ** (-2 * i / 42), rel_tol=1e-5)
+    assert torch.all(ang[0] == 0)
+
+
+def test_rope_preserves_norm_and_relative_position():
+    grid = (2, 3, 6)
+    ang = O.rope_3d_angles(grid, 128)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(1, 1, 36, 128, generator=g)
+    y = O.rope_3d_apply(x, ang)
+    assert torch.allclose(y.norm(dim=-1), x.norm(dim=-1), rtol=1e-5)
+    assert torch.equal(y[0, 0, 0], x[0, 0, 0])           # position (0,0,0) is the identity
+    # same content at every token: q.k depends only on the offset between positions
+    qv, kv = torch.randn(128, generator=g), torch.randn(128, generator=g)
+    q = O.rope_3d_apply(qv.expand(1, 1, 36, 128), ang)[0, 0]
+    k = O.rope_3d_apply(kv.expand(1, 1, 36, 128), ang)[0, 0]
+    tok = lambda t, h, w: (t * 3 + h) * 6 + w
+    d1 = q[tok(0, 1, 2)] @ k[tok(1, 2, 5)]
+    d2 = q[tok(0, 0, 0)] @ k[tok(1, 1, 3)]
+    assert math.isclose(d1.item(), d2.item(), rel_tol=1e-4, abs_tol=1e-4)
+
+
+def test_rope_pairs_are_interleaved():
+    ang = torch.zeros(1, 4)
+    ang[0, :2] = math.pi / 2
+    x = torch.tensor([1.0, 2.0, 3.0, 4.0]).view(1, 1, 1, 4)
+    y = O.rope_3d_apply(x, ang)
+    assert torch.allclose(y.flatten(), torch.tensor([-2.0, 1.0, 3.0, 4.0]), atol=1e-6)
