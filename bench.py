@@ -1,0 +1,199 @@
+"""Benchmark of the block-sparse attention forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4]
+
+A step is one pass of the whole operator (3-D chunk permute of q/k/v with fused
+pooling, pooled scores, top-k, block-sparse flash attention, unpermute) over one
+synthetic attention layer that is already resident in HBM.  Rank 0 prints ONE
+JSON line.  `value` is the sparse-actual TFLOP/s of the whole operator (only the
+FLOPs of the selected block pairs are counted; everything else in the step is
+overhead that lowers it).  `roofline` covers the dominant kernel, timed on its
+own with HIP events on the launch stream; `cpu_baseline` times the CPU oracle's
+masked-dense evaluation on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "longcat-video_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+
+WORKLOADS = {
+    # name: (latent grid, sparsity, seed, rms-normalised q/k, description)
+    "c2": ((24, 30, 52), 0.9375, 1, False, "480p layer: 32 heads x 128, grid 24x30x52 (37440 tokens), density 1/16"),
+    "c3": ((24, 45, 80), 0.9375, 2, True, "720p layer: 32 heads x 128, grid 24x45x80 (86400 tokens), density 1/16"),
+}
+CHUNK = (4, 4, 4)
+HEADS, D = 32, 128
+
+
+def make_inputs(torch, latent, seed, rms):
+    S = latent[0] * latent[1] * latent[2]
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    out = []
+    for i in range(3):
+        x = torch.randn(1, HEADS, S, D, generator=g, device="cuda")
+        if rms and i < 2:
+            x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6)
+        out.append(x.bfloat16())
+        del x
+    return out
+
+
+def time_events(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps      # ms per call
+
+
+def cpu_baseline(torch, latent, sparsity, seed, rms, budget_s):
+    """The oracle's masked-dense evaluation of the same layer on the host cores:
+    pool -> score -> top-k -> block mask -> fp32 softmax(QK^T/sqrt(D) + mask)V.
+    One head is prepared in full; query blocks are evaluated until the time
+    budget is spent, then scaled linearly to all heads and query blocks."""
+    from oracle import bsa_oracle as O
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    S = latent[0] * latent[1] * latent[2]
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = (torch.randn(1, 1, S, D, generator=g) for _ in range(3))
+    if rms:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + 1e-6)
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + 1e-6)
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    t0 = time.perf_counter()
+    qp = O.rearrange_thw_to_3d_block(q, latent, CHUNK)
+    kp = O.rearrange_thw_to_3d_block(k, latent, CHUNK)
+    vp = O.rearrange_thw_to_3d_block(v, latent, CHUNK)
+    score = O.cal_score(O.mean_pooling_compression(qp, 64), O.mean_pooling_compression(kp, 64))
+    nbq, nbk = score.shape[-2:]
+    k_sel = O.num_selected(sparsity, nbk)
+    idx, lens = O.select_topk(score, k_sel)
+    mask = O.block_mask_from_indices(idx, lens, nbk)
+    kvalid = torch.from_numpy(O.slot_validity(latent, CHUNK))
+    t_head_setup = time.perf_counter() - t0
+    done, t_attn = 0, 0.0
+    O.masked_dense_attention(qp, kp, vp, mask, 64, 64, 1 / math.sqrt(D), key_valid=kvalid, q_blocks=[0])   # warm-up
+    while done < nbq and t_attn < budget_s:
+        blocks = list(range(done, min(done + 8, nbq)))
+        t0 = time.perf_counter()
+        O.masked_dense_attention(qp, kp, vp, mask, 64, 64, 1 / math.sqrt(D), key_valid=kvalid, q_blocks=blocks)
+        t_attn += time.perf_counter() - t0
+        done += len(blocks)
+    layer_s = HEADS * (t_head_setup + t_attn * nbq / done)
+    flop = HEADS * nbq * k_sel * 4 * 64 * 64 * D
+    return {
+        "value": flop / layer_s / 1e12, "unit": "TFLOP/s (sparse-actual)", "cores": cores, "kind": "port",
+        "ms_per_layer": layer_s * 1e3,
+        "sample": "1 of %d heads: permute+pool+score+top-k in full (%.2f s), masked-dense fp32 attention on %d of %d "
+                  "query blocks against all keys (%.2f s); scaled linearly to %d heads x %d query blocks"
+                  % (HEADS, t_head_setup, done, nbq, t_attn, HEADS, nbq),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the CPU baseline's attention sample")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the operator shards over heads; "
+                 "run one process per GPU on its own heads). Use --gpus 1.")
+
+    import torch
+    from longcat_video_amd.block_sparse_attention import bsa_interface as I
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (there is no CPU path to measure)")
+    torch.cuda.set_device(0)
+    latent, sparsity, seed, rms, desc = WORKLOADS[args.workload]
+    q, k, v = make_inputs(torch, latent, seed, rms)
+    prm = dict(sparsity=sparsity, chunk_3d_shape_q=list(CHUNK), chunk_3d_shape_k=list(CHUNK))
+
+    # ---- whole operator: warm-up, then exactly K timed steps between synchronisations ----
+    for _ in range(args.warmup):
+        I.flash_attn_bsa_3d(q, k, v, latent, latent, **prm)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        o = I.flash_attn_bsa_3d(q, k, v, latent, latent, **prm)
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # ---- per-kernel timing with events on the launch stream ----
+    qp, q_cmp, _ = I._permute(q, latent, CHUNK, want_pooled=True)
+    kp, k_cmp, valid = I._permute(k, latent, CHUNK, want_pooled=True, want_valid=True)
+    vp, _, _ = I._permute(v, latent, CHUNK)
+    nbq, nbk = q_cmp.shape[2], k_cmp.shape[2]
+    k_sel = I.num_selected(sparsity, nbk)
+    idx, lens, _ = I._score_topk(q_cmp, k_cmp, k_sel)
+    padded = any(n % c for n, c in zip(latent, CHUNK))
+    tv = valid if padded else None
+    scale = 1 / math.sqrt(D)
+    ksteps, kwarm = max(args.steps, 5), max(min(args.warmup, 3), 1)
+    ms_attn = time_events(torch, lambda: I.attn_fwd_bsa_varlen(qp, kp, vp, scale, idx, lens, 64, 64, tile_valid=tv), ksteps, kwarm)
+    ms_permute = time_events(torch, lambda: I._permute(k, latent, CHUNK, want_pooled=True), ksteps, kwarm)
+    ms_unpermute = time_events(torch, lambda: I.rearrange_3d_block_to_THW(qp, *[-(-n // c) for n, c in zip(latent, CHUNK)], *CHUNK, D, latent_shape=latent), ksteps, kwarm)
+    ms_select = time_events(torch, lambda: I._score_topk(q_cmp, k_cmp, k_sel), ksteps, kwarm)
+
+    S = q.shape[2]
+    Sp = qp.shape[2]
+    pairs = HEADS * nbq * k_sel
+    flop = pairs * 4 * 64 * 64 * D
+    dense_flop = 4 * HEADS * S * S * D
+    tflops_step = flop / (ms_step * 1e-3) / 1e12
+    tflops_attn = flop / (ms_attn * 1e-3) / 1e12
+    es = 2
+    permute_bytes = HEADS * (S + Sp) * D * es
+
+    result = {
+        "metric": "BSA fwd ms/layer + sparse TFLOPS (% bf16 MFMA peak) at 720p 86.4k tokens",
+        "value": round(tflops_step, 2),
+        "unit": "TFLOP/s (sparse-actual, whole operator)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic N(0,1) q/k/v%s, seeded on the GPU" % (" with per-head RMS-normalised q/k" if rms else ""),
+        "config": {"workload": "%s: %s" % (args.workload, desc), "chunk": list(CHUNK), "kv_blocks": nbk, "k_sel": k_sel,
+                   "block_pairs": pairs, "padded_tokens": Sp},
+        "ms_per_layer": round(ms_step, 4),
+        "pct_of_bf16_peak_whole_operator": round(100 * tflops_step / PEAK_BF16_TFLOPS, 2),
+        "dense_equivalent_tflops": round(dense_flop / (ms_step * 1e-3) / 1e12, 1),
+        "kernels_ms": {"attention": round(ms_attn, 4), "permute_pool_one_tensor": round(ms_permute, 4),
+                       "unpermute": round(ms_unpermute, 4), "score_topk": round(ms_select, 4)},
+        "permute_gbs": round(permute_bytes / (ms_permute * 1e-3) / 1e9, 1),
+        "roofline": {"kernel": "fwd_mfma_kernel<bf16>", "bound": "mfma", "achieved": round(tflops_attn, 2),
+                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops_attn / PEAK_BF16_TFLOPS, 4),
+                     "traffic": None, "ms": round(ms_attn, 4)},
+    }
+    del o
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(torch, latent, sparsity, seed, rms, args.cpu_seconds)
+        result["cpu_baseline"]["value"] = round(result["cpu_baseline"]["value"], 5)
+        result["cpu_baseline"]["ms_per_layer"] = round(result["cpu_baseline"]["ms_per_layer"], 1)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -140,12 +140,12 @@ def _score_topk(q_cmp, k_cmp, k_sel):
     assert k_cmp.shape[0] == B and k_cmp.shape[1] == H and k_cmp.shape[3] == D
     q_cmp, k_cmp = q_cmp.contiguous(), k_cmp.contiguous()
     score = torch.empty(B, H, nbq, nbk, dtype=q_cmp.dtype, device=q_cmp.device)
-    idx = torch.empty(B * H * nbq * max(k_sel, 1), dtype=torch.int32, device=q_cmp.device)
-    idx = idx[: B * H * nbq * k_sel].view(B, H, nbq, k_sel)     # never a null pointer, even for k_sel == 0
+    buf = torch.empty(B * H * nbq * max(k_sel, 1), dtype=torch.int32, device=q_cmp.device)   # non-null even for k_sel == 0
+    idx = buf[: B * H * nbq * k_sel].view(B, H, nbq, k_sel)
     lens = torch.empty(B, H, nbq, dtype=torch.int32, device=q_cmp.device)
     lib = _capi.load()
     with torch.cuda.device(q_cmp.device):
-        _capi.check(lib.bsa_score_topk(_ptr(q_cmp), _ptr(k_cmp), _ptr(idx), _ptr(lens), _ptr(score),
+        _capi.check(lib.bsa_score_topk(_ptr(q_cmp), _ptr(k_cmp), _ptr(buf), _ptr(lens), _ptr(score),
                                        B, H, nbq, nbk, D, k_sel, _code(q_cmp), _stream(q_cmp)), "score_topk")
     return idx, lens, score
 
@@ -162,12 +162,12 @@ def get_select_indices_topk_from_score(score: torch.Tensor, sparsity: float):
     B, H, nbq, nbk = score.shape
     k_sel = num_selected(sparsity, nbk)
     score = score.contiguous()
-    idx = torch.empty(B * H * nbq * max(k_sel, 1), dtype=torch.int32, device=score.device)
-    idx = idx[: B * H * nbq * k_sel].view(B, H, nbq, k_sel)
+    buf = torch.empty(B * H * nbq * max(k_sel, 1), dtype=torch.int32, device=score.device)
+    idx = buf[: B * H * nbq * k_sel].view(B, H, nbq, k_sel)
     lens = torch.empty(B, H, nbq, dtype=torch.int32, device=score.device)
     lib = _capi.load()
     with torch.cuda.device(score.device):
-        _capi.check(lib.bsa_topk_from_score(_ptr(score), _ptr(idx), _ptr(lens), B, H, nbq, nbk, k_sel,
+        _capi.check(lib.bsa_topk_from_score(_ptr(score), _ptr(buf), _ptr(lens), B, H, nbq, nbk, k_sel,
                                             _code(score), _stream(score)), "topk")
     return idx.long(), lens
 

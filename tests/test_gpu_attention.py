@@ -1,0 +1,161 @@
+"""R5/R6 on the GPU: the block-sparse flash-attention kernel against the oracle.
+
+Tolerances (bf16 / fp16 outputs vs the fp32 masked-dense oracle): max-abs 2e-2,
+mean-abs 2e-3; fp32 kernel: 2e-5.  lse: 2e-3 absolute."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import bsa_oracle as O
+from conftest import seeded_qkv
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS = 2e-2, 2e-3
+
+
+def I():
+    from longcat_video_amd.block_sparse_attention import bsa_interface
+    return bsa_interface
+
+
+def run(q, k, v, idx, lens, bs_q=64, bs_k=64, scale=None, valid_bits=None):
+    scale = 1 / math.sqrt(q.shape[-1]) if scale is None else scale
+    tv = None if valid_bits is None else torch.from_numpy(valid_bits.view(np.int64)).cuda()
+    o, lse = I().attn_fwd_bsa_varlen(q.cuda(), k.cuda(), v.cuda(), scale, idx.cuda(), lens.cuda(), bs_q, bs_k,
+                                     tile_valid=tv)
+    torch.cuda.synchronize()
+    return o.cpu(), lse.cpu()
+
+
+def close(o, want, dtype):
+    d = (o.float() - want).abs()
+    if dtype == torch.float32:
+        assert d.max() <= 2e-5, d.max()
+    else:
+        assert d.max() <= MAX_ABS and d.mean() <= MEAN_ABS, (d.max(), d.mean())
+
+
+def random_lists(seed, B, H, nbq, nbk, k_sel):
+    g = torch.Generator().manual_seed(seed)
+    idx = torch.stack([torch.randperm(nbk, generator=g)[:k_sel] for _ in range(B * H * nbq)]).view(B, H, nbq, k_sel)
+    return idx, torch.full((B, H, nbq), k_sel, dtype=torch.int32)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_small_random_lists(dtype):
+    q, k, v = seeded_qkv(20, 1, 3, 192, 448, 128, dtype)
+    idx, lens = random_lists(20, 1, 3, 3, 7, 4)
+    o, lse = run(q, k, v, idx, lens)
+    assert o.dtype == dtype
+    want, want_lse = O.masked_dense_attention(q, k, v, O.block_mask_from_indices(idx, lens, 7), 64, 64, 1 / math.sqrt(128))
+    close(o, want, dtype)
+    assert torch.allclose(lse, want_lse, atol=2e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_matches_the_step_by_step_kernel_restatement(dtype):
+    q, k, v = seeded_qkv(21, 2, 2, 128, 256, 128, dtype)
+    idx, lens = random_lists(21, 2, 2, 2, 4, 3)
+    o, lse = run(q, k, v, idx, lens)
+    want, want_lse = O.blockwise_attention(q, k, v, idx, lens, 64, 64, 1 / math.sqrt(128))
+    d = (o.float() - want.float()).abs()
+    assert d.max() <= (2e-5 if dtype == torch.float32 else 1.6e-2)     # at most a couple of bf16 ulps at |o| <= 2
+    assert torch.allclose(lse, want_lse, atol=2e-3)
+
+
+def test_dense_special_case_equals_sdpa():
+    q, k, v = seeded_qkv(22, 1, 2, 256, 256, 128, torch.bfloat16)
+    idx = torch.arange(4).view(1, 1, 1, 4).expand(1, 2, 4, 4).contiguous()
+    lens = torch.full((1, 2, 4), 4, dtype=torch.int32)
+    o, _ = run(q, k, v, idx, lens)
+    want = F.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    close(o, want, torch.bfloat16)
+
+
+def test_variable_lengths_and_empty_rows():
+    q, k, v = seeded_qkv(23, 1, 2, 256, 384, 128, torch.bfloat16)
+    idx, _ = random_lists(23, 1, 2, 4, 6, 5)
+    lens = torch.tensor([[[5, 0, 1, 3], [2, 4, 0, 5]]], dtype=torch.int32)
+    o, lse = run(q, k, v, idx, lens)
+    want, want_lse = O.masked_dense_attention(q, k, v, O.block_mask_from_indices(idx, lens, 6), 64, 64, 1 / math.sqrt(128))
+    close(o, want, torch.bfloat16)
+    empty = (lens == 0).repeat_interleave(64, dim=-1)
+    assert torch.all(o[empty] == 0) and torch.all(torch.isinf(lse[empty]) & (lse[empty] < 0))
+    assert torch.allclose(lse[~empty], want_lse[~empty], atol=2e-3)
+
+
+@pytest.mark.parametrize("pattern", ["tail", "first16", "second_half", "sparse"])
+def test_padded_keys_are_masked(pattern):
+    q, k, v = seeded_qkv(24, 1, 1, 128, 256, 128, torch.bfloat16)
+    valid = torch.ones(256, dtype=torch.bool)
+    if pattern == "tail":
+        valid[200:] = False
+    elif pattern == "first16":                # a T-padded chunk: only slots 0..15 of each tile are real
+        valid.view(4, 64)[:, 16:] = False
+    elif pattern == "second_half":
+        valid.view(4, 64)[1:3, :32] = False
+    else:
+        valid[torch.randperm(256, generator=torch.Generator().manual_seed(1))[:150]] = False
+        valid[::64] = True                    # every block keeps a real key
+    bits = np.packbits(valid.numpy().reshape(-1, 64), axis=1, bitorder="little").view(np.uint64).reshape(-1)
+    idx, lens = random_lists(24, 1, 1, 2, 4, 3)
+    o, lse = run(q, k, v, idx, lens, valid_bits=bits)
+    want, want_lse = O.masked_dense_attention(q, k, v, O.block_mask_from_indices(idx, lens, 4), 64, 64,
+                                              1 / math.sqrt(128), key_valid=valid)
+    close(o, want, torch.bfloat16)
+    assert torch.allclose(lse, want_lse, atol=2e-3)
+
+
+def test_128_token_chunks():
+    """The reference's default 4x4x8 chunk: 128-token query and key blocks."""
+    q, k, v = seeded_qkv(25, 1, 2, 256, 640, 128, torch.bfloat16)
+    idx, lens = random_lists(25, 1, 2, 2, 5, 2)
+    o, lse = run(q, k, v, idx, lens, bs_q=128, bs_k=128)
+    want, want_lse = O.masked_dense_attention(q, k, v, O.block_mask_from_indices(idx, lens, 5), 128, 128, 1 / math.sqrt(128))
+    close(o, want, torch.bfloat16)
+    assert torch.allclose(lse, want_lse, atol=2e-3)
+
+
+def test_lse_merge_identity_and_determinism():
+    q, k, v = seeded_qkv(26, 1, 1, 64, 512, 128, torch.bfloat16)
+    full = torch.tensor([5, 1, 7, 2, 0, 6]).view(1, 1, 1, 6)
+    n = lambda c: torch.full((1, 1, 1), c, dtype=torch.int32)
+    o, lse = run(q, k, v, full, n(6))
+    oa, la = run(q, k, v, full[..., :3].contiguous(), n(3))
+    ob, lb = run(q, k, v, full[..., 3:].contiguous(), n(3))
+    om, lm = O.merge_partial_attention(oa, la, ob, lb)
+    assert (om - o.float()).abs().max() <= 1.6e-2 and torch.allclose(lm, lse, atol=2e-3)
+    o2, lse2 = run(q, k, v, full, n(6))
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)
+    o_rev, _ = run(q, k, v, full.flip(-1).contiguous(), n(6))
+    assert (o_rev.float() - o.float()).abs().max() <= 1.6e-2
+
+
+def test_large_logits_do_not_overflow():
+    q, k, v = seeded_qkv(27, 1, 1, 64, 128, 128, torch.bfloat16)
+    q = (q.float() * 30).bfloat16()
+    idx, lens = random_lists(27, 1, 1, 1, 2, 2)
+    o, lse = run(q, k, v, idx, lens)
+    want, want_lse = O.masked_dense_attention(q, k, v, O.block_mask_from_indices(idx, lens, 2), 64, 64, 1 / math.sqrt(128))
+    assert torch.isfinite(o.float()).all()
+    close(o, want, torch.bfloat16)
+    assert torch.allclose(lse, want_lse, rtol=1e-4, atol=2e-3)
+
+
+def test_480p_two_heads_sampled_rows():
+    """BASELINE config 2 geometry with 2 heads: 624 blocks, 39 selected per row,
+    checked on sampled query blocks against the gathered fp32 oracle."""
+    nb, ks = 624, 39
+    q, k, v = seeded_qkv(1, 1, 2, nb * 64, nb * 64, 128, torch.bfloat16)
+    idx, lens = random_lists(28, 1, 2, nb, nb, ks)
+    o, lse = run(q, k, v, idx, lens)
+    rows = [0, 1, 311, 622, 623]
+    want, want_lse = O.gathered_attention(q, k, v, idx, lens, 64, 64, 1 / math.sqrt(128), q_blocks=rows)
+    for m in rows:
+        sl = slice(m * 64, (m + 1) * 64)
+        close(o[:, :, sl], want[:, :, sl], torch.bfloat16)
+        assert torch.allclose(lse[:, :, sl], want_lse[:, :, sl], atol=2e-3)

@@ -1,0 +1,141 @@
+"""R8/R9 on the GPU: the whole operator through flash_attn_bsa_3d, from the
+BASELINE configs at reduced head count up to the full 720p shape."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import bsa_oracle as O
+from conftest import seeded_qkv
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS = 2e-2, 2e-3
+CH = dict(chunk_3d_shape_q=[4, 4, 4], chunk_3d_shape_k=[4, 4, 4])
+
+
+def I():
+    from longcat_video_amd.block_sparse_attention import bsa_interface
+    return bsa_interface
+
+
+def check_against_oracle(q, k, v, latent_q, latent_k, sparsity, o, idx, lens, score, q_blocks, heads=None,
+                         chunk=(4, 4, 4)):
+    """Selection: bit-exact given the GPU's scores.  Pooled scores: one ulp from the
+    oracle's.  Output: tolerance against the fp32 oracle evaluated with the
+    GPU's selection, on the sampled query blocks."""
+    bs = int(np.prod(chunk))
+    heads = list(range(q.shape[1])) if heads is None else heads
+    qh, kh, vh = q[:, heads], k[:, heads], v[:, heads]
+    qp = O.rearrange_thw_to_3d_block(qh, latent_q, chunk)
+    kp = O.rearrange_thw_to_3d_block(kh, latent_k, chunk)
+    vp = O.rearrange_thw_to_3d_block(vh, latent_k, chunk)
+    want_score = O.cal_score(O.mean_pooling_compression(qp, bs), O.mean_pooling_compression(kp, bs))
+    s_gpu = score[:, heads].cpu()
+    tol = 2.0 ** -6 if q.dtype != torch.float32 else 1e-5     # pooled means and the score are each one rounding
+    assert torch.all((s_gpu.float() - want_score.float()).abs() <= want_score.float().abs() * tol + 1e-3)
+    k_sel = O.num_selected(sparsity, s_gpu.shape[-1])
+    want_idx, _ = O.select_topk(s_gpu, k_sel)
+    assert torch.equal(idx[:, heads].cpu().long(), want_idx), "selection differs from the oracle on identical scores"
+    assert torch.all(lens.cpu() == k_sel)
+    kvalid = torch.from_numpy(O.slot_validity(latent_k, chunk))
+    want_o, _ = O.gathered_attention(qp, kp, vp, want_idx, lens[:, heads].cpu(), bs, bs, 1 / math.sqrt(q.shape[-1]),
+                                     key_valid=kvalid, q_blocks=q_blocks)
+    got_p = O.rearrange_thw_to_3d_block(o[:, heads].cpu(), latent_q, chunk)
+    qvalid = torch.from_numpy(O.slot_validity(latent_q, chunk))
+    for m in q_blocks:
+        rows = torch.arange(m * bs, (m + 1) * bs)[qvalid[m * bs:(m + 1) * bs]]
+        d = (got_p[:, :, rows].float() - want_o[:, :, rows]).abs()
+        if q.dtype == torch.float32:
+            assert d.max() <= 2e-5
+        else:
+            assert d.max() <= MAX_ABS and d.mean() <= MEAN_ABS, (m, d.max(), d.mean())
+
+
+def test_config1_fp32_plumbing():
+    q, k, v = seeded_qkv(0, 1, 4, 256, 256, 128, torch.float32)
+    o, idx, lens, score = I()._bsa_3d(q.cuda(), k.cuda(), v.cuda(), (4, 8, 8), (4, 8, 8), 0.5, (4, 4, 4), (4, 4, 4), True)
+    want, want_idx, _, want_score = O.flash_attn_bsa_3d(q, k, v, (4, 8, 8), (4, 8, 8), 0.5, (4, 4, 4), (4, 4, 4))
+    assert torch.allclose(score.cpu(), want_score, atol=1e-5)
+    assert torch.equal(idx.cpu().long(), want_idx)
+    assert (o.cpu() - want).abs().max() <= 2e-5
+    pub = I().flash_attn_bsa_3d(q.cuda(), k.cuda(), v.cuda(), (4, 8, 8), (4, 8, 8), sparsity=0.5, **CH)
+    assert torch.equal(pub, o) and pub.is_contiguous()
+
+
+def test_config1_in_bf16():
+    q, k, v = seeded_qkv(0, 1, 4, 256, 256, 128, torch.bfloat16)
+    o, idx, lens, score = I()._bsa_3d(q.cuda(), k.cuda(), v.cuda(), (4, 8, 8), (4, 8, 8), 0.5, (4, 4, 4), (4, 4, 4), True)
+    check_against_oracle(q, k, v, (4, 8, 8), (4, 8, 8), 0.5, o, idx, lens, score, q_blocks=range(4))
+
+
+@pytest.mark.parametrize("latent,sparsity", [((4, 6, 5), 0.5), ((5, 9, 13), 0.75), ((8, 30, 52), 0.9375)])
+def test_padded_grids(latent, sparsity):
+    S = int(np.prod(latent))
+    q, k, v = seeded_qkv(31, 1, 2, S, S, 128, torch.bfloat16)
+    o, idx, lens, score = I()._bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, sparsity, (4, 4, 4), (4, 4, 4), True)
+    nb = int(np.prod(O.block_grid(latent, (4, 4, 4))))
+    check_against_oracle(q, k, v, latent, latent, sparsity, o, idx, lens, score, q_blocks=sorted({0, 1, nb // 2, nb - 1}))
+    assert torch.isfinite(o.float()).all()
+
+
+def test_default_chunk_4x4x8():
+    latent = (8, 8, 16)
+    q, k, v = seeded_qkv(32, 1, 2, 1024, 1024, 128, torch.bfloat16)
+    o, idx, lens, score = I()._bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, 0.5, (4, 4, 8), (4, 4, 8), True)
+    check_against_oracle(q, k, v, latent, latent, 0.5, o, idx, lens, score, q_blocks=range(8), chunk=(4, 4, 8))
+    pub = I().flash_attn_bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, sparsity=0.5)   # reference defaults
+    assert torch.equal(pub, o)
+
+
+def test_rectangular_query_and_key_grids():
+    """Tq != Tk, as in the noise half of the cond/noise split (attention.py:132-133)."""
+    lq, lk = (4, 8, 8), (8, 8, 8)
+    q, _, _ = seeded_qkv(33, 1, 2, 256, 256, 128, torch.bfloat16)
+    _, k, v = seeded_qkv(34, 1, 2, 512, 512, 128, torch.bfloat16)
+    o, idx, lens, score = I()._bsa_3d(q.cuda(), k.cuda(), v.cuda(), lq, lk, 0.5, (4, 4, 4), (4, 4, 4), True)
+    assert idx.shape == (1, 2, 4, 4) and score.shape == (1, 2, 4, 8)
+    check_against_oracle(q, k, v, lq, lk, 0.5, o, idx, lens, score, q_blocks=range(4))
+
+
+def test_strided_inputs_from_a_qkv_projection():
+    latent = (4, 8, 8)
+    qkv = torch.randn(1, 256, 3, 2, 128, generator=torch.Generator().manual_seed(35)).bfloat16()
+    q, k, v = qkv.permute(2, 0, 3, 1, 4).unbind(0)
+    dq, dk, dv = qkv.cuda().permute(2, 0, 3, 1, 4).unbind(0)
+    o = I().flash_attn_bsa_3d(dq, dk, dv, latent, latent, sparsity=0.5, **CH)
+    o2 = I().flash_attn_bsa_3d(dq.contiguous(), dk.contiguous(), dv.contiguous(), latent, latent, sparsity=0.5, **CH)
+    assert torch.equal(o, o2)
+    assert torch.equal(dq.cpu(), q)      # inputs are not modified
+
+
+def test_480p_two_heads():
+    latent = (24, 30, 52)
+    q, k, v = seeded_qkv(1, 1, 2, 37440, 37440, 128, torch.bfloat16)
+    o, idx, lens, score = I()._bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, 0.9375, (4, 4, 4), (4, 4, 4), True)
+    assert idx.shape == (1, 2, 624, 39)
+    check_against_oracle(q, k, v, latent, latent, 0.9375, o, idx, lens, score, q_blocks=[0, 12, 300, 611, 623])
+
+
+def test_720p_full_shape_sampled():
+    """BASELINE config 3 at full size (32 heads, 86 400 tokens, RMS-normalised q/k,
+    density 1/16): two heads are checked against the oracle on sampled query
+    blocks; all heads for finiteness, determinism and row-stochastic bounds."""
+    latent = (24, 45, 80)
+    g = torch.Generator(device="cuda").manual_seed(2)
+    q = torch.randn(1, 32, 86400, 128, generator=g, device="cuda")
+    k = torch.randn(1, 32, 86400, 128, generator=g, device="cuda")
+    v = torch.randn(1, 32, 86400, 128, generator=g, device="cuda").bfloat16()
+    q = (q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
+    k = (k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
+    o, idx, lens, score = I()._bsa_3d(q, k, v, latent, latent, 0.9375, (4, 4, 4), (4, 4, 4), True)
+    assert idx.shape == (1, 32, 1440, 90) and torch.all(lens == 90)
+    assert torch.isfinite(o.float()).all()
+    # a convex combination of value rows cannot leave their range
+    assert float(o.float().abs().max()) <= float(v.float().abs().max())
+    heads = [5, 31]
+    check_against_oracle(q.cpu(), k.cpu(), v.cpu(), latent, latent, 0.9375, o, idx, lens, score,
+                         q_blocks=[0, 19, 700, 1439], heads=heads)
+    o2 = I().flash_attn_bsa_3d(q, k, v, latent, latent, sparsity=0.9375, **CH)
+    assert torch.equal(o, o2)

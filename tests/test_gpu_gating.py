@@ -1,0 +1,112 @@
+"""R2-R4 on the GPU: pooled scores and top-k selection.  Selection is bit-exact
+against the oracle's (-score, index) order given the same scores."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bsa_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def I():
+    from longcat_video_amd.block_sparse_attention import bsa_interface
+    return bsa_interface
+
+
+def topk_gpu(score, k_sel):
+    """Calls the C-ABI top-k directly with an explicit k_sel."""
+    from longcat_video_amd import _capi
+    B, H, nbq, nbk = score.shape
+    s = score.cuda().contiguous()
+    idx = torch.full((B * H * nbq * max(k_sel, 1),), -7, dtype=torch.int32, device="cuda")
+    lens = torch.empty(B, H, nbq, dtype=torch.int32, device="cuda")
+    code = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}[score.dtype]
+    _capi.check(_capi.load().bsa_topk_from_score(s.data_ptr(), idx.data_ptr(), lens.data_ptr(), B, H, nbq, nbk,
+                                                  k_sel, code, torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    return idx[: B * H * nbq * k_sel].view(B, H, nbq, k_sel).cpu().long(), lens.cpu()
+
+
+def test_score_exact_on_integer_inputs():
+    g = torch.Generator().manual_seed(1)
+    q = torch.randint(-3, 4, (1, 2, 70, 128), generator=g).float()
+    k = torch.randint(-3, 4, (1, 2, 131, 128), generator=g).float()
+    for dt in (torch.bfloat16, torch.float16, torch.float32):
+        got = I().cal_score(q.to(dt).cuda(), k.to(dt).cuda()).cpu()
+        assert torch.equal(got, O.cal_score(q.to(dt), k.to(dt)))
+
+
+@pytest.mark.parametrize("dtype,ulp", [(torch.bfloat16, 2.0 ** -7), (torch.float16, 2.0 ** -10), (torch.float32, 2.0 ** -20)])
+def test_score_random_within_one_ulp(dtype, ulp):
+    g = torch.Generator().manual_seed(2)
+    q = torch.randn(2, 3, 97, 128, generator=g).to(dtype)
+    k = torch.randn(2, 3, 160, 128, generator=g).to(dtype)
+    got = I().cal_score(q.cuda(), k.cuda()).cpu().float()
+    want64 = torch.einsum("bhmd,bhnd->bhmn", q.double(), k.double())
+    assert torch.all((got.double() - want64).abs() <= want64.abs() * ulp + 1e-4)
+
+
+@pytest.mark.parametrize("nbq,nbk,k_sel", [(4, 4, 2), (5, 37, 9), (3, 64, 64), (2, 65, 1), (7, 200, 0), (3, 624, 39),
+                                             (2, 1440, 90), (2, 1248, 156), (1, 2047, 300), (1, 4096, 1024)])
+def test_topk_bit_exact_with_ties(nbq, nbk, k_sel):
+    g = torch.Generator().manual_seed(nbk)
+    # few distinct values => many exact ties, resolved towards the lowest index
+    score = (torch.randint(-6, 7, (1, 2, nbq, nbk), generator=g).float() / 4).bfloat16()
+    got, lens = topk_gpu(score, k_sel)
+    want, want_lens = O.select_topk(score, k_sel)
+    assert torch.equal(lens, want_lens)
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_topk_random_scores_all_dtypes(dtype):
+    g = torch.Generator().manual_seed(7)
+    score = torch.randn(2, 2, 9, 333, generator=g).to(dtype)
+    got, _ = topk_gpu(score, 41)
+    want, _ = O.select_topk(score, 41)
+    assert torch.equal(got, want)
+    vals = torch.gather(score.float(), -1, got)
+    assert torch.equal(vals, torch.topk(score.float(), 41).values)
+
+
+def test_topk_special_values():
+    inf = float("inf")
+    row = torch.tensor([0.0, -0.0, 1.0, -inf, inf, -0.0, 0.0, -1.0, inf, 3.0])
+    for dt in (torch.bfloat16, torch.float32):
+        score = row.to(dt).view(1, 1, 1, -1)
+        for k in (1, 3, 6, 10):
+            got, _ = topk_gpu(score, k)
+            want, _ = O.select_topk(score, k)
+            assert got.flatten().tolist() == want.flatten().tolist()
+
+
+def test_score_topk_pipeline_matches_oracle_given_gpu_scores():
+    g = torch.Generator().manual_seed(9)
+    qc = torch.randn(1, 4, 312, 128, generator=g).bfloat16() * 0.2
+    kc = torch.randn(1, 4, 1248, 128, generator=g).bfloat16() * 0.2
+    idx, lens, score = I()._score_topk(qc.cuda(), kc.cuda(), 156)      # rectangular, config-4 noise shape
+    want, _ = O.select_topk(score.cpu(), 156)
+    assert torch.equal(idx.cpu().long(), want) and torch.all(lens.cpu() == 156)
+    idx64, lens2 = I().get_select_indices_topk(qc.cuda(), kc.cuda(), 0.875)
+    assert idx64.dtype == torch.int64 and torch.equal(idx64.cpu(), want)
+
+
+def test_full_size_720p_selection():
+    """32 heads x 1440 x 1440 bf16 scores: every row has k_sel distinct indices, the
+    selected values are exactly torch.topk's values, and sampled heads are
+    bit-exact against the oracle."""
+    g = torch.Generator(device="cuda").manual_seed(11)
+    qc = torch.randn(1, 32, 1440, 128, generator=g, device="cuda").bfloat16() * 0.125
+    kc = torch.randn(1, 32, 1440, 128, generator=g, device="cuda").bfloat16() * 0.125
+    idx, lens, score = I()._score_topk(qc, kc, 90)
+    assert torch.all(lens == 90)
+    srt = torch.sort(idx.long(), dim=-1).values
+    assert torch.all(srt[..., 1:] > srt[..., :-1]) and int(srt.min()) >= 0 and int(srt.max()) < 1440
+    vals = torch.gather(score.float(), -1, idx.long())
+    assert torch.equal(vals, torch.topk(score.float(), 90).values)
+    for h in (0, 13, 31):
+        want, _ = O.select_topk(score[:, h:h + 1].cpu(), 90)
+        assert torch.equal(idx[:, h:h + 1].cpu().long(), want)
+    idx2, _, _ = I()._score_topk(qc, kc, 90)
+    assert torch.equal(idx, idx2)
