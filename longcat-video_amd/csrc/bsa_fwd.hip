@@ -14,14 +14,28 @@
 // and 16 keys: the softmax state (running max, running sum) is one scalar per
 // lane, and P^T in the accumulator registers already has the layout the B
 // operand of the second product needs.  O^T (128 d x 32 queries) += V^T . P^T
-// is 8 more MFMAs whose A operand is read from a transposed copy of the V
-// tile.  The transpose happens while staging: each thread loads 4 key rows x
-// 8 d of V, transposes in registers and writes 8-byte key quads.
+// is 8 more MFMAs whose A operand (d along lanes, keys along the k slots) is
+// read from the row-major V tile with the transposing LDS read
+// ds_read_b64_tr_b16: 16 lanes fetch a 4-key x 16-d patch and each lane
+// receives the 4 keys of one d.
 //
-// LDS: 2 stages x (K tile 16 KB + V^T tile 16 KB) = 64 KB per workgroup, two
-// workgroups per CU.  Both tiles use XOR-swizzled 16-byte chunks so that the
-// ds_read_b128 of 16 consecutive lanes fall on distinct banks.
+// Data movement.  K and V tiles go from global memory straight into LDS
+// (global_load_lds_dwordx4, no staging registers): every wavefront issues
+// 4 + 4 loads of 1 KB per tile.  The LDS side of such a load is linear in the
+// lane index, so the XOR swizzle that keeps the later LDS reads free of bank
+// conflicts is applied on the global side: lane l of a load fetches the
+// 16-byte chunk (l%16) ^ f(row) of its row.  Two stages of (K 16 KB + V 16 KB)
+// per workgroup, two workgroups per CU; the tile for iteration i+1 is in
+// flight while iteration i computes, one barrier per iteration.
+//
+// Softmax.  The running maximum is only raised when a row's new maximum
+// exceeds it by more than 2^8 (lazy rescale): probabilities are then at most
+// 2^8 instead of 1, which bf16/fp32 hold without loss, and the 64-register
+// rescale of the output accumulator drops out of almost every iteration.  The
+// result is the same softmax up to fp32 rounding.
 #include "bsa_common.h"
+
+#include <type_traits>
 
 namespace bsa {
 namespace {
@@ -29,6 +43,8 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
 
 __device__ inline f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
@@ -42,14 +58,31 @@ template <> struct Vec8<_Float16> { typedef f16x8 type; };
 
 constexpr int kD = 128;          // head dim
 constexpr int kTile = 64;        // query rows per workgroup, keys per tile
+constexpr int kTileBytes = kTile * kD * 2;
 constexpr float kLog2e = 1.44269504f;
 constexpr float kLn2 = 0.6931471824645996f;
+constexpr float kLazyTau = 8.0f; // log2 headroom before the running max is raised
+constexpr int kListCap = 1024;   // tiles whose addresses are staged in LDS at a time
 
-// (x.lo16, y.lo16) and (x.hi16, y.hi16) packed into one dword
-__device__ inline uint32_t pack_lo(uint32_t x, uint32_t y) { return __builtin_amdgcn_perm(y, x, 0x05040100u); }
-__device__ inline uint32_t pack_hi(uint32_t x, uint32_t y) { return __builtin_amdgcn_perm(y, x, 0x07060302u); }
+typedef __attribute__((address_space(3))) void* lds_ptr;
+typedef const __attribute__((address_space(1))) void* gbl_ptr;
 
-__device__ inline int vt_swizzle(int d) { return (d & 7) ^ ((d >> 3) & 7); }
+// 16 bytes per lane from global memory straight into LDS.  The LDS address is
+// m0 + 16*lane; the global address is sbase + voff.  Issued from inline assembly
+// so that the compiler does not order later LDS reads of other stages behind it;
+// completion is awaited explicitly (s_waitcnt vmcnt) before the stage is read.
+__device__ inline void load_to_lds_16(const void* sbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+__device__ inline uint32_t lds_address(const void* p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+
+// 4 keys x 16 d patch -> this lane's d, 4 keys (see the header comment)
+__device__ inline s16x4 lds_read_tr16(const void* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
+}
 
 template <typename T>
 __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
@@ -58,8 +91,11 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     const uint64_t* __restrict__ tile_valid, T* __restrict__ o, float* __restrict__ lse,
     int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride, float qk_scale) {
     typedef typename Vec8<T>::type V8;
-    // [stage][0 = K tile, row-major | 1 = V tile, transposed][64*128]
-    __shared__ __attribute__((aligned(16))) T smem[2][2][kTile * kD];
+    // [stage][0 = K tile | 1 = V tile][64 rows x 128], rows swizzled in 16-byte chunks
+    __shared__ __attribute__((aligned(1024))) T smem[2][2][kTile * kD];
+    // the tile list of this query block: first key row and validity word per tile
+    __shared__ int32_t tile_row_sm[kListCap];
+    __shared__ uint64_t tile_mask_sm[kListCap];
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -73,8 +109,8 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     const int32_t* list = idx + ((int64_t)bh * nbq + qblock) * idx_stride;
     const int ntiles = lens[(int64_t)bh * nbq + qblock] * nsub;
 
-    const T* kbase = k + (int64_t)bh * Sk * kD;
-    const T* vbase = v + (int64_t)bh * Sk * kD;
+    const char* kbase = reinterpret_cast<const char*>(k + (int64_t)bh * Sk * kD);
+    const char* vbase = reinterpret_cast<const char*>(v + (int64_t)bh * Sk * kD);
 
     // Q as the B operand: lane holds row 32*qh + lr, d = 16*s + 8*lh .. +8
     V8 qreg[8];
@@ -82,51 +118,50 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
         const T* qp = q + ((int64_t)bh * Sq + qrow0 + 32 * qh + lr) * kD + 8 * lh;
 #pragma unroll
         for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const V8*>(qp + 16 * s);
+        // consume the loads here: otherwise their vmcnt waits land inside the tile loop,
+        // where they would also wait for the LDS loads of the next tile
+#pragma unroll
+        for (int s = 0; s < 8; ++s) asm volatile("" :: "v"(qreg[s]));
     }
 
-    // staging roles
-    const int kc = tid & 15, kr = tid >> 4;   // K: 16-byte chunk kc of rows kr + 16*i
-    const int vd = tid & 15, vq = tid >> 4;   // V: d-octet vd of key rows 4*vq + i
-    const int v_chunk = ((vq >> 3) << 2) | (((vq >> 2) & 1) << 1) | (vq & 1);
-    const int v_half = (vq >> 1) & 1;
+    // ---- global -> LDS: load i of this wavefront fills LDS rows 4*(4*i + wave) .. +4 ----
+    // lane: physical row 16*i + 4*wave + lane/16, physical chunk lane%16,
+    // fetches logical chunk (lane%16) ^ f(row);  f_K(row) = row & 15, f_V(row) = (row & 3) << 2
+    const int drow = 4 * wave + (lane >> 4);
+    const uint32_t koff = (uint32_t)(drow * 256 + (((lane & 15) ^ (drow & 15)) << 4));
+    const uint32_t voff = (uint32_t)(drow * 256 + (((lane & 15) ^ ((drow & 3) << 2)) << 4));
+    uint32_t koffs[4], voffs[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { koffs[i] = koff + i * 4096u; voffs[i] = voff + i * 4096u; }
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(&smem[0][0][0]) + wave * 1024);
+    auto issue_tile = [&](int row0, int st) {
+        const char* kt = kbase + (int64_t)row0 * (kD * 2);
+        const char* vt = vbase + (int64_t)row0 * (kD * 2);
+        const uint32_t kl = lds0 + st * (2 * kTileBytes);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            load_to_lds_16(kt, koffs[i], kl + i * 4096);
+            load_to_lds_16(vt, voffs[i], kl + kTileBytes + i * 4096);
+        }
+    };
 
-    uint4 kreg[4], vreg[4];
-    auto tile_row0 = [&](int it) -> int64_t {
-        return (int64_t)list[it / nsub] * bs_k + (int64_t)(it % nsub) * kTile;
-    };
-    auto load_tile = [&](int64_t row0) {
+    // ---- LDS read addresses (element offsets inside a tile) ----
+    // K, A operand of S^T: row 32*kh + lr, logical chunk 2*c + lh
+    const int krow = 32 * kh + lr;
+    int kaddr[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            kreg[i] = *reinterpret_cast<const uint4*>(kbase + (row0 + kr + 16 * i) * kD + kc * 8);
-            vreg[i] = *reinterpret_cast<const uint4*>(vbase + (row0 + 4 * vq + i) * kD + vd * 8);
-        }
-    };
-    auto store_tile = [&](int st) {
-        T* ks = smem[st][0];
-        T* vt = smem[st][1];
+    for (int c = 0; c < 8; ++c) kaddr[c] = krow * kD + (((2 * c + lh) ^ (krow & 15)) << 3);
+    // V, transposing read for (d tile t, key step c, half r):
+    //   source lane s = lane%16 points at key 32*kh + 8*(2c + r) + 4*lh + s/4, d = 32*t + 16*g1 + 4*(s%4)
+    const int s16 = lane & 15, g1 = (lane >> 4) & 1;
+    const int vkey0 = 32 * kh + 4 * lh + (s16 >> 2);          // + 8*(2c + r)
+    const int vsw = (vkey0 & 3) << 2;                          // key & 3 does not depend on c, r
+    int vaddr[4];                                              // per d tile t, for key offset 0
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = kr + 16 * i;
-            *reinterpret_cast<uint4*>(ks + r * kD + ((kc ^ (r & 15)) << 3)) = kreg[i];
-        }
-        const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&vreg[0]);
-        const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&vreg[1]);
-        const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&vreg[2]);
-        const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&vreg[3]);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int d = 8 * vd + e;
-            uint2 w;
-            if (e & 1) {
-                w.x = pack_hi(r0[e >> 1], r1[e >> 1]);
-                w.y = pack_hi(r2[e >> 1], r3[e >> 1]);
-            } else {
-                w.x = pack_lo(r0[e >> 1], r1[e >> 1]);
-                w.y = pack_lo(r2[e >> 1], r3[e >> 1]);
-            }
-            *reinterpret_cast<uint2*>(vt + d * kTile + ((v_chunk ^ vt_swizzle(d)) << 3) + v_half * 4) = w;
-        }
-    };
+    for (int t = 0; t < 4; ++t) {
+        const int chunk = 4 * t + 2 * g1 + ((s16 & 3) >> 1);
+        vaddr[t] = vkey0 * kD + ((chunk ^ vsw) << 3) + (s16 & 1) * 4;
+    }
 
     f32x16 oacc[4];
 #pragma unroll
@@ -135,38 +170,39 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
         for (int i = 0; i < 16; ++i) oacc[t][i] = 0.f;
     float m_i = -INFINITY, l_i = 0.f;
 
-    uint64_t vmask_next = ~0ull;
-    if (ntiles > 0) {
-        const int64_t row0 = tile_row0(0);
-        if (tile_valid) vmask_next = tile_valid[row0 / kTile];
-        load_tile(row0);
-        store_tile(0);
+    for (int chunk0 = 0; chunk0 < ntiles; chunk0 += kListCap) {
+    const int nloc = min(ntiles - chunk0, kListCap);
+    __syncthreads();                          // previous chunk fully consumed
+    for (int j = tid; j < nloc; j += 256) {
+        const int it = chunk0 + j;
+        const int64_t row0 = (int64_t)list[it / nsub] * bs_k + (int64_t)(it % nsub) * kTile;
+        tile_row_sm[j] = (int)row0;
+        tile_mask_sm[j] = tile_valid ? tile_valid[row0 / kTile] : ~0ull;
     }
     __syncthreads();
+    issue_tile(__builtin_amdgcn_readfirstlane(tile_row_sm[0]), 0);
+    int row_next = nloc > 1 ? tile_row_sm[1] : 0;
 
-    for (int it = 0; it < ntiles; ++it) {
-        const int st = it & 1;
-        const uint64_t vmask = vmask_next;
-        if (it + 1 < ntiles) {
-            const int64_t row0 = tile_row0(it + 1);
-            if (tile_valid) vmask_next = tile_valid[row0 / kTile];
-            load_tile(row0);
-        }
+    // one tile; the stage is a compile-time constant so that every LDS address is a
+    // loop-invariant register plus an immediate offset
+    auto step = [&](int it, auto stage) {
+        constexpr int st = decltype(stage)::value;
+        const uint64_t vmask = tile_mask_sm[it];
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's share of tile `it` is in LDS
+        __syncthreads();                                     // ... and everybody else's; stage st^1 is free again
+        if (it + 1 < nloc) issue_tile(__builtin_amdgcn_readfirstlane(row_next), st ^ 1);
+        if (it + 2 < nloc) row_next = tile_row_sm[it + 2];
         const T* ks = smem[st][0];
-        const T* vt = smem[st][1];
+        const T* vs = smem[st][1];
 
         // S^T = K_half . Q^T
         f32x16 s;
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[i] = 0.f;
-        {
-            const int row = 32 * kh + lr;
-            const T* kp = ks + row * kD;
 #pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                const V8 a = *reinterpret_cast<const V8*>(kp + (((2 * c + lh) ^ (row & 15)) << 3));
-                s = mfma32(a, qreg[c], s);
-            }
+        for (int c = 0; c < 8; ++c) {
+            const V8 a = *reinterpret_cast<const V8*>(ks + kaddr[c]);
+            s = mfma32(a, qreg[c], s);
         }
         // accumulator i <-> key 32*kh + 8*(i/4) + 4*lh + i%4, query lr
         if (vmask != ~0ull) {
@@ -178,10 +214,21 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
         float mx = s[0];
 #pragma unroll
         for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_i, mx * qk_scale);
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_i - m_safe);
+        {   // combine with the other key group of the same query (lane ^ 32)
+            const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+            mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])) * qk_scale;
+        }
+        if (__any(mx > m_i + kLazyTau)) {
+            const float m_new = fmaxf(m_i, mx);
+            const float alpha = __builtin_amdgcn_exp2f(m_i - ((m_new == -INFINITY) ? 0.f : m_new));
+            m_i = m_new;
+            l_i *= alpha;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) oacc[t][i] *= alpha;
+        }
+        const float m_safe = (m_i == -INFINITY) ? 0.f : m_i;
         float psum = 0.f;
         float p[16];
 #pragma unroll
@@ -189,14 +236,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
             p[i] = __builtin_amdgcn_exp2f(fmaf(s[i], qk_scale, -m_safe));
             psum += p[i];
         }
-        l_i = fmaf(l_i, alpha, psum);
-        m_i = m_new;
-        if (__any(alpha != 1.0f)) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) oacc[t][i] *= alpha;
-        }
+        l_i += psum;
         // P^T as B operand: k-slot (lh, j) of step c <-> accumulator 8*c + j
         V8 pb[2];
 #pragma unroll
@@ -206,20 +246,24 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
         // O^T += V^T . P^T
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            const int d = 32 * t + lr;
-            const T* vp = vt + d * kTile;
-            const int sw = vt_swizzle(d);
 #pragma unroll
             for (int c = 0; c < 2; ++c) {
-                const V8 a = *reinterpret_cast<const V8*>(vp + (((kh * 4 + 2 * c + lh) ^ sw) << 3));
-                oacc[t] = mfma32(a, pb[c], oacc[t]);
+                const s16x4 lo = lds_read_tr16(vs + vaddr[t] + (8 * (2 * c)) * kD);
+                const s16x4 hi = lds_read_tr16(vs + vaddr[t] + (8 * (2 * c + 1)) * kD);
+                const s16x8 av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                oacc[t] = mfma32(__builtin_bit_cast(V8, av), pb[c], oacc[t]);
             }
         }
-        if (it + 1 < ntiles) store_tile(st ^ 1);
-        __syncthreads();
+    };
+    for (int it = 0; it < nloc; it += 2) {
+        step(it, std::integral_constant<int, 0>{});
+        if (it + 1 < nloc) step(it + 1, std::integral_constant<int, 1>{});
     }
+    }
+    __syncthreads();
 
     // ---- epilogue: merge the two key halves, normalise, store coalesced ----
+    const int kc = tid & 15, kr = tid >> 4;
     float* xch = reinterpret_cast<float*>(&smem[0][0][0]);                  // [qh][66][64] fp32
     T* ost = reinterpret_cast<T*>(reinterpret_cast<char*>(xch) + 2 * 66 * 64 * 4);   // [64][128]
     if (kh == 1) {
