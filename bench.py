@@ -33,6 +33,9 @@ WORKLOADS = {
     "c2": ((24, 30, 52), 0.9375, 1, False, "480p layer: 32 heads x 128, grid 24x30x52 (37440 tokens), density 1/16"),
     "c3": ((24, 45, 80), 0.9375, 2, True, "720p layer: 32 heads x 128, grid 24x45x80 (86400 tokens), density 1/16"),
 }
+# HBM-side bytes per launch of the attention kernel, from rocprofv3 --pmc FETCH_SIZE (x2) and
+# WRITE_SIZE (x1) as recorded in profiles/bsa_operator_c3_720p.md; re-measure after kernel changes.
+ATTENTION_TRAFFIC_BYTES = {"c3": 124999.7e6 + 762.8e6}
 CHUNK = (4, 4, 4)
 HEADS, D = 32, 128
 
@@ -185,7 +188,7 @@ def main():
         "permute_gbs": round(permute_bytes / (ms_permute * 1e-3) / 1e9, 1),
         "roofline": {"kernel": "fwd_mfma_kernel<bf16>", "bound": "mfma", "achieved": round(tflops_attn, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops_attn / PEAK_BF16_TFLOPS, 4),
-                     "traffic": None, "ms": round(ms_attn, 4)},
+                     "traffic": ATTENTION_TRAFFIC_BYTES.get(args.workload), "ms": round(ms_attn, 4)},
     }
     del o
     if not args.no_cpu_baseline:
