@@ -164,6 +164,33 @@ int bsa_fwd_3d(const bsa_3d_params* p,
                void* workspace, size_t workspace_bytes,
                int32_t* idx_out, int32_t* lens_out, void* score_out, void* stream);
 
+/*
+ * R11 glue of the attention module (longcat_video/modules/attention.py:107-147).
+ */
+
+/* Row RMSNorm: out = cast(x * rsqrt(mean(x^2) + eps)) * weight, rows of `dim` elements (dim % 8 == 0),
+ * fp32 statistics, result rounded to `dtype` before and after the weight multiply.
+ * Replaces RMSNorm_FP32.forward, longcat_video/modules/blocks.py:42-53.  bf16 / fp16. */
+int bsa_rmsnorm(const void* x, const void* weight, void* out, int64_t rows, int dim, float eps,
+                int dtype, void* stream);
+
+/* In-place per-head RMSNorm (blocks.py:42-53, called attention.py:116) followed by 3-D RoPE
+ * (longcat_video/modules/rope_3d.py:99-120, called attention.py:121) on q and k.
+ *   q, k  [B, Hn, T*H*W, 128] with element strides {B, Hn, S} (views of the QKV projection are fine)
+ *   q_weight, k_weight  [128] in `dtype`
+ *   rope_table  fp32, concatenation of cos_t[T][22], sin_t[T][22], cos_h[H][21], sin_h[H][21],
+ *               cos_w[W][21], sin_w[W][21]: cos/sin of position * frequency per rotation pair
+ *               (rope_3d.py:70-87; the d axis is split 44/42/42 between t, h, w) */
+int bsa_qk_norm_rope(void* q, const int64_t q_strides[3], void* k, const int64_t k_strides[3],
+                     const void* q_weight, const void* k_weight, const float* rope_table,
+                     int B, int Hn, int T, int H, int W, int D, float eps, int dtype, void* stream);
+
+/* out[M,N] = x[M,K] . w[N,K]^T (+ bias[N]) (+ residual[M,N]), bf16 in/out, fp32 accumulate, on MFMA
+ * through hipBLASLt.  Replaces the nn.Linear calls attention.py:111 and :142.  `workspace` may be
+ * null with workspace_bytes 0.  Creates one process-wide hipBLASLt handle on first use. */
+int bsa_linear_bf16(const void* x, const void* w, const void* bias, const void* residual, void* out,
+                    int64_t M, int N, int K, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -237,7 +237,8 @@ def flash_attn_bsa(q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold,
 # ---------------------------------------------------------------------------
 # R9: the operator
 # ---------------------------------------------------------------------------
-def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k, want_selection=False):
+def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k, want_selection=False, out=None):
+    """`out`: optional [B,H,Sq,D] view (any B/H/S strides, contiguous D) to write into."""
     _need_gpu(q, k, v)
     B, H, Sq, D = q.shape
     Tq, Hq, Wq = (int(x) for x in latent_shape_q)
@@ -256,7 +257,8 @@ def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k,
         _capi.check(lib.bsa_fwd_3d(C.byref(prm), None, None, None, None, None, None, None, None, None, 0,
                                    None, None, None, None), "flash_attn_bsa_3d")
     ws = torch.empty(need, dtype=torch.uint8, device=q.device)
-    o = torch.empty(B, H, Sq, D, dtype=q.dtype, device=q.device)
+    o = torch.empty(B, H, Sq, D, dtype=q.dtype, device=q.device) if out is None else out
+    assert o.shape == (B, H, Sq, D) and o.dtype == q.dtype and o.stride(3) == 1
     idx = lens = score = None
     if want_selection:
         idx = torch.empty(B, H, nbq, k_sel, dtype=torch.int32, device=q.device)

@@ -1,0 +1,208 @@
+"""Self-attention module of the LongCat-Video DiT on the MI355X engine.
+
+Mirrors ``Attention`` of the reference (longcat_video/modules/attention.py:14-181):
+same constructor arguments, same parameter names (``qkv``, ``q_norm.weight``,
+``k_norm.weight``, ``proj``) so a reference state dict loads unchanged, same
+``forward(x, shape, num_cond_latents)`` contract.  Every stage runs through the
+C-ABI of the engine:
+
+    qkv = Linear(x)                      bsa_linear_bf16   (attention.py:111)
+    q, k = RMSNorm(q), RMSNorm(k); RoPE  bsa_qk_norm_rope  (attention.py:116, :121)
+    block-sparse attention               bsa_fwd_3d        (attention.py:58-67, :124-137)
+    x = Linear(o)                        bsa_linear_bf16   (attention.py:139-142)
+
+q, k, v stay strided views of the projection output and the attention output is
+written token-major, so none of the reference's ``.contiguous()`` / transpose
+copies (attention.py:127-135, :140-141) exist here.  Only the block-sparse branch
+is built: dense back ends (flash-attn, xformers) and the KV-cache variant
+(attention.py:149-181) raise ``NotImplementedError``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import List, Optional
+
+import torch
+import torch.nn as nn
+
+from .. import _capi
+from ..block_sparse_attention.bsa_interface import _bsa_3d, _ptr, _stream
+
+
+class RMSNorm_FP32(nn.Module):
+    """Parameter holder with the reference's name and layout (blocks.py:42-53);
+    ``forward`` normalises rows of ``dim`` elements with the engine's kernel."""
+
+    def __init__(self, dim: int, eps: float):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return rms_norm(x, self.weight, self.eps)
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    if not x.is_cuda:
+        raise RuntimeError("the engine runs on the GPU only")
+    x = x.contiguous()
+    w = weight.to(x.dtype).contiguous()
+    out = torch.empty_like(x)
+    dim = x.shape[-1]
+    code = {torch.bfloat16: _capi.BSA_BF16, torch.float16: _capi.BSA_F16}.get(x.dtype)
+    if code is None:
+        raise NotImplementedError("rms_norm: dtype %s is not built (bf16, fp16)" % x.dtype)
+    with torch.cuda.device(x.device):
+        _capi.check(_capi.load().bsa_rmsnorm(_ptr(x), _ptr(w), _ptr(out), x.numel() // dim, dim, float(eps), code,
+                                             _stream(x)), "rmsnorm")
+    return out
+
+
+def linear_bf16(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                residual: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x @ weight.T + bias (+ residual)`` for bf16 tensors, weight in nn.Linear layout [out, in]."""
+    if not x.is_cuda:
+        raise RuntimeError("the engine runs on the GPU only")
+    if x.dtype != torch.bfloat16:
+        raise NotImplementedError("linear: only bf16 is built")
+    K = x.shape[-1]
+    N = weight.shape[0]
+    assert weight.shape[1] == K
+    x2 = x.reshape(-1, K).contiguous()
+    w = weight.to(torch.bfloat16).contiguous()
+    b = None if bias is None else bias.to(torch.bfloat16).contiguous()
+    out = torch.empty(x2.shape[0], N, dtype=torch.bfloat16, device=x.device)
+    r = None
+    if residual is not None:
+        r = residual.reshape(-1, N).contiguous()
+        assert r.shape == out.shape and r.dtype == torch.bfloat16
+    if workspace is None:
+        workspace = torch.empty(32 << 20, dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        _capi.check(_capi.load().bsa_linear_bf16(_ptr(x2), _ptr(w), _ptr(b), _ptr(r), _ptr(out), x2.shape[0], N, K,
+                                                 _ptr(workspace), workspace.numel(), _stream(x)), "linear")
+    return out.view(*x.shape[:-1], N)
+
+
+_ROPE_TABLES = {}
+
+
+def rope_table(grid_size, head_dim: int, device, base: float = 10000.0) -> torch.Tensor:
+    """cos/sin of position x frequency per axis and rotation pair, following
+    rope_3d.py:68-87 (axis dims D-4*(D//6), 2*(D//6), 2*(D//6); frequency i of an
+    axis = base^(-2i/dim_axis); integer grid positions), evaluated in fp32 on the
+    device like the reference (rope_3d.py:112-115).  Layout: cos_t, sin_t, cos_h,
+    sin_h, cos_w, sin_w, each [positions, pairs]."""
+    key = (tuple(int(g) for g in grid_size), head_dim, str(device), base)
+    tab = _ROPE_TABLES.get(key)
+    if tab is None:
+        dims = (head_dim - 4 * (head_dim // 6), 2 * (head_dim // 6), 2 * (head_dim // 6))
+        parts = []
+        for n, dim in zip(key[0], dims):
+            freqs = 1.0 / (base ** (torch.arange(0, dim, 2)[: dim // 2].float() / dim))
+            ang = (torch.arange(n, dtype=torch.float32)[:, None] * freqs[None, :]).to(device)
+            parts += [ang.cos().reshape(-1), ang.sin().reshape(-1)]
+        tab = torch.cat(parts).contiguous()
+        _ROPE_TABLES[key] = tab
+    return tab
+
+
+def qk_norm_rope_(q: torch.Tensor, k: torch.Tensor, q_weight, k_weight, grid_size, eps: float = 1e-6) -> None:
+    """In place on q and k ([B,H,S,128] views, contiguous D): per-head RMSNorm then 3-D RoPE."""
+    B, H, S, D = q.shape
+    T, Hg, Wg = (int(g) for g in grid_size)
+    assert k.shape == q.shape and S == T * Hg * Wg and q.stride(3) == 1 and k.stride(3) == 1
+    code = {torch.bfloat16: _capi.BSA_BF16, torch.float16: _capi.BSA_F16}.get(q.dtype)
+    if code is None:
+        raise NotImplementedError("qk_norm_rope: dtype %s is not built (bf16, fp16)" % q.dtype)
+    tab = rope_table(grid_size, D, q.device)
+    qw, kw = q_weight.to(q.dtype).contiguous(), k_weight.to(q.dtype).contiguous()
+    with torch.cuda.device(q.device):
+        _capi.check(_capi.load().bsa_qk_norm_rope(
+            _ptr(q), _capi.strides3(q.stride()[:3]), _ptr(k), _capi.strides3(k.stride()[:3]), _ptr(qw), _ptr(kw),
+            _ptr(tab), B, H, T, Hg, Wg, D, float(eps), code, _stream(q)), "qk_norm_rope")
+
+
+class Attention(nn.Module):
+    def __init__(
+        self,
+        dim: int,
+        num_heads: int,
+        enable_flashattn3: bool = False,
+        enable_flashattn2: bool = False,
+        enable_xformers: bool = False,
+        enable_bsa: bool = False,
+        bsa_params: dict = None,
+        cp_split_hw: Optional[List[int]] = None,
+    ) -> None:
+        super().__init__()
+        assert dim % num_heads == 0, "dim should be divisible by num_heads"
+        self.dim = dim
+        self.num_heads = num_heads
+        self.head_dim = dim // num_heads
+        self.scale = self.head_dim ** -0.5
+        self.enable_flashattn3 = enable_flashattn3
+        self.enable_flashattn2 = enable_flashattn2
+        self.enable_xformers = enable_xformers
+        self.enable_bsa = enable_bsa
+        self.bsa_params = bsa_params
+        self.cp_split_hw = cp_split_hw if cp_split_hw is not None else [1, 1]
+
+        self.qkv = nn.Linear(dim, dim * 3, bias=True)
+        self.q_norm = RMSNorm_FP32(self.head_dim, eps=1e-6)
+        self.k_norm = RMSNorm_FP32(self.head_dim, eps=1e-6)
+        self.proj = nn.Linear(dim, dim)
+
+    def _process_attn(self, q, k, v, shape, out=None):
+        """attention.py:50-105, block-sparse branch; writes into `out` ([B,H,SQ,D] view) if given."""
+        B, H, SQ, D = q.shape
+        SKV = k.shape[2]
+        if not (self.enable_bsa and shape[0] > 1):
+            raise NotImplementedError("only the block-sparse branch (enable_bsa, more than one latent frame) is built")
+        assert self.bsa_params is not None
+        _, Hh, W = shape
+        if self.cp_split_hw[0] * self.cp_split_hw[1] != 1:
+            raise NotImplementedError("context parallelism is not built: one GPU holds every head and token")
+        Tq, Tk = SQ // (Hh * W), SKV // (Hh * W)
+        prm = dict(sparsity=0.875, cdf_threshold=None, chunk_3d_shape_q=[4, 4, 8], chunk_3d_shape_k=[4, 4, 8])
+        prm.update(self.bsa_params)
+        if prm["cdf_threshold"] is not None:
+            raise NotImplementedError("CDF-threshold selection is not built; pass cdf_threshold=None")
+        if prm["sparsity"] is None:
+            raise ValueError
+        return _bsa_3d(q, k, v, (Tq, Hh, W), (Tk, Hh, W), float(prm["sparsity"]), prm["chunk_3d_shape_q"],
+                       prm["chunk_3d_shape_k"], out=out)
+
+    @torch.no_grad()
+    def forward(self, x: torch.Tensor, shape=None, num_cond_latents=None, return_kv=False,
+                residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """attention.py:107-147.  `residual` (extension): added to the projection output inside the GEMM."""
+        if return_kv:
+            raise NotImplementedError("the KV-cache variant is not built")
+        B, N, C = x.shape
+        Hn, D = self.num_heads, self.head_dim
+        qkv = linear_bf16(x, self.qkv.weight, self.qkv.bias)                      # [B, N, 3C]
+        q, k, v = qkv.view(B, N, 3, Hn, D).permute(2, 0, 3, 1, 4).unbind(0)       # strided [B, H, N, D] views
+        qk_norm_rope_(q, k, self.q_norm.weight, self.k_norm.weight, shape, self.q_norm.eps)
+
+        o = torch.empty(B, N, Hn, D, dtype=x.dtype, device=x.device)             # token-major: reshape below is free
+        ov = o.permute(0, 2, 1, 3)                                                # [B, H, N, D] view
+        if num_cond_latents is not None and num_cond_latents > 0:
+            n = num_cond_latents * (N // shape[0])
+            self._process_attn(q[:, :, :n], k[:, :, :n], v[:, :, :n], shape, out=ov[:, :, :n])   # attention.py:127-130
+            self._process_attn(q[:, :, n:], k, v, shape, out=ov[:, :, n:])                       # attention.py:132-133
+        else:
+            self._process_attn(q, k, v, shape, out=ov)
+        return linear_bf16(o.view(B, N, C), self.proj.weight, self.proj.bias, residual=residual)
+
+    def forward_with_kv_cache(self, *args, **kwargs):
+        raise NotImplementedError("the KV-cache variant (attention.py:149-181) is not built")
+
+
+@torch.no_grad()
+def attention_block_forward(x: torch.Tensor, pre_norm_weight: torch.Tensor, attn: Attention, shape,
+                            num_cond_latents=None, eps: float = 1e-6) -> torch.Tensor:
+    """RMSNorm -> QKV projection -> QK RMSNorm -> 3-D RoPE -> block-sparse attention -> out projection
+    -> residual: the attention sub-chain of one DiT block as BASELINE config 5 words it."""
+    y = rms_norm(x, pre_norm_weight, eps)
+    return attn(y, shape=shape, num_cond_latents=num_cond_latents, residual=x)

@@ -118,6 +118,27 @@ def test_480p_two_heads():
     check_against_oracle(q, k, v, latent, latent, 0.9375, o, idx, lens, score, q_blocks=[0, 12, 300, 611, 623])
 
 
+def test_long_video_continuation_two_heads():
+    """BASELINE config 4 geometry with 2 heads: grid 48x30x52, the first 12 latent frames are
+    conditioning tokens.  Two operator calls as in attention.py:124-135: conditioning queries
+    against conditioning keys (312 blocks, 39 kept), noise queries against all keys
+    (936 x 1248 blocks, 156 kept)."""
+    T, Hh, W, cond = 48, 30, 52, 12
+    S, n = T * Hh * W, cond * Hh * W
+    q, k, v = seeded_qkv(3, 1, 2, S, S, 128, torch.bfloat16)
+    dq, dk, dv = q.cuda(), k.cuda(), v.cuda()
+    out = torch.empty(1, S, 2, 128, dtype=torch.bfloat16, device="cuda").permute(0, 2, 1, 3)
+    o_c, idx_c, lens_c, score_c = I()._bsa_3d(dq[:, :, :n], dk[:, :, :n], dv[:, :, :n], (cond, Hh, W), (cond, Hh, W),
+                                              0.875, (4, 4, 4), (4, 4, 4), True, out=out[:, :, :n])
+    o_n, idx_n, lens_n, score_n = I()._bsa_3d(dq[:, :, n:], dk, dv, (T - cond, Hh, W), (T, Hh, W),
+                                              0.875, (4, 4, 4), (4, 4, 4), True, out=out[:, :, n:])
+    assert idx_c.shape == (1, 2, 312, 39) and idx_n.shape == (1, 2, 936, 156)
+    check_against_oracle(q[:, :, :n], k[:, :, :n], v[:, :, :n], (cond, Hh, W), (cond, Hh, W), 0.875,
+                         out[:, :, :n], idx_c, lens_c, score_c, q_blocks=[0, 155, 311])
+    check_against_oracle(q[:, :, n:], k, v, (T - cond, Hh, W), (T, Hh, W), 0.875,
+                         out[:, :, n:], idx_n, lens_n, score_n, q_blocks=[0, 500, 935])
+
+
 def test_720p_full_shape_sampled():
     """BASELINE config 3 at full size (32 heads, 86 400 tokens, RMS-normalised q/k,
     density 1/16): two heads are checked against the oracle on sampled query
