@@ -150,7 +150,7 @@ def main():
     vp, _, _ = I._permute(v, latent, CHUNK)
     nbq, nbk = q_cmp.shape[2], k_cmp.shape[2]
     k_sel = I.num_selected(sparsity, nbk)
-    idx, lens, _ = I._score_topk(q_cmp, k_cmp, k_sel)
+    idx, lens, _ = I._score_topk(q_cmp, k_cmp, k_sel, order="block")      # the order the operator itself uses
     padded = any(n % c for n, c in zip(latent, CHUNK))
     tv = valid if padded else None
     scale = 1 / math.sqrt(D)
@@ -186,7 +186,7 @@ def main():
         "kernels_ms": {"attention": round(ms_attn, 4), "permute_pool_one_tensor": round(ms_permute, 4),
                        "unpermute": round(ms_unpermute, 4), "score_topk": round(ms_select, 4)},
         "permute_gbs": round(permute_bytes / (ms_permute * 1e-3) / 1e9, 1),
-        "roofline": {"kernel": "fwd_mfma_kernel<bf16>", "bound": "mfma", "achieved": round(tflops_attn, 2),
+        "roofline": {"kernel": "fwd_mfma_kernel<bf16> (all launches of one layer)", "bound": "mfma", "achieved": round(tflops_attn, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops_attn / PEAK_BF16_TFLOPS, 4),
                      "traffic": ATTENTION_TRAFFIC_BYTES.get(args.workload), "ms": round(ms_attn, 4)},
     }

@@ -103,17 +103,20 @@ int bsa_mean_pool(const void* x, void* out, int B, int Hn, int64_t S, int block,
  *   score = q_cmp . k_cmp^T, fp32 accumulate, rounded once to `dtype`, unscaled
  *   idx_out   int32 [B, Hn, nbq, k_sel]: the k_sel best blocks of every row in
  *             descending score order, ties broken towards the lowest index
+ *   idx_sorted_out  the same set in ascending block index (the order in which
+ *             the attention kernel is most cache friendly); at least one of
+ *             idx_out / idx_sorted_out must be given
  *   lens_out  int32 [B, Hn, nbq], every entry k_sel (bsa:217-222)
  *   score_out optional [B, Hn, nbq, nbk] in `dtype`
  * Limits: D == 128, 0 <= k_sel <= nbk <= 4096, k_sel <= 1024.
  * NaN scores order above +inf, as torch.topk orders them.
  */
-int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32_t* lens_out,
-                   void* score_out, int B, int Hn, int nbq, int nbk, int D, int k_sel,
-                   int dtype, void* stream);
+int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32_t* idx_sorted_out,
+                   int32_t* lens_out, void* score_out, int B, int Hn, int nbq, int nbk, int D,
+                   int k_sel, int dtype, void* stream);
 
 /* R4 alone, from a caller-supplied score tensor [B, Hn, nbq, nbk] in `dtype`. */
-int bsa_topk_from_score(const void* score, int32_t* idx_out, int32_t* lens_out,
+int bsa_topk_from_score(const void* score, int32_t* idx_out, int32_t* idx_sorted_out, int32_t* lens_out,
                         int B, int Hn, int nbq, int nbk, int k_sel, int dtype, void* stream);
 
 /*

@@ -135,17 +135,17 @@ static int check_topk(int B, int Hn, int nbq, int nbk, int k_sel, int dtype) {
     return BSA_OK;
 }
 
-int bsa_topk_from_score(const void* score, int32_t* idx_out, int32_t* lens_out, int B, int Hn, int nbq,
-                        int nbk, int k_sel, int dtype, void* stream) {
-    if (!score || !idx_out || !lens_out) return set_error(BSA_ERR_BAD_ARG, "top-k: null pointer");
+int bsa_topk_from_score(const void* score, int32_t* idx_out, int32_t* idx_sorted_out, int32_t* lens_out, int B,
+                        int Hn, int nbq, int nbk, int k_sel, int dtype, void* stream) {
+    if (!score || !lens_out || (!idx_out && !idx_sorted_out)) return set_error(BSA_ERR_BAD_ARG, "top-k: null pointer");
     BSA_TRY(check_topk(B, Hn, nbq, nbk, k_sel, dtype));
-    const hipError_t e = launch_topk(score, idx_out, lens_out, (int64_t)B * Hn * nbq, nbk, k_sel, dtype, (hipStream_t)stream);
+    const hipError_t e = launch_topk(score, idx_out, idx_sorted_out, lens_out, (int64_t)B * Hn * nbq, nbk, k_sel, dtype, (hipStream_t)stream);
     return e == hipSuccess ? BSA_OK : hip_fail(e, "top-k launch");
 }
 
-int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32_t* lens_out, void* score_out,
-                   int B, int Hn, int nbq, int nbk, int D, int k_sel, int dtype, void* stream) {
-    if (!q_cmp || !k_cmp || !idx_out || !lens_out) return set_error(BSA_ERR_BAD_ARG, "score_topk: null pointer");
+int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32_t* idx_sorted_out, int32_t* lens_out,
+                   void* score_out, int B, int Hn, int nbq, int nbk, int D, int k_sel, int dtype, void* stream) {
+    if (!q_cmp || !k_cmp || !lens_out || (!idx_out && !idx_sorted_out)) return set_error(BSA_ERR_BAD_ARG, "score_topk: null pointer");
     if (!score_out) return set_error(BSA_ERR_BAD_ARG, "score_topk: a score buffer of B*heads*nbq*nbk elements is required");
     BSA_TRY(check_topk(B, Hn, nbq, nbk, k_sel, dtype));
     if (D <= 0 || D % 16 != 0 || D > 256) return set_error(BSA_ERR_UNSUPPORTED, "score: head dim %d must be a multiple of 16, at most 256", D);
@@ -153,7 +153,7 @@ int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32
     if (!aligned16(q_cmp) || !aligned16(k_cmp)) return set_error(BSA_ERR_BAD_ARG, "score: pooled tensors must be 16-byte aligned");
     hipError_t e = launch_score(q_cmp, k_cmp, score_out, B * Hn, nbq, nbk, D, dtype, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "score launch");
-    e = launch_topk(score_out, idx_out, lens_out, (int64_t)B * Hn * nbq, nbk, k_sel, dtype, (hipStream_t)stream);
+    e = launch_topk(score_out, idx_out, idx_sorted_out, lens_out, (int64_t)B * Hn * nbq, nbk, k_sel, dtype, (hipStream_t)stream);
     return e == hipSuccess ? BSA_OK : hip_fail(e, "top-k launch");
 }
 
@@ -171,6 +171,8 @@ int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, con
     if (Sq % bs_q != 0 || Sk % bs_k != 0)
         return set_error(BSA_ERR_SHAPE, "fwd: Sq=%lld / Sk=%lld are not multiples of the chunk sizes %d / %d", (long long)Sq, (long long)Sk, bs_q, bs_k);
     if (!(sm_scale > 0.f) || !std::isfinite(sm_scale)) return set_error(BSA_ERR_BAD_ARG, "fwd: sm_scale must be positive and finite");
+    if ((Sq / 64) * (int64_t)B * Hn > 0x7fffffffLL || Sk > 0x7fffffffLL)
+        return set_error(BSA_ERR_UNSUPPORTED, "fwd: problem too large for 32-bit work item / key row indices");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
         return set_error(BSA_ERR_BAD_ARG, "fwd: q/k/v/o must be 16-byte aligned");
     const hipError_t e = launch_fwd(q, k, v, idx, lens, tile_valid, o, lse, B, Hn, Sq, Sk, bs_q, bs_k, idx_stride,
@@ -184,7 +186,7 @@ struct Plan {
     Grid3 gq, gk;
     int64_t Sqp, Skp;
     int nbq, nbk, es;
-    size_t off_qp, off_kp, off_vp, off_op, off_qc, off_kc, off_score, off_idx, off_lens, off_valid, total;
+    size_t off_qp, off_kp, off_vp, off_op, off_qc, off_kc, off_score, off_idx, off_idx_sorted, off_lens, off_valid, total;
 };
 inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
@@ -216,6 +218,7 @@ int make_plan(const bsa_3d_params* p, Plan* pl) {
     pl->off_kc = take(bh * pl->nbk * p->D * pl->es);
     pl->off_score = take(bh * pl->nbq * (size_t)pl->nbk * pl->es);
     pl->off_idx = take(bh * pl->nbq * (size_t)(p->k_sel > 0 ? p->k_sel : 1) * sizeof(int32_t));
+    pl->off_idx_sorted = take(bh * pl->nbq * (size_t)(p->k_sel > 0 ? p->k_sel : 1) * sizeof(int32_t));
     pl->off_lens = take(bh * pl->nbq * sizeof(int32_t));
     pl->off_valid = take((size_t)(pl->Skp / 64) * sizeof(uint64_t));
     pl->total = off;
@@ -250,6 +253,7 @@ int bsa_fwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3]
     void* qp = ws + pl.off_qp; void* kp = ws + pl.off_kp; void* vp = ws + pl.off_vp; void* op = ws + pl.off_op;
     void* qc = ws + pl.off_qc; void* kc = ws + pl.off_kc; void* score = ws + pl.off_score;
     int32_t* idx = reinterpret_cast<int32_t*>(ws + pl.off_idx);
+    int32_t* idx_sorted = reinterpret_cast<int32_t*>(ws + pl.off_idx_sorted);
     int32_t* lens = reinterpret_cast<int32_t*>(ws + pl.off_lens);
     uint64_t* valid = reinterpret_cast<uint64_t*>(ws + pl.off_valid);
     const bool padded_k = (p->Tk % p->tk) || (p->Hk % p->hk) || (p->Wk % p->wk);
@@ -260,8 +264,10 @@ int bsa_fwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3]
     BSA_HIP(launch_permute(k, k_strides, kp, kc, padded_k ? valid : nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st), "permute k");
     BSA_HIP(launch_permute(v, v_strides, vp, nullptr, nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st), "permute v");
     BSA_HIP(launch_score(qc, kc, score, p->B * p->Hn, pl.nbq, pl.nbk, p->D, p->dtype, st), "score");
-    BSA_HIP(launch_topk(score, idx, lens, (int64_t)p->B * p->Hn * pl.nbq, pl.nbk, p->k_sel, p->dtype, st), "top-k");
-    BSA_HIP(launch_fwd(qp, kp, vp, idx, lens, padded_k ? valid : nullptr, op, nullptr, p->B, p->Hn, pl.Sqp, pl.Skp,
+    // the attention kernel walks each list in ascending block order (L2 locality); the score
+    // order is only produced when the caller asks for the selection
+    BSA_HIP(launch_topk(score, idx_out ? idx : nullptr, idx_sorted, lens, (int64_t)p->B * p->Hn * pl.nbq, pl.nbk, p->k_sel, p->dtype, st), "top-k");
+    BSA_HIP(launch_fwd(qp, kp, vp, idx_sorted, lens, padded_k ? valid : nullptr, op, nullptr, p->B, p->Hn, pl.Sqp, pl.Skp,
                        pl.gq.chunk(), pl.gk.chunk(), p->k_sel, p->sm_scale, p->dtype, st), "attention");
     BSA_HIP(launch_unpermute(op, o, o_strides, p->B, p->Hn, pl.gq, p->D, p->dtype, st), "unpermute");
     const size_t bh = (size_t)p->B * p->Hn;

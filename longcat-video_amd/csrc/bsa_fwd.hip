@@ -2,22 +2,21 @@
 // plain fp32 kernel for fp32 inputs.
 //
 // Work decomposition (MFMA kernel).  One workgroup = 256 threads = 4
-// wavefronts owns 64 query rows and walks the list of selected KV blocks in
-// 64-key tiles.  Wavefront (qh, kh) owns query rows 32*qh..+32 and keys
-// 32*kh..+32 of every tile and runs an independent online softmax over its
-// key half; the two halves are merged once, in the epilogue, with the usual
-// log-sum-exp rescale.  No per-tile exchange between wavefronts is needed.
+// wavefronts processes one work item at a time: 64 query rows against the
+// list of selected KV blocks, walked in 64-key tiles.  Wavefront (qh, kh) owns
+// query rows 32*qh..+32 and keys 32*kh..+32 of every tile and runs an
+// independent online softmax over its key half; the two halves are merged once
+// per work item, in the epilogue, with the usual log-sum-exp rescale.
 //
 // Per tile and wavefront: S^T (32 keys x 32 queries) = K_half . Q^T as 8
 // v_mfma_f32_32x32x16 over d = 128 (A = K rows from LDS, B = Q held in
-// registers for the whole kernel), so every lane ends up with one query column
-// and 16 keys: the softmax state (running max, running sum) is one scalar per
-// lane, and P^T in the accumulator registers already has the layout the B
-// operand of the second product needs.  O^T (128 d x 32 queries) += V^T . P^T
-// is 8 more MFMAs whose A operand (d along lanes, keys along the k slots) is
-// read from the row-major V tile with the transposing LDS read
-// ds_read_b64_tr_b16: 16 lanes fetch a 4-key x 16-d patch and each lane
-// receives the 4 keys of one d.
+// registers), so every lane ends up with one query column and 16 keys: the
+// softmax state (running max, running sum) is one scalar per lane, and P^T in
+// the accumulator registers already has the layout the B operand of the second
+// product needs.  O^T (128 d x 32 queries) += V^T . P^T is 8 more MFMAs whose A
+// operand (d along lanes, keys along the k slots) is read from the row-major V
+// tile with the transposing LDS read ds_read_b64_tr_b16: 16 lanes fetch a
+// 4-key x 16-d patch and each lane receives the 4 keys of one d.
 //
 // Data movement.  K and V tiles go from global memory straight into LDS
 // (global_load_lds_dwordx4, no staging registers): every wavefront issues
@@ -25,14 +24,29 @@
 // lane index, so the XOR swizzle that keeps the later LDS reads free of bank
 // conflicts is applied on the global side: lane l of a load fetches the
 // 16-byte chunk (l%16) ^ f(row) of its row.  Two stages of (K 16 KB + V 16 KB)
-// per workgroup, two workgroups per CU; the tile for iteration i+1 is in
-// flight while iteration i computes, one barrier per iteration.
+// per workgroup, two workgroups per CU, one barrier per tile.
+//
+// Software pipeline.  MFMA and plain VALU instructions of one SIMD do not
+// overlap on this hardware (measured), but transcendental instructions do, and
+// a wavefront that waits on an MFMA result leaves the SIMD to its neighbour.
+// In iteration i the 8 MFMAs of S(i+1) are therefore interleaved with the
+// exp2 of tile i, and the 8 MFMAs of O += P(i) V(i) with the row sum.
 //
 // Softmax.  The running maximum is only raised when a row's new maximum
 // exceeds it by more than 2^8 (lazy rescale): probabilities are then at most
 // 2^8 instead of 1, which bf16/fp32 hold without loss, and the 64-register
 // rescale of the output accumulator drops out of almost every iteration.  The
 // result is the same softmax up to fp32 rounding.
+//
+// Scheduling.  The work items of one (batch, head) are launched in rounds of as
+// many workgroups as the device runs at once (2 per CU).  The workgroups of a
+// round start together and, because every item of a top-k selection has the
+// same number of tiles, stay roughly in step.  With KV lists in ascending block
+// order the workgroups of an XCD then sweep the K/V of a head in the same
+// direction at the same time, which turns a large part of the tile fetches into
+// L2 hits (the 4 MB L2 of an XCD cannot hold the 47 MB of K/V of one 720p head,
+// and L2 misses are served at only ~8 TB/s for 16 KB tiles).  One launch of the
+// whole grid loses this: workgroups then start whenever a slot frees up.
 #include "bsa_common.h"
 
 #include <type_traits>
@@ -57,15 +71,12 @@ template <> struct Vec8<__bf16> { typedef bf16x8 type; };
 template <> struct Vec8<_Float16> { typedef f16x8 type; };
 
 constexpr int kD = 128;          // head dim
-constexpr int kTile = 64;        // query rows per workgroup, keys per tile
+constexpr int kTile = 64;        // query rows per work item, keys per tile
 constexpr int kTileBytes = kTile * kD * 2;
 constexpr float kLog2e = 1.44269504f;
 constexpr float kLn2 = 0.6931471824645996f;
 constexpr float kLazyTau = 8.0f; // log2 headroom before the running max is raised
 constexpr int kListCap = 1024;   // tiles whose addresses are staged in LDS at a time
-
-typedef __attribute__((address_space(3))) void* lds_ptr;
-typedef const __attribute__((address_space(1))) void* gbl_ptr;
 
 // 16 bytes per lane from global memory straight into LDS.  The LDS address is
 // m0 + 16*lane; the global address is sbase + voff.  Issued from inline assembly
@@ -78,22 +89,20 @@ __device__ inline void load_to_lds_16(const void* sbase, uint32_t voff, uint32_t
 __device__ inline uint32_t lds_address(const void* p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
 }
-
 // 4 keys x 16 d patch -> this lane's d, 4 keys (see the header comment)
 __device__ inline s16x4 lds_read_tr16(const void* p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
 }
-
 template <typename T>
 __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
     const int32_t* __restrict__ idx, const int32_t* __restrict__ lens,
     const uint64_t* __restrict__ tile_valid, T* __restrict__ o, float* __restrict__ lse,
-    int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride, float qk_scale) {
+    int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride, float qk_scale, int item_begin, int item_end) {
     typedef typename Vec8<T>::type V8;
     // [stage][0 = K tile | 1 = V tile][64 rows x 128], rows swizzled in 16-byte chunks
     __shared__ __attribute__((aligned(1024))) T smem[2][2][kTile * kD];
-    // the tile list of this query block: first key row and validity word per tile
+    // the tile list of the current work item: first key row and validity word per tile
     __shared__ int32_t tile_row_sm[kListCap];
     __shared__ uint64_t tile_mask_sm[kListCap];
 
@@ -101,28 +110,9 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     const int wave = tid >> 6, lane = tid & 63;
     const int qh = wave & 1, kh = wave >> 1;
     const int lr = lane & 31, lh = lane >> 5;
-    const int bh = blockIdx.y;
-    const int64_t qrow0 = (int64_t)blockIdx.x * kTile;
     const int nbq = (int)(Sq / bs_q);
-    const int qblock = (int)(qrow0 / bs_q);
+    const int nqt = (int)(Sq / kTile);
     const int nsub = bs_k / kTile;
-    const int32_t* list = idx + ((int64_t)bh * nbq + qblock) * idx_stride;
-    const int ntiles = lens[(int64_t)bh * nbq + qblock] * nsub;
-
-    const char* kbase = reinterpret_cast<const char*>(k + (int64_t)bh * Sk * kD);
-    const char* vbase = reinterpret_cast<const char*>(v + (int64_t)bh * Sk * kD);
-
-    // Q as the B operand: lane holds row 32*qh + lr, d = 16*s + 8*lh .. +8
-    V8 qreg[8];
-    {
-        const T* qp = q + ((int64_t)bh * Sq + qrow0 + 32 * qh + lr) * kD + 8 * lh;
-#pragma unroll
-        for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const V8*>(qp + 16 * s);
-        // consume the loads here: otherwise their vmcnt waits land inside the tile loop,
-        // where they would also wait for the LDS loads of the next tile
-#pragma unroll
-        for (int s = 0; s < 8; ++s) asm volatile("" :: "v"(qreg[s]));
-    }
 
     // ---- global -> LDS: load i of this wavefront fills LDS rows 4*(4*i + wave) .. +4 ----
     // lane: physical row 16*i + 4*wave + lane/16, physical chunk lane%16,
@@ -134,16 +124,6 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) { koffs[i] = koff + i * 4096u; voffs[i] = voff + i * 4096u; }
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(&smem[0][0][0]) + wave * 1024);
-    auto issue_tile = [&](int row0, int st) {
-        const char* kt = kbase + (int64_t)row0 * (kD * 2);
-        const char* vt = vbase + (int64_t)row0 * (kD * 2);
-        const uint32_t kl = lds0 + st * (2 * kTileBytes);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            load_to_lds_16(kt, koffs[i], kl + i * 4096);
-            load_to_lds_16(vt, voffs[i], kl + kTileBytes + i * 4096);
-        }
-    };
 
     // ---- LDS read addresses (element offsets inside a tile) ----
     // K, A operand of S^T: row 32*kh + lr, logical chunk 2*c + lh
@@ -163,6 +143,35 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
         vaddr[t] = vkey0 * kD + ((chunk ^ vsw) << 3) + (s16 & 1) * 4;
     }
 
+    for (int item = item_begin + blockIdx.x; item < item_end; item += gridDim.x) {
+    const int bh = item / nqt;
+    const int64_t qrow0 = (int64_t)(item % nqt) * kTile;
+    const int qblock = (int)(qrow0 / bs_q);
+    const int32_t* list = idx + ((int64_t)bh * nbq + qblock) * idx_stride;
+    const int ntiles = lens[(int64_t)bh * nbq + qblock] * nsub;
+    const char* kbase = reinterpret_cast<const char*>(k + (int64_t)bh * Sk * kD);
+    const char* vbase = reinterpret_cast<const char*>(v + (int64_t)bh * Sk * kD);
+
+    // Q as the B operand: lane holds row 32*qh + lr, d = 16*s + 8*lh .. +8
+    V8 qreg[8];
+    {
+        const T* qp = q + ((int64_t)bh * Sq + qrow0 + 32 * qh + lr) * kD + 8 * lh;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const V8*>(qp + 16 * s);
+    }
+    auto issue_k = [&](int row0, int st) {
+        const char* kt = kbase + (int64_t)row0 * (kD * 2);
+        const uint32_t kl = lds0 + st * (2 * kTileBytes);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load_to_lds_16(kt, koffs[i], kl + i * 4096);
+    };
+    auto issue_v = [&](int row0, int st) {
+        const char* vt = vbase + (int64_t)row0 * (kD * 2);
+        const uint32_t vl = lds0 + st * (2 * kTileBytes) + kTileBytes;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load_to_lds_16(vt, voffs[i], vl + i * 4096);
+    };
+
     f32x16 oacc[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
@@ -172,48 +181,37 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
 
     for (int chunk0 = 0; chunk0 < ntiles; chunk0 += kListCap) {
     const int nloc = min(ntiles - chunk0, kListCap);
-    __syncthreads();                          // previous chunk fully consumed
+    __syncthreads();                          // previous chunk / previous item fully consumed
     for (int j = tid; j < nloc; j += 256) {
         const int it = chunk0 + j;
         const int64_t row0 = (int64_t)list[it / nsub] * bs_k + (int64_t)(it % nsub) * kTile;
         tile_row_sm[j] = (int)row0;
         tile_mask_sm[j] = tile_valid ? tile_valid[row0 / kTile] : ~0ull;
     }
+    // consume the Q loads here: otherwise their vmcnt waits land inside the tile loop,
+    // where they would also wait for the LDS loads of the next tile
+#pragma unroll
+    for (int s = 0; s < 8; ++s) asm volatile("" :: "v"(qreg[s]));
     __syncthreads();
-    issue_tile(__builtin_amdgcn_readfirstlane(tile_row_sm[0]), 0);
-    int row_next = nloc > 1 ? tile_row_sm[1] : 0;
 
-    // one tile; the stage is a compile-time constant so that every LDS address is a
-    // loop-invariant register plus an immediate offset
-    auto step = [&](int it, auto stage) {
-        constexpr int st = decltype(stage)::value;
-        const uint64_t vmask = tile_mask_sm[it];
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's share of tile `it` is in LDS
-        __syncthreads();                                     // ... and everybody else's; stage st^1 is free again
-        if (it + 1 < nloc) issue_tile(__builtin_amdgcn_readfirstlane(row_next), st ^ 1);
-        if (it + 2 < nloc) row_next = tile_row_sm[it + 2];
-        const T* ks = smem[st][0];
-        const T* vs = smem[st][1];
-
-        // S^T = K_half . Q^T
-        f32x16 s;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] = 0.f;
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            const V8 a = *reinterpret_cast<const V8*>(ks + kaddr[c]);
-            s = mfma32(a, qreg[c], s);
-        }
-        // accumulator i <-> key 32*kh + 8*(i/4) + 4*lh + i%4, query lr
+    // Padded keys of tile j get -inf (accumulator i <-> key 32*kh + 8*(i/4) + 4*lh + i%4, query lr).
+    auto mask_tile = [&](f32x16& s, int j) {
+        const uint64_t vmask = tile_mask_sm[j];
         if (vmask != ~0ull) {
             const uint32_t half = (uint32_t)(vmask >> (32 * kh));
 #pragma unroll
             for (int i = 0; i < 16; ++i)
                 if (!((half >> (8 * (i / 4) + 4 * lh + (i % 4))) & 1u)) s[i] = -INFINITY;
         }
-        float mx = s[0];
+    };
+    // Row maximum of a finished S^T tile; raises the running maximum (and rescales the
+    // accumulators) only when some row exceeds it by more than 2^kLazyTau.
+    auto update_max = [&](const f32x16& s) {
+        // a linear chain: the compiler folds pairs into v_max3_f32 (and inserts the wait states that
+        // reading fresh MFMA results requires, which hand-written assembly would not get)
+        float mx = fmaxf(s[0], s[1]);
 #pragma unroll
-        for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
+        for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
         {   // combine with the other key group of the same query (lane ^ 32)
             const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
             mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])) * qk_scale;
@@ -228,31 +226,97 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
 #pragma unroll
                 for (int i = 0; i < 16; ++i) oacc[t][i] *= alpha;
         }
-        const float m_safe = (m_i == -INFINITY) ? 0.f : m_i;
-        float psum = 0.f;
-        float p[16];
+    };
+    auto qk_plain = [&](auto stage) -> f32x16 {      // S^T from K stage st, nothing interleaved
+        constexpr int st = decltype(stage)::value;
+        const T* ks = smem[st][0];
+        f32x16 s;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            p[i] = __builtin_amdgcn_exp2f(fmaf(s[i], qk_scale, -m_safe));
-            psum += p[i];
+        for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) s = mfma32(*reinterpret_cast<const V8*>(ks + kaddr[c]), qreg[c], s);
+        return s;
+    };
+
+    // K(i) and V(i) live in stage i&1.  Iteration i, with S(i) finished and the running maximum
+    // already raised for it:
+    //   X: the 8 MFMAs of S(i+1), each followed by the exp2 of two probabilities of tile i;
+    //   Y: the 8 MFMAs of O += P(i) V(i), interleaved with the row sum of P(i);
+    //   then the maximum of S(i+1) (its rare rescale waits for Y by data dependence).
+    // At the top of iteration i the loads issued one iteration earlier (V(i), K(i+1)) are awaited,
+    // then V(i+1) and K(i+2) are issued.
+    issue_k(__builtin_amdgcn_readfirstlane(tile_row_sm[0]), 0);
+    issue_v(__builtin_amdgcn_readfirstlane(tile_row_sm[0]), 0);
+    if (nloc > 1) issue_k(__builtin_amdgcn_readfirstlane(tile_row_sm[1]), 1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    f32x16 s_cur = qk_plain(std::integral_constant<int, 0>{});
+    mask_tile(s_cur, 0);
+    update_max(s_cur);
+
+    auto step = [&](int it, auto stage) {
+        constexpr int st = decltype(stage)::value;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's share of V(it), K(it+1) is in LDS
+        __syncthreads();                                     // ... and everybody else's; K(it), V(it-1) are consumed
+        if (it + 1 < nloc) issue_v(__builtin_amdgcn_readfirstlane(tile_row_sm[it + 1]), st ^ 1);
+        if (it + 2 < nloc) issue_k(__builtin_amdgcn_readfirstlane(tile_row_sm[it + 2]), st);
+        const bool more = it + 1 < nloc;
+        const T* ks = smem[st ^ 1][0];
+        const T* vs = smem[st][1];
+        const float neg_m = (m_i == -INFINITY) ? 0.f : -m_i;
+        float p[16];
+        f32x16 s_next;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s_next[i] = 0.f;
+        // ---- X ----
+        if (more) {
+            V8 a = *reinterpret_cast<const V8*>(ks + kaddr[0]);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                V8 a_nxt = a;
+                if (c < 7) a_nxt = *reinterpret_cast<const V8*>(ks + kaddr[c + 1]);
+                s_next = mfma32(a, qreg[c], s_next);
+                p[2 * c] = __builtin_amdgcn_exp2f(fmaf(s_cur[2 * c], qk_scale, neg_m));
+                p[2 * c + 1] = __builtin_amdgcn_exp2f(fmaf(s_cur[2 * c + 1], qk_scale, neg_m));
+                a = a_nxt;
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) p[i] = __builtin_amdgcn_exp2f(fmaf(s_cur[i], qk_scale, neg_m));
         }
-        l_i += psum;
         // P^T as B operand: k-slot (lh, j) of step c <-> accumulator 8*c + j
         V8 pb[2];
 #pragma unroll
         for (int c = 0; c < 2; ++c)
 #pragma unroll
             for (int j = 0; j < 8; ++j) pb[c][j] = (T)p[8 * c + j];
-        // O^T += V^T . P^T
+        // ---- Y ----
+        float psum = 0.f;
+        {
+            s16x4 lo = lds_read_tr16(vs + vaddr[0]);
+            s16x4 hi = lds_read_tr16(vs + vaddr[0] + 8 * kD);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-#pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const s16x4 lo = lds_read_tr16(vs + vaddr[t] + (8 * (2 * c)) * kD);
-                const s16x4 hi = lds_read_tr16(vs + vaddr[t] + (8 * (2 * c + 1)) * kD);
+            for (int u = 0; u < 8; ++u) {        // u = 2*t + c
+                const int t = u >> 1, c = u & 1;
+                s16x4 lo_n = lo, hi_n = hi;
+                if (u < 7) {
+                    const int t2 = (u + 1) >> 1, c2 = (u + 1) & 1;
+                    lo_n = lds_read_tr16(vs + vaddr[t2] + (8 * (2 * c2)) * kD);
+                    hi_n = lds_read_tr16(vs + vaddr[t2] + (8 * (2 * c2 + 1)) * kD);
+                }
                 const s16x8 av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                 oacc[t] = mfma32(__builtin_bit_cast(V8, av), pb[c], oacc[t]);
+                psum += p[2 * u] + p[2 * u + 1];
+                lo = lo_n; hi = hi_n;
+                __builtin_amdgcn_sched_barrier(0);
             }
+        }
+        l_i += psum;
+        if (more) {
+            mask_tile(s_next, it + 1);
+            update_max(s_next);
+            s_cur = s_next;
         }
     };
     for (int it = 0; it < nloc; it += 2) {
@@ -314,6 +378,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
                 *reinterpret_cast<const uint4*>(ost + r * kD + kc * 8);
         }
     }
+    }   // work items
 }
 
 // ------------------------------------------------------------------ fp32
@@ -392,24 +457,53 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(
 
 }  // namespace
 
+// Workgroups the device runs at once with this kernel (2 per CU), cached per device.
+static int resident_workgroups() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 512;
+    if (cached[dev] == 0) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        cached[dev] = 2 * cus;
+    }
+    return cached[dev];
+}
+
 hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t* idx,
                       const int32_t* lens, const uint64_t* tile_valid, void* o, float* lse, int B,
                       int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride,
                       float sm_scale, int dtype, hipStream_t st) {
-    dim3 grid((unsigned)(Sq / kTile), (unsigned)(B * Hn)), block(256);
     const float qk_scale = sm_scale * kLog2e;
-    if (dtype == BSA_BF16)
-        hipLaunchKernelGGL((fwd_mfma_kernel<__bf16>), grid, block, 0, st, (const __bf16*)q,
-                           (const __bf16*)k, (const __bf16*)v, idx, lens, tile_valid, (__bf16*)o,
-                           lse, Sq, Sk, bs_q, bs_k, idx_stride, qk_scale);
-    else if (dtype == BSA_F16)
-        hipLaunchKernelGGL((fwd_mfma_kernel<_Float16>), grid, block, 0, st, (const _Float16*)q,
-                           (const _Float16*)k, (const _Float16*)v, idx, lens, tile_valid,
-                           (_Float16*)o, lse, Sq, Sk, bs_q, bs_k, idx_stride, qk_scale);
-    else
+    const dim3 block(256);
+    if (dtype == BSA_F32) {
+        const dim3 grid((unsigned)(Sq / kTile), (unsigned)(B * Hn));
         hipLaunchKernelGGL(fwd_f32_kernel, grid, block, 0, st, (const float*)q, (const float*)k,
                            (const float*)v, idx, lens, tile_valid, (float*)o, lse, Sq, Sk, bs_q,
                            bs_k, idx_stride, qk_scale);
+        return hipGetLastError();
+    }
+    // One launch per round of as many work items as the device runs at once: the workgroups of a
+    // launch start together and walk their (ascending) KV lists in step, so that a tile fetched
+    // by one of them is still in L2 when its neighbours ask for it.  Rounds do not straddle a
+    // (batch, head) boundary: all workgroups of a round share one head's K/V.
+    const int per_head = (int)(Sq / kTile);
+    const int round = resident_workgroups();
+    for (int bh = 0; bh < B * Hn; ++bh) {
+        for (int first = 0; first < per_head; first += round) {
+            const int begin = bh * per_head + first;
+            const int end = bh * per_head + (first + round < per_head ? first + round : per_head);
+            const dim3 grid((unsigned)(end - begin));
+            if (dtype == BSA_BF16)
+                hipLaunchKernelGGL((fwd_mfma_kernel<__bf16>), grid, block, 0, st, (const __bf16*)q,
+                                   (const __bf16*)k, (const __bf16*)v, idx, lens, tile_valid, (__bf16*)o,
+                                   lse, Sq, Sk, bs_q, bs_k, idx_stride, qk_scale, begin, end);
+            else
+                hipLaunchKernelGGL((fwd_mfma_kernel<_Float16>), grid, block, 0, st, (const _Float16*)q,
+                                   (const _Float16*)k, (const _Float16*)v, idx, lens, tile_valid,
+                                   (_Float16*)o, lse, Sq, Sk, bs_q, bs_k, idx_stride, qk_scale, begin, end);
+        }
+    }
     return hipGetLastError();
 }
 

@@ -120,6 +120,7 @@ constexpr int kMaxSel = 1024;   // keys kept in LDS per wavefront
 template <typename S, int NPL>
 __global__ __launch_bounds__(256) void topk_kernel(const S* __restrict__ score,
                                                    int32_t* __restrict__ idx_out,
+                                                   int32_t* __restrict__ idx_sorted_out,
                                                    int32_t* __restrict__ lens_out, int64_t rows,
                                                    int nbk, int k_sel) {
     typedef typename KeyOf<S>::type K;
@@ -162,22 +163,29 @@ __global__ __launch_bounds__(256) void topk_kernel(const S* __restrict__ score,
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): LDS writes of this wavefront landed
     __builtin_amdgcn_wave_barrier();
-    int32_t* out = idx_out + row * k_sel;
+    // idx_out: descending score, ties towards the lowest index (the order of the keys);
+    // idx_sorted_out: the same set in ascending block index
     for (int e = lane; e < k_sel; e += 64) {
         const K me = mine[e];
-        int rank = 0;
-        for (int o = 0; o < k_sel; ++o) rank += mine[o] > me;
-        out[rank] = KeyOf<S>::index(me);
+        const int my_idx = KeyOf<S>::index(me);
+        int rank = 0, rank_idx = 0;
+        for (int o = 0; o < k_sel; ++o) {
+            const K other = mine[o];
+            rank += other > me;
+            rank_idx += KeyOf<S>::index(other) < my_idx;
+        }
+        if (idx_out) idx_out[row * k_sel + rank] = my_idx;
+        if (idx_sorted_out) idx_sorted_out[row * k_sel + rank_idx] = my_idx;
     }
 }
 
 template <typename S>
-hipError_t launch_topk_t(const S* score, int32_t* idx, int32_t* lens, int64_t rows, int nbk,
-                         int k_sel, hipStream_t st) {
+hipError_t launch_topk_t(const S* score, int32_t* idx, int32_t* idx_sorted, int32_t* lens, int64_t rows,
+                         int nbk, int k_sel, hipStream_t st) {
     dim3 grid((unsigned)((rows + 3) / 4)), block(256);
 #define BSA_TOPK(N)                                                                          \
-    hipLaunchKernelGGL((topk_kernel<S, N>), grid, block, 0, st, score, idx, lens, rows, nbk, \
-                       k_sel)
+    hipLaunchKernelGGL((topk_kernel<S, N>), grid, block, 0, st, score, idx, idx_sorted, lens, rows, \
+                       nbk, k_sel)
     if (nbk <= 4 * 64) BSA_TOPK(4);
     else if (nbk <= 8 * 64) BSA_TOPK(8);
     else if (nbk <= 16 * 64) BSA_TOPK(16);
@@ -210,11 +218,11 @@ hipError_t launch_score(const void* q_cmp, const void* k_cmp, void* score, int B
     return hipGetLastError();
 }
 
-hipError_t launch_topk(const void* score, int32_t* idx, int32_t* lens, int64_t rows, int nbk,
-                       int k_sel, int dtype, hipStream_t st) {
+hipError_t launch_topk(const void* score, int32_t* idx, int32_t* idx_sorted, int32_t* lens, int64_t rows,
+                       int nbk, int k_sel, int dtype, hipStream_t st) {
     if (dtype == BSA_F32)
-        return launch_topk_t<uint32_t>((const uint32_t*)score, idx, lens, rows, nbk, k_sel, st);
-    return launch_topk_t<uint16_t>((const uint16_t*)score, idx, lens, rows, nbk, k_sel, st);
+        return launch_topk_t<uint32_t>((const uint32_t*)score, idx, idx_sorted, lens, rows, nbk, k_sel, st);
+    return launch_topk_t<uint16_t>((const uint16_t*)score, idx, idx_sorted, lens, rows, nbk, k_sel, st);
 }
 
 }  // namespace bsa

@@ -38,8 +38,8 @@ SIGNATURES = {
     "bsa_permute_thw_to_blocks": (_i, [_p, _strides, _p, _p, _p] + [_i] * 10 + [_p]),
     "bsa_unpermute_blocks_to_thw": (_i, [_p, _p, _strides] + [_i] * 10 + [_p]),
     "bsa_mean_pool": (_i, [_p, _p, _i, _i, _i64, _i, _i, _i, _p]),
-    "bsa_score_topk": (_i, [_p, _p, _p, _p, _p] + [_i] * 7 + [_p]),
-    "bsa_topk_from_score": (_i, [_p, _p, _p] + [_i] * 6 + [_p]),
+    "bsa_score_topk": (_i, [_p, _p, _p, _p, _p, _p] + [_i] * 7 + [_p]),
+    "bsa_topk_from_score": (_i, [_p, _p, _p, _p] + [_i] * 6 + [_p]),
     "bsa_fwd": (_i, [_p] * 8 + [_i, _i, _i64, _i64, _i, _i, _i, _i, _f, _i, _p]),
     "bsa_workspace_bytes": (C.c_size_t, [C.POINTER(Bsa3dParams)]),
     "bsa_fwd_3d": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,

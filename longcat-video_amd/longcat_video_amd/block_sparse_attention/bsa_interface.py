@@ -133,7 +133,8 @@ def mean_pooling_compression(x: torch.Tensor, block_size: int) -> torch.Tensor:
     return out
 
 
-def _score_topk(q_cmp, k_cmp, k_sel):
+def _score_topk(q_cmp, k_cmp, k_sel, order="score"):
+    """order: "score" = descending score (the reference's torch.topk order), "block" = ascending block index."""
     _need_gpu(q_cmp, k_cmp)
     B, H, nbq, D = q_cmp.shape
     nbk = k_cmp.shape[2]
@@ -145,7 +146,9 @@ def _score_topk(q_cmp, k_cmp, k_sel):
     lens = torch.empty(B, H, nbq, dtype=torch.int32, device=q_cmp.device)
     lib = _capi.load()
     with torch.cuda.device(q_cmp.device):
-        _capi.check(lib.bsa_score_topk(_ptr(q_cmp), _ptr(k_cmp), _ptr(buf), _ptr(lens), _ptr(score),
+        by_score = order == "score"
+        _capi.check(lib.bsa_score_topk(_ptr(q_cmp), _ptr(k_cmp), _ptr(buf) if by_score else None,
+                                       None if by_score else _ptr(buf), _ptr(lens), _ptr(score),
                                        B, H, nbq, nbk, D, k_sel, _code(q_cmp), _stream(q_cmp)), "score_topk")
     return idx, lens, score
 
@@ -167,7 +170,7 @@ def get_select_indices_topk_from_score(score: torch.Tensor, sparsity: float):
     lens = torch.empty(B, H, nbq, dtype=torch.int32, device=score.device)
     lib = _capi.load()
     with torch.cuda.device(score.device):
-        _capi.check(lib.bsa_topk_from_score(_ptr(score), _ptr(buf), _ptr(lens), B, H, nbq, nbk, k_sel,
+        _capi.check(lib.bsa_topk_from_score(_ptr(score), _ptr(buf), None, _ptr(lens), B, H, nbq, nbk, k_sel,
                                             _code(score), _stream(score)), "topk")
     return idx.long(), lens
 
@@ -229,7 +232,7 @@ def flash_attn_bsa(q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold,
         raise ValueError
     if cdf_threshold is not None:
         raise NotImplementedError("CDF-threshold selection is not built; pass cdf_threshold=None")
-    idx, lens, _ = _score_topk(q_cmp, k_cmp, num_selected(sparsity, k_cmp.shape[2]))
+    idx, lens, _ = _score_topk(q_cmp, k_cmp, num_selected(sparsity, k_cmp.shape[2]), order="block")
     o, _ = attn_fwd_bsa_varlen(q, k, v, sm_scale, idx, lens, chunk_size_q, chunk_size_k, sparsity, tile_valid)
     return o
 

@@ -70,12 +70,13 @@ def test_permute_rejects_bad_arguments():
 
 def test_topk_rejects_bad_arguments():
     lib = _capi.load()
-    assert lib.bsa_topk_from_score(FAKE, FAKE, FAKE, 1, 1, 4, 4, 5, _capi.BSA_BF16, None) == _capi.BSA_ERR_SHAPE
-    assert lib.bsa_topk_from_score(FAKE, FAKE, FAKE, 1, 1, 4, 5000, 5, _capi.BSA_BF16, None) == _capi.BSA_ERR_UNSUPPORTED
-    assert lib.bsa_topk_from_score(FAKE, FAKE, FAKE, 1, 1, 4, 4096, 2000, _capi.BSA_BF16, None) == _capi.BSA_ERR_UNSUPPORTED
-    assert lib.bsa_topk_from_score(None, FAKE, FAKE, 1, 1, 4, 4, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_BAD_ARG
-    assert lib.bsa_score_topk(FAKE, FAKE, FAKE, FAKE, FAKE, 1, 1, 4, 4, 100, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_UNSUPPORTED
-    assert lib.bsa_score_topk(FAKE, FAKE, FAKE, FAKE, None, 1, 1, 4, 4, 128, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_BAD_ARG
+    assert lib.bsa_topk_from_score(FAKE, FAKE, None, FAKE, 1, 1, 4, 4, 5, _capi.BSA_BF16, None) == _capi.BSA_ERR_SHAPE
+    assert lib.bsa_topk_from_score(FAKE, FAKE, None, FAKE, 1, 1, 4, 5000, 5, _capi.BSA_BF16, None) == _capi.BSA_ERR_UNSUPPORTED
+    assert lib.bsa_topk_from_score(FAKE, FAKE, None, FAKE, 1, 1, 4, 4096, 2000, _capi.BSA_BF16, None) == _capi.BSA_ERR_UNSUPPORTED
+    assert lib.bsa_topk_from_score(None, FAKE, None, FAKE, 1, 1, 4, 4, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_BAD_ARG
+    assert lib.bsa_score_topk(FAKE, FAKE, FAKE, None, FAKE, FAKE, 1, 1, 4, 4, 100, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_UNSUPPORTED
+    assert lib.bsa_score_topk(FAKE, FAKE, FAKE, None, FAKE, None, 1, 1, 4, 4, 128, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_BAD_ARG
+    assert lib.bsa_score_topk(FAKE, FAKE, None, None, FAKE, FAKE, 1, 1, 4, 4, 128, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_BAD_ARG
 
 
 def test_fwd_rejects_bad_arguments():
@@ -119,13 +120,13 @@ def test_fwd_3d_plan_and_workspace():
 
 def test_status_to_exception_mapping():
     lib = _capi.load()
-    rc = lib.bsa_topk_from_score(FAKE, FAKE, FAKE, 1, 1, 4, 4, 5, _capi.BSA_BF16, None)
+    rc = lib.bsa_topk_from_score(FAKE, FAKE, None, FAKE, 1, 1, 4, 4, 5, _capi.BSA_BF16, None)
     with pytest.raises(AssertionError):
         _capi.check(rc)
-    rc = lib.bsa_topk_from_score(None, FAKE, FAKE, 1, 1, 4, 4, 2, _capi.BSA_BF16, None)
+    rc = lib.bsa_topk_from_score(None, FAKE, None, FAKE, 1, 1, 4, 4, 2, _capi.BSA_BF16, None)
     with pytest.raises(ValueError):
         _capi.check(rc)
-    rc = lib.bsa_topk_from_score(FAKE, FAKE, FAKE, 1, 1, 4, 5000, 5, _capi.BSA_BF16, None)
+    rc = lib.bsa_topk_from_score(FAKE, FAKE, None, FAKE, 1, 1, 4, 5000, 5, _capi.BSA_BF16, None)
     with pytest.raises(NotImplementedError):
         _capi.check(rc)
     _capi.check(0)

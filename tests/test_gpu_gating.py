@@ -14,7 +14,7 @@ def I():
     return bsa_interface
 
 
-def topk_gpu(score, k_sel):
+def topk_gpu(score, k_sel, sorted_too=False):
     """Calls the C-ABI top-k directly with an explicit k_sel."""
     from longcat_video_amd import _capi
     B, H, nbq, nbk = score.shape
@@ -22,10 +22,15 @@ def topk_gpu(score, k_sel):
     idx = torch.full((B * H * nbq * max(k_sel, 1),), -7, dtype=torch.int32, device="cuda")
     lens = torch.empty(B, H, nbq, dtype=torch.int32, device="cuda")
     code = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}[score.dtype]
-    _capi.check(_capi.load().bsa_topk_from_score(s.data_ptr(), idx.data_ptr(), lens.data_ptr(), B, H, nbq, nbk,
-                                                  k_sel, code, torch.cuda.current_stream().cuda_stream))
+    srt = torch.full_like(idx, -7) if sorted_too else None
+    _capi.check(_capi.load().bsa_topk_from_score(s.data_ptr(), idx.data_ptr(), None if srt is None else srt.data_ptr(),
+                                                  lens.data_ptr(), B, H, nbq, nbk, k_sel, code,
+                                                  torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
-    return idx[: B * H * nbq * k_sel].view(B, H, nbq, k_sel).cpu().long(), lens.cpu()
+    out = idx[: B * H * nbq * k_sel].view(B, H, nbq, k_sel).cpu().long()
+    if sorted_too:
+        return out, lens.cpu(), srt[: B * H * nbq * k_sel].view(B, H, nbq, k_sel).cpu().long()
+    return out, lens.cpu()
 
 
 def test_score_exact_on_integer_inputs():
@@ -68,6 +73,16 @@ def test_topk_random_scores_all_dtypes(dtype):
     assert torch.equal(got, want)
     vals = torch.gather(score.float(), -1, got)
     assert torch.equal(vals, torch.topk(score.float(), 41).values)
+
+
+def test_block_ordered_list_is_the_same_set_in_ascending_order():
+    g = torch.Generator().manual_seed(8)
+    score = (torch.randint(-6, 7, (1, 2, 5, 700), generator=g).float() / 4).bfloat16()
+    got, _, srt = topk_gpu(score, 77, sorted_too=True)
+    assert torch.equal(torch.sort(got, dim=-1).values, srt)
+    idx_b, lens_b, _ = I()._score_topk(torch.randn(1, 2, 9, 128, generator=g).bfloat16().cuda(),
+                                       torch.randn(1, 2, 300, 128, generator=g).bfloat16().cuda(), 40, order="block")
+    assert torch.all(idx_b[..., 1:] > idx_b[..., :-1]) and torch.all(lens_b == 40)
 
 
 def test_topk_special_values():
