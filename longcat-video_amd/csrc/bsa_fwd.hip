@@ -120,9 +120,6 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     const int drow = 4 * wave + (lane >> 4);
     const uint32_t koff = (uint32_t)(drow * 256 + (((lane & 15) ^ (drow & 15)) << 4));
     const uint32_t voff = (uint32_t)(drow * 256 + (((lane & 15) ^ ((drow & 3) << 2)) << 4));
-    uint32_t koffs[4], voffs[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { koffs[i] = koff + i * 4096u; voffs[i] = voff + i * 4096u; }
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(&smem[0][0][0]) + wave * 1024);
 
     // ---- LDS read addresses (element offsets inside a tile) ----
@@ -163,13 +160,13 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
         const char* kt = kbase + (int64_t)row0 * (kD * 2);
         const uint32_t kl = lds0 + st * (2 * kTileBytes);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_to_lds_16(kt, koffs[i], kl + i * 4096);
+        for (int i = 0; i < 4; ++i) load_to_lds_16(kt + i * 4096, koff, kl + i * 4096);
     };
     auto issue_v = [&](int row0, int st) {
         const char* vt = vbase + (int64_t)row0 * (kD * 2);
         const uint32_t vl = lds0 + st * (2 * kTileBytes) + kTileBytes;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_to_lds_16(vt, voffs[i], vl + i * 4096);
+        for (int i = 0; i < 4; ++i) load_to_lds_16(vt + i * 4096, voff, vl + i * 4096);
     };
 
     f32x16 oacc[4];
@@ -195,8 +192,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     __syncthreads();
 
     // Padded keys of tile j get -inf (accumulator i <-> key 32*kh + 8*(i/4) + 4*lh + i%4, query lr).
-    auto mask_tile = [&](f32x16& s, int j) {
-        const uint64_t vmask = tile_mask_sm[j];
+    auto mask_tile = [&](f32x16& s, uint64_t vmask) {
         if (vmask != ~0ull) {
             const uint32_t half = (uint32_t)(vmask >> (32 * kh));
 #pragma unroll
@@ -204,18 +200,9 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
                 if (!((half >> (8 * (i / 4) + 4 * lh + (i % 4))) & 1u)) s[i] = -INFINITY;
         }
     };
-    // Row maximum of a finished S^T tile; raises the running maximum (and rescales the
-    // accumulators) only when some row exceeds it by more than 2^kLazyTau.
-    auto update_max = [&](const f32x16& s) {
-        // a linear chain: the compiler folds pairs into v_max3_f32 (and inserts the wait states that
-        // reading fresh MFMA results requires, which hand-written assembly would not get)
-        float mx = fmaxf(s[0], s[1]);
-#pragma unroll
-        for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
-        {   // combine with the other key group of the same query (lane ^ 32)
-            const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
-            mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])) * qk_scale;
-        }
+    // Raises the running maximum (and rescales the accumulators) only when some row's new maximum
+    // `mx` (already combined over the tile and scaled) exceeds it by more than 2^kLazyTau.
+    auto raise_max = [&](float mx) {
         if (__any(mx > m_i + kLazyTau)) {
             const float m_new = fmaxf(m_i, mx);
             const float alpha = __builtin_amdgcn_exp2f(m_i - ((m_new == -INFINITY) ? 0.f : m_new));
@@ -226,6 +213,17 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
 #pragma unroll
                 for (int i = 0; i < 16; ++i) oacc[t][i] *= alpha;
         }
+    };
+    // combine a lane's maximum with the other key group of the same query (lane ^ 32) and scale it
+    auto finish_max = [&](float mx) -> float {
+        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+        return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])) * qk_scale;
+    };
+    auto update_max = [&](const f32x16& s) {
+        float mx = fmaxf(s[0], s[1]);
+#pragma unroll
+        for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, s[i]), s[i + 1]);
+        raise_max(finish_max(mx));
     };
     auto qk_plain = [&](auto stage) -> f32x16 {      // S^T from K stage st, nothing interleaved
         constexpr int st = decltype(stage)::value;
@@ -250,78 +248,109 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     if (nloc > 1) issue_k(__builtin_amdgcn_readfirstlane(tile_row_sm[1]), 1);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    f32x16 s_cur = qk_plain(std::integral_constant<int, 0>{});
-    mask_tile(s_cur, 0);
-    update_max(s_cur);
+    // S^T of the current and of the next tile alternate between two register sets
+    f32x16 s_a = qk_plain(std::integral_constant<int, 0>{}), s_b;
+    mask_tile(s_a, tile_mask_sm[0]);
+    update_max(s_a);
+    int row_v = nloc > 1 ? __builtin_amdgcn_readfirstlane(tile_row_sm[1]) : 0;   // first key row of tile it+1
+    int row_pref = tile_row_sm[nloc > 2 ? 2 : 0];                                     // ... of tile it+2, read ahead
 
-    auto step = [&](int it, auto stage) {
+    // An LDS read takes about as long as four MFMAs, so every fragment is requested four MFMAs
+    // before the one that consumes it; sched_barrier pins that order.
+    // full_step: tile `it` is not the last one of the list.  S(it+1) runs on the MFMA unit while the
+    // VALU turns S(it) into P(it); then O += P(it) V(it).
+    auto full_step = [&](int it, auto stage, f32x16& s_cur, f32x16& s_next) {
         constexpr int st = decltype(stage)::value;
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's share of V(it), K(it+1) is in LDS
-        __syncthreads();                                     // ... and everybody else's; K(it), V(it-1) are consumed
-        if (it + 1 < nloc) issue_v(__builtin_amdgcn_readfirstlane(tile_row_sm[it + 1]), st ^ 1);
-        if (it + 2 < nloc) issue_k(__builtin_amdgcn_readfirstlane(tile_row_sm[it + 2]), st);
-        const bool more = it + 1 < nloc;
         const T* ks = smem[st ^ 1][0];
         const T* vs = smem[st][1];
+        auto read_v = [&](int u) -> V8 {             // u = 2*t + c
+            const int t = u >> 1, c = u & 1;
+            const s16x4 lo = lds_read_tr16(vs + vaddr[t] + (8 * (2 * c)) * kD);
+            const s16x4 hi = lds_read_tr16(vs + vaddr[t] + (8 * (2 * c + 1)) * kD);
+            return __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        };
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's share of V(it), K(it+1) is in LDS
+        __syncthreads();                                     // ... and everybody else's; K(it), V(it-1) are consumed
+        V8 kf[8], vf[8];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) kf[c] = *reinterpret_cast<const V8*>(ks + kaddr[c]);
+        const uint64_t mask_next = tile_mask_sm[it + 1];     // needed only after the 8 MFMAs below
+        __builtin_amdgcn_sched_barrier(0);
+        issue_v(row_v, st ^ 1);
+        row_v = __builtin_amdgcn_readfirstlane(row_pref);    // tile it+2: K now, V in the next step
+        if (it + 2 < nloc) issue_k(row_v, st);
         const float neg_m = (m_i == -INFINITY) ? 0.f : -m_i;
-        float p[16];
-        f32x16 s_next;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s_next[i] = 0.f;
-        // ---- X ----
-        if (more) {
-            V8 a = *reinterpret_cast<const V8*>(ks + kaddr[0]);
-#pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                V8 a_nxt = a;
-                if (c < 7) a_nxt = *reinterpret_cast<const V8*>(ks + kaddr[c + 1]);
-                s_next = mfma32(a, qreg[c], s_next);
-                p[2 * c] = __builtin_amdgcn_exp2f(fmaf(s_cur[2 * c], qk_scale, neg_m));
-                p[2 * c + 1] = __builtin_amdgcn_exp2f(fmaf(s_cur[2 * c + 1], qk_scale, neg_m));
-                a = a_nxt;
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) p[i] = __builtin_amdgcn_exp2f(fmaf(s_cur[i], qk_scale, neg_m));
-        }
-        // P^T as B operand: k-slot (lh, j) of step c <-> accumulator 8*c + j
-        V8 pb[2];
-#pragma unroll
-        for (int c = 0; c < 2; ++c)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) pb[c][j] = (T)p[8 * c + j];
-        // ---- Y ----
+        V8 pb[2];      // P^T as B operand: k-slot (lh, j) of step c <-> accumulator 8*c + j
         float psum = 0.f;
-        {
-            s16x4 lo = lds_read_tr16(vs + vaddr[0]);
-            s16x4 hi = lds_read_tr16(vs + vaddr[0] + 8 * kD);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {        // u = 2*t + c
-                const int t = u >> 1, c = u & 1;
-                s16x4 lo_n = lo, hi_n = hi;
-                if (u < 7) {
-                    const int t2 = (u + 1) >> 1, c2 = (u + 1) & 1;
-                    lo_n = lds_read_tr16(vs + vaddr[t2] + (8 * (2 * c2)) * kD);
-                    hi_n = lds_read_tr16(vs + vaddr[t2] + (8 * (2 * c2 + 1)) * kD);
-                }
-                const s16x8 av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                oacc[t] = mfma32(__builtin_bit_cast(V8, av), pb[c], oacc[t]);
-                psum += p[2 * u] + p[2 * u + 1];
-                lo = lo_n; hi = hi_n;
-                __builtin_amdgcn_sched_barrier(0);
+        for (int c = 0; c < 8; ++c) {
+            if (c + 4 < 8) kf[c + 4] = *reinterpret_cast<const V8*>(ks + kaddr[c + 4]);
+            else vf[c - 4] = read_v(c - 4);
+            if (c == 0) {
+                f32x16 zero;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) zero[i] = 0.f;
+                s_next = mfma32(kf[0], qreg[0], zero);
+            } else {
+                s_next = mfma32(kf[c], qreg[c], s_next);
             }
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(s_cur[2 * c], qk_scale, neg_m));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(s_cur[2 * c + 1], qk_scale, neg_m));
+            psum += p0 + p1;
+            pb[c >> 2][(2 * c) & 7] = (T)p0;
+            pb[c >> 2][(2 * c + 1) & 7] = (T)p1;
+            __builtin_amdgcn_sched_barrier(0);
         }
         l_i += psum;
-        if (more) {
-            mask_tile(s_next, it + 1);
-            update_max(s_next);
-            s_cur = s_next;
+        mask_tile(s_next, mask_next);
+        row_pref = tile_row_sm[it + 3 < nloc ? it + 3 : 0];  // consumed at the top of the next step
+        // O += P(it) V(it); the row maximum of S(it+1) fills the VALU slots between the MFMAs
+        float mx = fmaxf(s_next[0], s_next[1]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {        // u = 2*t + c
+            if (u + 4 < 8) vf[u + 4] = read_v(u + 4);
+            oacc[u >> 1] = mfma32(vf[u], pb[u & 1], oacc[u >> 1]);
+            if (u < 7) mx = fmaxf(fmaxf(mx, s_next[2 * u + 2]), s_next[2 * u + 3]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        raise_max(finish_max(mx));
+    };
+    // last_step: the final tile of the list, nothing left to prefetch or to overlap with.
+    auto last_step = [&](int it, auto stage, f32x16& s_cur) {
+        constexpr int st = decltype(stage)::value;
+        const T* vs = smem[st][1];
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const float neg_m = (m_i == -INFINITY) ? 0.f : -m_i;
+        V8 pb[2];
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float p = __builtin_amdgcn_exp2f(fmaf(s_cur[i], qk_scale, neg_m));
+            psum += p;
+            pb[i >> 3][i & 7] = (T)p;
+        }
+        l_i += psum;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int t = u >> 1, c = u & 1;
+            const s16x4 lo = lds_read_tr16(vs + vaddr[t] + (8 * (2 * c)) * kD);
+            const s16x4 hi = lds_read_tr16(vs + vaddr[t] + (8 * (2 * c + 1)) * kD);
+            const s16x8 av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            oacc[t] = mfma32(__builtin_bit_cast(V8, av), pb[c], oacc[t]);
         }
     };
-    for (int it = 0; it < nloc; it += 2) {
-        step(it, std::integral_constant<int, 0>{});
-        if (it + 1 < nloc) step(it + 1, std::integral_constant<int, 1>{});
+    int it = 0;
+    for (; it + 2 < nloc; it += 2) {
+        full_step(it, std::integral_constant<int, 0>{}, s_a, s_b);
+        full_step(it + 1, std::integral_constant<int, 1>{}, s_b, s_a);
+    }
+    if (nloc - it == 2) {
+        full_step(it, std::integral_constant<int, 0>{}, s_a, s_b);
+        last_step(it + 1, std::integral_constant<int, 1>{}, s_b);
+    } else {
+        last_step(it, std::integral_constant<int, 0>{}, s_a);
     }
     }
     __syncthreads();
