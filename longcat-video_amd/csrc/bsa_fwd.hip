@@ -300,6 +300,9 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
             psum += p0 + p1;
             pb[c >> 2][(2 * c) & 7] = (T)p0;
             pb[c >> 2][(2 * c + 1) & 7] = (T)p1;
+            // keep this VALU work here, between the MFMAs: without a use in this block the compiler
+            // sinks it below the branch that follows the loop
+            asm volatile("" : "+v"(psum), "+v"(pb[c >> 2]));
             __builtin_amdgcn_sched_barrier(0);
         }
         l_i += psum;
