@@ -33,9 +33,10 @@ WORKLOADS = {
     "c2": ((24, 30, 52), 0.9375, 1, False, "480p layer: 32 heads x 128, grid 24x30x52 (37440 tokens), density 1/16"),
     "c3": ((24, 45, 80), 0.9375, 2, True, "720p layer: 32 heads x 128, grid 24x45x80 (86400 tokens), density 1/16"),
 }
-# HBM-side bytes per launch of the attention kernel, from rocprofv3 --pmc FETCH_SIZE (x2) and
-# WRITE_SIZE (x1) as recorded in profiles/bsa_operator_c3_720p.md; re-measure after kernel changes.
-ATTENTION_TRAFFIC_BYTES = {"c3": 124999.7e6 + 762.8e6}
+# Bytes that leave L2 per layer in the attention kernel (all of its launches), from rocprofv3 --pmc
+# FETCH_SIZE (x2) and WRITE_SIZE (x1) as recorded in profiles/bsa_operator_c3_720p.md: 96 launches
+# x (764.7 MB + 7.9 MB).  Re-measure after kernel changes.
+ATTENTION_TRAFFIC_BYTES = {"c3": 96 * (764.7e6 + 7.9e6)}
 CHUNK = (4, 4, 4)
 HEADS, D = 32, 128
 
