@@ -193,7 +193,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
 
     // Padded keys of tile j get -inf (accumulator i <-> key 32*kh + 8*(i/4) + 4*lh + i%4, query lr).
     auto mask_tile = [&](f32x16& s, uint64_t vmask) {
-        if (vmask != ~0ull) {
+        if (__builtin_expect(vmask != ~0ull, 0)) {
             const uint32_t half = (uint32_t)(vmask >> (32 * kh));
 #pragma unroll
             for (int i = 0; i < 16; ++i)
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     // Raises the running maximum (and rescales the accumulators) only when some row's new maximum
     // `mx` (already combined over the tile and scaled) exceeds it by more than 2^kLazyTau.
     auto raise_max = [&](float mx) {
-        if (__any(mx > m_i + kLazyTau)) {
+        if (__builtin_expect(__any(mx > m_i + kLazyTau), 0)) {
             const float m_new = fmaxf(m_i, mx);
             const float alpha = __builtin_amdgcn_exp2f(m_i - ((m_new == -INFINITY) ? 0.f : m_new));
             m_i = m_new;
