@@ -171,8 +171,8 @@ int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, con
     if (Sq % bs_q != 0 || Sk % bs_k != 0)
         return set_error(BSA_ERR_SHAPE, "fwd: Sq=%lld / Sk=%lld are not multiples of the chunk sizes %d / %d", (long long)Sq, (long long)Sk, bs_q, bs_k);
     if (!(sm_scale > 0.f) || !std::isfinite(sm_scale)) return set_error(BSA_ERR_BAD_ARG, "fwd: sm_scale must be positive and finite");
-    if ((Sq / 64) * (int64_t)B * Hn > 0x7fffffffLL || Sk > 0x7fffffffLL)
-        return set_error(BSA_ERR_UNSUPPORTED, "fwd: problem too large for 32-bit work item / key row indices");
+    if ((Sq / 64) * (int64_t)B * Hn > 0x7fffffffLL || Sk > 0x7fffffffLL || (dtype != BSA_F32 && Sk >= (1 << 24)))
+        return set_error(BSA_ERR_UNSUPPORTED, "fwd: problem too large (32-bit work item indices, 24-bit key rows for the 16-bit types)");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
         return set_error(BSA_ERR_BAD_ARG, "fwd: q/k/v/o must be 16-byte aligned");
     const hipError_t e = launch_fwd(q, k, v, idx, lens, tile_valid, o, lse, B, Hn, Sq, Sk, bs_q, bs_k, idx_stride,
@@ -186,7 +186,8 @@ struct Plan {
     Grid3 gq, gk;
     int64_t Sqp, Skp;
     int nbq, nbk, es;
-    size_t off_qp, off_kp, off_vp, off_op, off_qc, off_kc, off_score, off_idx, off_idx_sorted, off_lens, off_valid, total;
+    bool direct_qo, direct_kv;
+    size_t off_qp, off_kp, off_vp, off_op, off_qc, off_kc, off_score, off_idx, off_idx_sorted, off_lens, off_valid, off_qrows, off_ktiles, total;
 };
 inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
@@ -210,10 +211,16 @@ int make_plan(const bsa_3d_params* p, Plan* pl) {
     const size_t bh = (size_t)p->B * p->Hn;
     size_t off = 0;
     auto take = [&](size_t bytes) { const size_t o = off; off += up256(bytes); return o; };
-    pl->off_qp = take(bh * pl->Sqp * p->D * pl->es);
-    pl->off_kp = take(bh * pl->Skp * p->D * pl->es);
-    pl->off_vp = take(bh * pl->Skp * p->D * pl->es);
-    pl->off_op = take(bh * pl->Sqp * p->D * pl->es);
+    // The MFMA kernel reads q and writes o in THW order itself, and gathers k and v tiles from THW
+    // order when the kv grid allows it; blocked copies are only made for the fp32 kernel and for
+    // kv grids that do not qualify.
+    pl->direct_qo = p->dtype != BSA_F32;
+    pl->direct_kv = pl->direct_qo && kv_direct_ok(pl->gk, (int64_t)p->D * pl->es);
+    pl->off_qp = take(pl->direct_qo ? 0 : bh * pl->Sqp * p->D * pl->es);
+    const size_t kv_rows = pl->direct_kv ? (size_t)edge_count(pl->gk) * pl->gk.chunk() : (size_t)pl->Skp;
+    pl->off_kp = take(bh * kv_rows * p->D * pl->es);
+    pl->off_vp = take(bh * kv_rows * p->D * pl->es);
+    pl->off_op = take(pl->direct_qo ? 0 : bh * pl->Sqp * p->D * pl->es);
     pl->off_qc = take(bh * pl->nbq * p->D * pl->es);
     pl->off_kc = take(bh * pl->nbk * p->D * pl->es);
     pl->off_score = take(bh * pl->nbq * (size_t)pl->nbk * pl->es);
@@ -221,6 +228,8 @@ int make_plan(const bsa_3d_params* p, Plan* pl) {
     pl->off_idx_sorted = take(bh * pl->nbq * (size_t)(p->k_sel > 0 ? p->k_sel : 1) * sizeof(int32_t));
     pl->off_lens = take(bh * pl->nbq * sizeof(int32_t));
     pl->off_valid = take((size_t)(pl->Skp / 64) * sizeof(uint64_t));
+    pl->off_qrows = take(pl->direct_qo ? (size_t)pl->Sqp * sizeof(int32_t) : 0);
+    pl->off_ktiles = take(pl->direct_kv ? (size_t)(pl->Skp / 64) * sizeof(uint32_t) : 0);
     pl->total = off;
     return BSA_OK;
 }
@@ -260,16 +269,44 @@ int bsa_fwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3]
     hipStream_t st = (hipStream_t)stream;
     hipError_t e;
 #define BSA_HIP(call, what) do { e = (call); if (e != hipSuccess) return hip_fail(e, what); } while (0)
-    BSA_HIP(launch_permute(q, q_strides, qp, qc, nullptr, p->B, p->Hn, pl.gq, p->D, p->dtype, st), "permute q");
-    BSA_HIP(launch_permute(k, k_strides, kp, kc, padded_k ? valid : nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st), "permute k");
-    BSA_HIP(launch_permute(v, v_strides, vp, nullptr, nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st), "permute v");
+    int32_t* qrows = pl.direct_qo ? reinterpret_cast<int32_t*>(ws + pl.off_qrows) : nullptr;
+    uint32_t* ktiles = pl.direct_kv ? reinterpret_cast<uint32_t*>(ws + pl.off_ktiles) : nullptr;
+    BSA_HIP(launch_permute(q, q_strides, pl.direct_qo ? nullptr : qp, qc, nullptr, p->B, p->Hn, pl.gq, p->D, p->dtype, st, false, qrows, nullptr), "permute q");
+    if (pl.direct_kv && (k_strides[2] != v_strides[2] || !kv_direct_ok(pl.gk, k_strides[2] * pl.es)))
+        return set_error(BSA_ERR_UNSUPPORTED, "fwd_3d: k and v must share one token stride (got %lld and %lld elements) "
+                         "small enough for 32-bit offsets inside a tile; pass contiguous copies",
+                         (long long)k_strides[2], (long long)v_strides[2]);
+    BSA_HIP(launch_permute(k, k_strides, kp, kc, padded_k ? valid : nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st, pl.direct_kv, nullptr, ktiles), "permute k");
+    if (!pl.direct_kv || padded_k)
+        BSA_HIP(launch_permute(v, v_strides, vp, nullptr, nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st, pl.direct_kv), "permute v");
     BSA_HIP(launch_score(qc, kc, score, p->B * p->Hn, pl.nbq, pl.nbk, p->D, p->dtype, st), "score");
     // the attention kernel walks each list in ascending block order (L2 locality); the score
     // order is only produced when the caller asks for the selection
     BSA_HIP(launch_topk(score, idx_out ? idx : nullptr, idx_sorted, lens, (int64_t)p->B * p->Hn * pl.nbq, pl.nbk, p->k_sel, p->dtype, st), "top-k");
-    BSA_HIP(launch_fwd(qp, kp, vp, idx_sorted, lens, padded_k ? valid : nullptr, op, nullptr, p->B, p->Hn, pl.Sqp, pl.Skp,
-                       pl.gq.chunk(), pl.gk.chunk(), p->k_sel, p->sm_scale, p->dtype, st), "attention");
-    BSA_HIP(launch_unpermute(op, o, o_strides, p->B, p->Hn, pl.gq, p->D, p->dtype, st), "unpermute");
+    if (pl.direct_qo) {
+        FwdLayout L;
+        L.q_rows = qrows;
+        L.k_tiles = ktiles;
+        L.k_edge = kp;
+        L.v_edge = vp;
+        for (int i = 0; i < 3; ++i) { L.q_st[i] = q_strides[i]; L.o_st[i] = o_strides[i]; }
+        if (pl.direct_kv) {
+            for (int i = 0; i < 3; ++i) { L.k_st[i] = k_strides[i]; L.v_st[i] = v_strides[i]; }
+            L.kw = pl.gk.w; L.kh = pl.gk.h; L.kH = pl.gk.H; L.kW = pl.gk.W;
+        } else {
+            L.k_st[0] = L.v_st[0] = (int64_t)p->Hn * pl.Skp * p->D;
+            L.k_st[1] = L.v_st[1] = pl.Skp * p->D;
+            L.k_st[2] = L.v_st[2] = p->D;
+            L.kw = 4; L.kh = 16; L.kH = 16; L.kW = 4;
+        }
+        BSA_HIP(launch_fwd(q, pl.direct_kv ? k : kp, pl.direct_kv ? v : vp, idx_sorted, lens, padded_k ? valid : nullptr, o, nullptr,
+                           p->B, p->Hn, pl.Sqp, pl.Skp, pl.gq.chunk(), pl.gk.chunk(), p->k_sel, p->sm_scale, p->dtype, st, &L,
+                           (int64_t)p->Tq * p->Hq * p->Wq, (int64_t)edge_count(pl.gk) * pl.gk.chunk() * p->D * pl.es), "attention");
+    } else {
+        BSA_HIP(launch_fwd(qp, kp, vp, idx_sorted, lens, padded_k ? valid : nullptr, op, nullptr, p->B, p->Hn, pl.Sqp, pl.Skp,
+                           pl.gq.chunk(), pl.gk.chunk(), p->k_sel, p->sm_scale, p->dtype, st), "attention");
+        BSA_HIP(launch_unpermute(op, o, o_strides, p->B, p->Hn, pl.gq, p->D, p->dtype, st), "unpermute");
+    }
     const size_t bh = (size_t)p->B * p->Hn;
     if (idx_out && p->k_sel > 0)
         BSA_HIP(hipMemcpyAsync(idx_out, idx, bh * pl.nbq * p->k_sel * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy idx");

@@ -23,6 +23,64 @@ inline Grid3 make_grid(int T, int H, int W, int t, int h, int w) {
     return g;
 }
 
+// Where the rows of the attention operands live.  Blocked order: tile i of a (batch, head) is rows
+// 64*i .. 64*i+63 of a contiguous [B, Hn, S, D] tensor.  THW order: tile i is (a 64-slot part of)
+// chunk i of the grid and its slots are gathered from / scattered to token positions, so the
+// separate permute and unpermute passes over that tensor disappear.  Strides are in elements:
+// batch, head, token.
+struct FwdLayout {
+    // token row of every blocked-order query slot, -1 for padding ([Sq]); null: q and o are in
+    // blocked order themselves
+    const int32_t* q_rows;
+    // per 64-slot kv tile: token row of its first slot (< 2^24) when the tile is read where it
+    // lies, or 2^24 + index of the tile in the edge copies ([Sk / 64]); null: k and v are in
+    // blocked order themselves
+    const uint32_t* k_tiles;
+    int64_t q_st[3], o_st[3], k_st[3], v_st[3];   // k_st[2] == v_st[2]
+    // blocked-order, zero-padded copies of the chunks that touch the padded high edge of the kv
+    // grid, [B*Hn][edge_count][chunk][D]; every other chunk is read where it lies
+    const void* k_edge;
+    const void* v_edge;
+    int kw, kh, kH, kW;        // kv tile geometry: runs of kw slots, kh runs per plane, grid H and W
+};
+
+// Chunks with padded slots ("edge chunks") are numbered densely: first the whole last t layer if
+// T is ragged, then the last h row of the remaining layers if H is ragged, then the last w column
+// of what is left if W is ragged.  Returns -1 for a chunk without padding.
+__host__ __device__ inline int edge_index(const Grid3& g, int blk) {
+    const int nw = blk % g.Nw, nh = (blk / g.Nw) % g.Nh, nt = blk / (g.Nw * g.Nh);
+    const bool rt = g.T % g.t != 0, rh = g.H % g.h != 0, rw = g.W % g.w != 0;
+    const int Nt1 = g.Nt - (rt ? 1 : 0), Nh1 = g.Nh - (rh ? 1 : 0);
+    int base = 0;
+    if (rt) {
+        if (nt == g.Nt - 1) return nh * g.Nw + nw;
+        base += g.Nh * g.Nw;
+    }
+    if (rh) {
+        if (nh == g.Nh - 1) return base + nt * g.Nw + nw;
+        base += Nt1 * g.Nw;
+    }
+    if (rw && nw == g.Nw - 1) return base + nt * Nh1 + nh;
+    return -1;
+}
+inline int edge_count(const Grid3& g) {
+    const bool rt = g.T % g.t != 0, rh = g.H % g.h != 0, rw = g.W % g.w != 0;
+    const int Nt1 = g.Nt - (rt ? 1 : 0), Nh1 = g.Nh - (rh ? 1 : 0);
+    return (rt ? g.Nh * g.Nw : 0) + (rh ? Nt1 * g.Nw : 0) + (rw ? Nt1 * Nh1 : 0);
+}
+
+// k and v tiles can be gathered from THW order when a 64-slot tile is a whole number of (h, w)
+// planes of its chunk, built from runs of at least 4 tokens along w, and when all offsets inside
+// a tile fit 32 bits.
+inline bool kv_direct_ok(const Grid3& g, int64_t token_stride_bytes) {
+    auto pow2 = [](int x) { return x > 0 && (x & (x - 1)) == 0; };
+    if (!pow2(g.w) || !pow2(g.h) || g.w < 4 || g.w > 64) return false;
+    if ((64 / g.w) % g.h != 0) return false;
+    if ((int64_t)g.T * g.H * g.W >= (1 << 24)) return false;
+    const int64_t planes = 64 / (g.w * g.h);
+    return token_stride_bytes > 0 && planes * g.H * g.W * token_stride_bytes < ((int64_t)1 << 32);
+}
+
 inline int dtype_size(int dtype) {
     switch (dtype) {
         case BSA_BF16: case BSA_F16: return 2;
@@ -36,9 +94,13 @@ int set_error(int code, const char* fmt, ...);
 
 // Kernel launchers (one per source file); all validate nothing and assume the
 // C-ABI layer has checked shapes.  Each returns a hipError_t from the launch.
+// edge_only: dst is [B*Hn][edge_count(g)][chunk][D] and only chunks with padded slots are copied
+// row_table ([S_padded] int32): token row of every blocked-order slot, -1 for padding.
+// tile_table ([S_padded/64] uint32): FwdLayout::k_tiles.  Both optional.
 hipError_t launch_permute(const void* src, const int64_t strides[3], void* dst, void* pooled,
                           uint64_t* tile_valid, int B, int Hn, const Grid3& g, int D, int dtype,
-                          hipStream_t st);
+                          hipStream_t st, bool edge_only = false, int32_t* row_table = nullptr,
+                          uint32_t* tile_table = nullptr);
 hipError_t launch_unpermute(const void* src, void* dst, const int64_t strides[3], int B, int Hn,
                             const Grid3& g, int D, int dtype, hipStream_t st);
 hipError_t launch_mean_pool(const void* x, void* out, int B, int Hn, int64_t S, int block, int D,
@@ -51,6 +113,7 @@ hipError_t launch_topk(const void* score, int32_t* idx, int32_t* idx_sorted, int
 hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t* idx,
                       const int32_t* lens, const uint64_t* tile_valid, void* o, float* lse,
                       int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride,
-                      float sm_scale, int dtype, hipStream_t st);
+                      float sm_scale, int dtype, hipStream_t st, const FwdLayout* layout = nullptr,
+                      int64_t layout_lse_rows = 0, int64_t layout_edge_bytes = 0);
 
 }  // namespace bsa

@@ -98,7 +98,8 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
     const int32_t* __restrict__ idx, const int32_t* __restrict__ lens,
     const uint64_t* __restrict__ tile_valid, T* __restrict__ o, float* __restrict__ lse,
-    int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride, float qk_scale, int item_begin, int item_end) {
+    int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride, float qk_scale, int item_begin, int item_end,
+    int Hn, int64_t lse_S, int64_t edge_bh_bytes, FwdLayout L) {
     typedef typename Vec8<T>::type V8;
     // [stage][0 = K tile | 1 = V tile][64 rows x 128], rows swizzled in 16-byte chunks
     __shared__ __attribute__((aligned(1024))) T smem[2][2][kTile * kD];
@@ -117,10 +118,22 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     // ---- global -> LDS: load i of this wavefront fills LDS rows 4*(4*i + wave) .. +4 ----
     // lane: physical row 16*i + 4*wave + lane/16, physical chunk lane%16,
     // fetches logical chunk (lane%16) ^ f(row);  f_K(row) = row & 15, f_V(row) = (row & 3) << 2
+    // The four rows of such a load are a run of 4 consecutive slots of the tile, which are 4
+    // consecutive tokens along w in THW order as well: the lane part of the address (row in the
+    // run, chunk in the row) is the same for every load and the position of the run goes into the
+    // scalar base.  In blocked order the runs simply follow each other.
     const int drow = 4 * wave + (lane >> 4);
-    const uint32_t koff = (uint32_t)(drow * 256 + (((lane & 15) ^ (drow & 15)) << 4));
-    const uint32_t voff = (uint32_t)(drow * 256 + (((lane & 15) ^ ((drow & 3) << 2)) << 4));
+    const uint32_t kv_sb = (uint32_t)(L.k_st[2] * (int64_t)sizeof(T));        // token stride in bytes
+    const uint32_t koff = (uint32_t)(lane >> 4) * kv_sb + (uint32_t)(((lane & 15) ^ (drow & 15)) << 4);
+    const uint32_t voff = (uint32_t)(lane >> 4) * kv_sb + (uint32_t)(((lane & 15) ^ ((drow & 3) << 2)) << 4);
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(&smem[0][0][0]) + wave * 1024);
+    uint32_t run_off[4];     // load i of this wavefront fetches run 4*i + wave of the tile
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int slot = 16 * i + 4 * wave;
+        const uint32_t rows = (uint32_t)(((slot / (L.kw * L.kh)) * L.kH + (slot / L.kw) % L.kh) * L.kW + slot % L.kw);
+        run_off[i] = __builtin_amdgcn_readfirstlane(rows * kv_sb);
+    }
 
     // ---- LDS read addresses (element offsets inside a tile) ----
     // K, A operand of S^T: row 32*kh + lr, logical chunk 2*c + lh
@@ -142,31 +155,50 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
 
     for (int item = item_begin + blockIdx.x; item < item_end; item += gridDim.x) {
     const int bh = item / nqt;
-    const int64_t qrow0 = (int64_t)(item % nqt) * kTile;
+    const int qtile = item % nqt;
+    const int64_t qrow0 = (int64_t)qtile * kTile;
     const int qblock = (int)(qrow0 / bs_q);
+    const int64_t q_bh = (int64_t)(bh / Hn) * L.q_st[0] + (int64_t)(bh % Hn) * L.q_st[1];
+    const int64_t o_bh = (int64_t)(bh / Hn) * L.o_st[0] + (int64_t)(bh % Hn) * L.o_st[1];
     const int32_t* list = idx + ((int64_t)bh * nbq + qblock) * idx_stride;
     const int ntiles = lens[(int64_t)bh * nbq + qblock] * nsub;
-    const char* kbase = reinterpret_cast<const char*>(k + (int64_t)bh * Sk * kD);
-    const char* vbase = reinterpret_cast<const char*>(v + (int64_t)bh * Sk * kD);
+    const char* kbase = reinterpret_cast<const char*>(k + (int64_t)(bh / Hn) * L.k_st[0] + (int64_t)(bh % Hn) * L.k_st[1]);
+    const char* vbase = reinterpret_cast<const char*>(v + (int64_t)(bh / Hn) * L.v_st[0] + (int64_t)(bh % Hn) * L.v_st[1]);
 
     // Q as the B operand: lane holds row 32*qh + lr, d = 16*s + 8*lh .. +8
     V8 qreg[8];
     {
-        const T* qp = q + ((int64_t)bh * Sq + qrow0 + 32 * qh + lr) * kD + 8 * lh;
+        // padded query slots read token 0 (always there); their rows are never stored
+        int64_t row = qrow0 + 32 * qh + lr;
+        if (L.q_rows != nullptr) row = max(L.q_rows[row], 0);
+        const T* qp = q + q_bh + row * L.q_st[2] + 8 * lh;
 #pragma unroll
         for (int s = 0; s < 8; ++s) qreg[s] = *reinterpret_cast<const V8*>(qp + 16 * s);
     }
-    auto issue_k = [&](int row0, int st) {
-        const char* kt = kbase + (int64_t)row0 * (kD * 2);
-        const uint32_t kl = lds0 + st * (2 * kTileBytes);
+    // `entry` < 2^24: first token row of the tile, fetched run by run from where it lies.
+    // Otherwise: 2^24 + index of a 64-slot tile in the blocked-order copies of the edge chunks.
+    auto issue_tile = [&](const char* base, const char* edge, uint32_t entry, uint32_t lds, uint32_t off, int vswz) {
+        if (__builtin_expect(entry < (1u << 24), 1)) {
+            const char* tile = base + (uint64_t)entry * kv_sb;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_to_lds_16(kt + i * 4096, koff, kl + i * 4096);
+            for (int i = 0; i < 4; ++i) load_to_lds_16(tile + run_off[i], off, lds + i * 4096);
+        } else {
+            // rare: the lane part for 256-byte rows is rebuilt from the thread index, which costs
+            // nothing while the common path runs
+            int t2 = tid;
+            asm volatile("" : "+v"(t2));
+            const int l2 = t2 & 63, d2 = 4 * (t2 >> 6) + (l2 >> 4);
+            const uint32_t off2 = (uint32_t)(d2 * 256 + (((l2 & 15) ^ (vswz ? (d2 & 3) << 2 : d2 & 15)) << 4));
+            const char* tile = edge + (uint64_t)(entry & 0xffffffu) * kTileBytes;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) load_to_lds_16(tile + i * 4096, off2, lds + i * 4096);
+        }
     };
-    auto issue_v = [&](int row0, int st) {
-        const char* vt = vbase + (int64_t)row0 * (kD * 2);
-        const uint32_t vl = lds0 + st * (2 * kTileBytes) + kTileBytes;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) load_to_lds_16(vt + i * 4096, voff, vl + i * 4096);
+    const char* kedge = reinterpret_cast<const char*>(L.k_edge) + (int64_t)bh * edge_bh_bytes;
+    const char* vedge = reinterpret_cast<const char*>(L.v_edge) + (int64_t)bh * edge_bh_bytes;
+    auto issue_k = [&](uint32_t entry, int st) { issue_tile(kbase, kedge, entry, lds0 + st * (2 * kTileBytes), koff, 0); };
+    auto issue_v = [&](uint32_t entry, int st) {
+        issue_tile(vbase, vedge, entry, lds0 + st * (2 * kTileBytes) + kTileBytes, voff, 1);
     };
 
     f32x16 oacc[4];
@@ -181,9 +213,10 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     __syncthreads();                          // previous chunk / previous item fully consumed
     for (int j = tid; j < nloc; j += 256) {
         const int it = chunk0 + j;
-        const int64_t row0 = (int64_t)list[it / nsub] * bs_k + (int64_t)(it % nsub) * kTile;
-        tile_row_sm[j] = (int)row0;
-        tile_mask_sm[j] = tile_valid ? tile_valid[row0 / kTile] : ~0ull;
+        const int tile = list[it / nsub] * nsub + it % nsub;
+        const uint32_t entry = L.k_tiles != nullptr ? L.k_tiles[tile] : (uint32_t)tile * kTile;
+        tile_row_sm[j] = (int)entry;
+        tile_mask_sm[j] = tile_valid ? tile_valid[tile] : ~0ull;
     }
     // consume the Q loads here: otherwise their vmcnt waits land inside the tile loop,
     // where they would also wait for the LDS loads of the next tile
@@ -397,17 +430,22 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
                 }
                 *reinterpret_cast<uint2*>(orow + 32 * t + 8 * g + 4 * lh) = *reinterpret_cast<uint2*>(out4);
             }
-        if (lse != nullptr && lh == 0)
-            lse[(int64_t)bh * Sq + qrow0 + 32 * qh + lr] = l > 0.f ? (m + __builtin_log2f(l)) * kLn2 : -INFINITY;
+        if (lse != nullptr && lh == 0) {
+            int64_t row = qrow0 + 32 * qh + lr;
+            if (L.q_rows != nullptr) row = L.q_rows[row];
+            if (row >= 0) lse[(int64_t)bh * lse_S + row] = l > 0.f ? (m + __builtin_log2f(l)) * kLn2 : -INFINITY;
+        }
     }
     __syncthreads();
     {
-        T* ob = o + ((int64_t)bh * Sq + qrow0) * kD;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int r = kr + 16 * i;
-            *reinterpret_cast<uint4*>(ob + (int64_t)r * kD + kc * 8) =
-                *reinterpret_cast<const uint4*>(ost + r * kD + kc * 8);
+            int64_t row = qrow0 + r;
+            if (L.q_rows != nullptr) row = L.q_rows[row];
+            if (row >= 0)
+                *reinterpret_cast<uint4*>(o + o_bh + row * L.o_st[2] + kc * 8) =
+                    *reinterpret_cast<const uint4*>(ost + r * kD + kc * 8);
         }
     }
     }   // work items
@@ -505,8 +543,26 @@ static int resident_workgroups() {
 hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t* idx,
                       const int32_t* lens, const uint64_t* tile_valid, void* o, float* lse, int B,
                       int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride,
-                      float sm_scale, int dtype, hipStream_t st) {
+                      float sm_scale, int dtype, hipStream_t st, const FwdLayout* layout, int64_t layout_lse_rows,
+                      int64_t layout_edge_bytes) {
     const float qk_scale = sm_scale * kLog2e;
+    FwdLayout L;
+    int64_t lse_S = Sq, edge_bh_bytes = 0;
+    if (layout != nullptr) {
+        L = *layout;
+        lse_S = layout_lse_rows;
+        edge_bh_bytes = layout_edge_bytes;
+    } else {
+        L.q_rows = nullptr;
+        L.k_tiles = nullptr;
+        L.k_edge = L.v_edge = nullptr;
+        L.q_st[0] = L.o_st[0] = (int64_t)Hn * Sq * kD;
+        L.q_st[1] = L.o_st[1] = Sq * kD;
+        L.k_st[0] = L.v_st[0] = (int64_t)Hn * Sk * kD;
+        L.k_st[1] = L.v_st[1] = Sk * kD;
+        L.q_st[2] = L.o_st[2] = L.k_st[2] = L.v_st[2] = kD;
+        L.kw = 4; L.kh = 16; L.kH = 16; L.kW = 4;     // 16 runs of 4 rows, one after the other
+    }
     const dim3 block(256);
     if (dtype == BSA_F32) {
         const dim3 grid((unsigned)(Sq / kTile), (unsigned)(B * Hn));
@@ -529,11 +585,11 @@ hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t
             if (dtype == BSA_BF16)
                 hipLaunchKernelGGL((fwd_mfma_kernel<__bf16>), grid, block, 0, st, (const __bf16*)q,
                                    (const __bf16*)k, (const __bf16*)v, idx, lens, tile_valid, (__bf16*)o,
-                                   lse, Sq, Sk, bs_q, bs_k, idx_stride, qk_scale, begin, end);
+                                   lse, Sq, Sk, bs_q, bs_k, idx_stride, qk_scale, begin, end, Hn, lse_S, edge_bh_bytes, L);
             else
                 hipLaunchKernelGGL((fwd_mfma_kernel<_Float16>), grid, block, 0, st, (const _Float16*)q,
                                    (const _Float16*)k, (const _Float16*)v, idx, lens, tile_valid,
-                                   (_Float16*)o, lse, Sq, Sk, bs_q, bs_k, idx_stride, qk_scale, begin, end);
+                                   (_Float16*)o, lse, Sq, Sk, bs_q, bs_k, idx_stride, qk_scale, begin, end, Hn, lse_S, edge_bh_bytes, L);
         }
     }
     return hipGetLastError();

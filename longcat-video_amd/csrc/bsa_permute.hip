@@ -43,7 +43,8 @@ __device__ inline void finish_pool(float* acc, float* red, T* out_row, int cpr, 
 template <typename T, bool POOL>
 __global__ __launch_bounds__(kThreads) void permute_kernel(
     const T* __restrict__ src, int64_t sB, int64_t sH, int64_t sS, T* __restrict__ dst,
-    T* __restrict__ pooled, uint64_t* __restrict__ tile_valid, Grid3 g, int Hn, int D) {
+    T* __restrict__ pooled, uint64_t* __restrict__ tile_valid, Grid3 g, int Hn, int D, int edge_only, int n_edge,
+    int32_t* __restrict__ row_table, uint32_t* __restrict__ tile_table) {
     extern __shared__ float red[];
     constexpr int EPV = Piece<T>::EPV;
     const int blk = blockIdx.x;
@@ -56,6 +57,31 @@ __global__ __launch_bounds__(kThreads) void permute_kernel(
     const int c = threadIdx.x % cpr, rg = threadIdx.x / cpr, RG = kThreads / cpr;
     const T* sbase = src + (int64_t)b * sB + (int64_t)hd * sH;
     T* dbase = dst + ((int64_t)bh * nb + blk) * bs * D;
+    if (bh == 0 && row_table != nullptr) {
+        for (int r = threadIdx.x; r < bs; r += kThreads) {
+            const int wi = r % g.w, hi = (r / g.w) % g.h, ti = r / (g.w * g.h);
+            const int tt = nt * g.t + ti, hh = nh * g.h + hi, ww = nw * g.w + wi;
+            row_table[(int64_t)blk * bs + r] = (tt < g.T && hh < g.H && ww < g.W) ? (tt * g.H + hh) * g.W + ww : -1;
+        }
+    }
+    if (bh == 0 && tile_table != nullptr && threadIdx.x < bs / 64) {
+        const int sub = threadIdx.x, nsub = bs / 64, e = edge_index(g, blk);
+        const int planes = 64 / (g.w * g.h);          // a tile is a whole number of (h, w) planes here
+        tile_table[(int64_t)blk * nsub + sub] =
+            e < 0 ? (uint32_t)(((nt * g.t + sub * planes) * g.H + nh * g.h) * g.W + nw * g.w)
+                  : (1u << 24) + (uint32_t)(e * nsub + sub);
+    }
+    if (edge_only) {
+        const int e = edge_index(g, blk);
+        if (e < 0) {
+            dbase = nullptr;
+            if (!POOL && tile_valid == nullptr) return;      // nothing to do for this chunk
+        } else {
+            dbase = dst + ((int64_t)bh * n_edge + e) * bs * D;
+        }
+    } else if (dst == nullptr) {
+        dbase = nullptr;
+    }
     float acc[EPV];
 #pragma unroll
     for (int i = 0; i < EPV; ++i) acc[i] = 0.f;
@@ -68,7 +94,7 @@ __global__ __launch_bounds__(kThreads) void permute_kernel(
             const int64_t s = ((int64_t)tt * g.H + hh) * g.W + ww;
             val = *reinterpret_cast<const uint4*>(sbase + s * sS + c * EPV);
         }
-        *reinterpret_cast<uint4*>(dbase + (int64_t)r * D + c * EPV) = val;
+        if (dbase != nullptr) *reinterpret_cast<uint4*>(dbase + (int64_t)r * D + c * EPV) = val;
         if (POOL) accumulate<T>(acc, val);
     }
     if (tile_valid != nullptr && bh == 0) {
@@ -142,16 +168,17 @@ inline size_t red_bytes(int D, int esize) {
 
 hipError_t launch_permute(const void* src, const int64_t st3[3], void* dst, void* pooled,
                           uint64_t* tile_valid, int B, int Hn, const Grid3& g, int D, int dtype,
-                          hipStream_t st) {
+                          hipStream_t st, bool edge_only, int32_t* row_table, uint32_t* tile_table) {
     dim3 grid(g.blocks(), B * Hn), block(kThreads);
     const size_t smem = pooled ? red_bytes(D, dtype_size(dtype)) : 0;
+    const int eo = edge_only ? 1 : 0, ne = edge_only ? edge_count(g) : 0;
 #define BSA_LAUNCH(T)                                                                          \
     if (pooled)                                                                                \
         hipLaunchKernelGGL((permute_kernel<T, true>), grid, block, smem, st, (const T*)src,     \
-                           st3[0], st3[1], st3[2], (T*)dst, (T*)pooled, tile_valid, g, Hn, D);  \
+                           st3[0], st3[1], st3[2], (T*)dst, (T*)pooled, tile_valid, g, Hn, D, eo, ne, row_table, tile_table); \
     else                                                                                       \
         hipLaunchKernelGGL((permute_kernel<T, false>), grid, block, smem, st, (const T*)src,    \
-                           st3[0], st3[1], st3[2], (T*)dst, (T*)pooled, tile_valid, g, Hn, D);
+                           st3[0], st3[1], st3[2], (T*)dst, (T*)pooled, tile_valid, g, Hn, D, eo, ne, row_table, tile_table);
     if (dtype == BSA_BF16) { BSA_LAUNCH(__bf16) }
     else if (dtype == BSA_F16) { BSA_LAUNCH(_Float16) }
     else { BSA_LAUNCH(float) }

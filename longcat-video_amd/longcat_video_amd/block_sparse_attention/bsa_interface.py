@@ -250,6 +250,10 @@ def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k,
     tk, hk, wk = (int(x) for x in chunk_k)
     lib = _capi.load()
     q, k, v = _rows_ok(q), _rows_ok(k), _rows_ok(v)
+    if k.stride(2) != v.stride(2) or max(1, 64 // (wk * hk)) * Hk * Wk * k.stride(2) * k.element_size() >= 2 ** 32:
+        # the engine gathers k and v tiles with one set of in-tile offsets (32 bits); views that
+        # do not fit are copied once
+        k, v = k.contiguous(), v.contiguous()
     nbk = lib.bsa_padded_tokens(Tk, Hk, Wk, tk, hk, wk) // (tk * hk * wk)
     nbq = lib.bsa_padded_tokens(Tq, Hq, Wq, tq, hq, wq) // (tq * hq * wq)
     k_sel = num_selected(sparsity, nbk)

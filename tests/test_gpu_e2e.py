@@ -89,6 +89,36 @@ def test_default_chunk_4x4x8():
     assert torch.equal(pub, o)
 
 
+@pytest.mark.parametrize("latent,chunk", [
+    ((5, 6, 12), (4, 4, 8)),     # 128-slot chunks on a ragged grid: one 64-slot tile of the last layer is padding only
+    ((3, 9, 20), (2, 8, 4)),     # tiles of two (h, w) planes
+    ((6, 5, 36), (1, 4, 16)),    # one plane per tile, long runs along w, ragged h
+    ((4, 8, 6), (4, 8, 2)),      # runs of 2 tokens: k and v go through blocked copies
+    ((6, 7, 9), (4, 2, 8)),      # four planes of two runs per tile
+    ((2, 40, 8), (1, 32, 4)),    # a 64-slot tile is half a plane: blocked copies again
+])
+def test_chunk_shapes_on_ragged_grids(latent, chunk):
+    S = int(np.prod(latent))
+    q, k, v = seeded_qkv(36, 1, 2, S, S, 128, torch.bfloat16)
+    o, idx, lens, score = I()._bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, 0.5, chunk, chunk, True)
+    nb = int(np.prod(O.block_grid(latent, chunk)))
+    check_against_oracle(q, k, v, latent, latent, 0.5, o, idx, lens, score, q_blocks=range(nb), chunk=chunk)
+    assert torch.isfinite(o.float()).all()
+
+
+def test_strided_inputs_on_a_ragged_grid():
+    """q, k, v as views of one [B, S, 3, H, D] projection output and o written into a [B, S, H, D]
+    buffer, on a grid with padded chunks in every direction."""
+    latent = (5, 9, 13)
+    S = int(np.prod(latent))
+    qkv = torch.randn(1, S, 3, 2, 128, generator=torch.Generator().manual_seed(37)).bfloat16().cuda()
+    dq, dk, dv = qkv.permute(2, 0, 3, 1, 4).unbind(0)
+    out = torch.full((1, S, 2, 128), float("nan"), dtype=torch.bfloat16, device="cuda")
+    I()._bsa_3d(dq, dk, dv, latent, latent, 0.75, (4, 4, 4), (4, 4, 4), out=out.permute(0, 2, 1, 3))
+    ref = I()._bsa_3d(dq.contiguous(), dk.contiguous(), dv.contiguous(), latent, latent, 0.75, (4, 4, 4), (4, 4, 4))
+    assert torch.equal(out.permute(0, 2, 1, 3), ref)
+
+
 def test_rectangular_query_and_key_grids():
     """Tq != Tk, as in the noise half of the cond/noise split (attention.py:132-133)."""
     lq, lk = (4, 8, 8), (8, 8, 8)
