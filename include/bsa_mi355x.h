@@ -148,6 +148,10 @@ int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, con
  *   padded KV block count.  workspace: bsa_workspace_bytes() bytes, 256-byte
  *   aligned.  idx_out/lens_out/score_out are optional copies for inspection
  *   (shapes as in bsa_score_topk).
+ * For bf16 / fp16 no permuted copy of q, k, v or o is made: one pass over q and k
+ * produces the pooled means (and the tables of bsa_thw_prepare), and the attention
+ * kernel reads and writes THW order directly; k and v must then share one token
+ * stride (BSA_ERR_UNSUPPORTED otherwise).  fp32 goes through blocked copies.
  */
 typedef struct bsa_3d_params {
     int B, Hn, D, dtype;
@@ -166,6 +170,33 @@ int bsa_fwd_3d(const bsa_3d_params* p,
                void* o, const int64_t o_strides[3],
                void* workspace, size_t workspace_bytes,
                int32_t* idx_out, int32_t* lens_out, void* score_out, void* stream);
+
+/*
+ * R1 + R5 + R6 + R7 with a caller-supplied selection, bf16 / fp16: attention over THW-order
+ * tensors without permuted copies.  Replaces the sequence rearrange_THW_to_3d_block x3 (bsa:650-652),
+ * attn_fwd_bsa_varlen_triton (bsa:290-341), rearrange_3d_block_to_THW (bsa:659) for callers that
+ * select KV blocks themselves.  Two steps on one workspace of bsa_workspace_bytes(p) bytes:
+ *
+ * bsa_thw_prepare: builds what depends on the grids and on k, v only: the token row of every
+ *   blocked-order query slot, the position of every 64-slot kv tile, the tile validity words, and
+ *   blocked-order copies of the kv chunks that touch the padded high edge of the grid (all kv
+ *   chunks when the chunk shape does not allow gathering: w a power of two >= 4, h a power of two,
+ *   64-slot tiles made of whole (h, w) planes).  Call again whenever k or v change.
+ * bsa_fwd_thw: the attention kernel alone.  idx / lens / idx_stride / lse as in bsa_fwd, block
+ *   indices counted in the padded chunk grids; lse is [B, Hn, Tq*Hq*Wq] in THW order.
+ *   p->k_sel is not used.  k and v must share one token stride.
+ */
+int bsa_thw_prepare(const bsa_3d_params* p, const void* k, const int64_t k_strides[3],
+                    const void* v, const int64_t v_strides[3],
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+int bsa_fwd_thw(const bsa_3d_params* p,
+                const void* q, const int64_t q_strides[3],
+                const void* k, const int64_t k_strides[3],
+                const void* v, const int64_t v_strides[3],
+                void* o, const int64_t o_strides[3],
+                const int32_t* idx, const int32_t* lens, int idx_stride, float* lse,
+                void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * R11 glue of the attention module (longcat_video/modules/attention.py:107-147).

@@ -241,77 +241,171 @@ size_t bsa_workspace_bytes(const bsa_3d_params* p) {
     return pl.total;
 }
 
+namespace {
+struct Ws {
+    void *qp, *kp, *vp, *op, *qc, *kc, *score;
+    int32_t *idx, *idx_sorted, *lens, *qrows;
+    uint32_t* ktiles;
+    uint64_t* valid;
+};
+int carve(const Plan& pl, void* workspace, size_t workspace_bytes, const char* who, Ws* w) {
+    if (!workspace) return set_error(BSA_ERR_BAD_ARG, "%s: workspace is null", who);
+    if (workspace_bytes < pl.total)
+        return set_error(BSA_ERR_WORKSPACE, "%s: workspace of %zu bytes is smaller than the %zu required", who, workspace_bytes, pl.total);
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return set_error(BSA_ERR_BAD_ARG, "%s: workspace must be 256-byte aligned", who);
+    char* ws = static_cast<char*>(workspace);
+    w->qp = ws + pl.off_qp; w->kp = ws + pl.off_kp; w->vp = ws + pl.off_vp; w->op = ws + pl.off_op;
+    w->qc = ws + pl.off_qc; w->kc = ws + pl.off_kc; w->score = ws + pl.off_score;
+    w->idx = reinterpret_cast<int32_t*>(ws + pl.off_idx);
+    w->idx_sorted = reinterpret_cast<int32_t*>(ws + pl.off_idx_sorted);
+    w->lens = reinterpret_cast<int32_t*>(ws + pl.off_lens);
+    w->valid = reinterpret_cast<uint64_t*>(ws + pl.off_valid);
+    w->qrows = pl.direct_qo ? reinterpret_cast<int32_t*>(ws + pl.off_qrows) : nullptr;
+    w->ktiles = pl.direct_kv ? reinterpret_cast<uint32_t*>(ws + pl.off_ktiles) : nullptr;
+    return BSA_OK;
+}
+bool kv_padded(const bsa_3d_params* p) { return (p->Tk % p->tk) || (p->Hk % p->hk) || (p->Wk % p->wk); }
+
+int check_kv_views(const Plan& pl, const int64_t k_strides[3], const int64_t v_strides[3], const char* who) {
+    if (pl.direct_kv && (k_strides[2] != v_strides[2] || !kv_direct_ok(pl.gk, k_strides[2] * pl.es)))
+        return set_error(BSA_ERR_UNSUPPORTED, "%s: k and v must share one token stride (got %lld and %lld elements) small "
+                         "enough for 32-bit offsets inside a tile; pass contiguous copies",
+                         who, (long long)k_strides[2], (long long)v_strides[2]);
+    return BSA_OK;
+}
+
+// Everything the attention kernel needs besides the selection, for the 16-bit types: the row table
+// of q, and for k and v the tile table, the validity words and the copies of the edge chunks (or
+// of all chunks when the kv grid does not allow gathering).  With `pool`, q and k are also read in
+// full and their chunk means stored (one pass over each).
+hipError_t prepare_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, const void* q, const int64_t q_strides[3],
+                       const void* k, const int64_t k_strides[3], const void* v, const int64_t v_strides[3], bool pool,
+                       hipStream_t st) {
+    hipError_t e;
+    const bool padded_k = kv_padded(p);
+    if (pool)
+        e = launch_permute(q, q_strides, nullptr, w.qc, nullptr, p->B, p->Hn, pl.gq, p->D, p->dtype, st, false, w.qrows, nullptr);
+    else    // tables only: one (batch, head) slice of workgroups, no row is read
+        e = launch_permute(q, q_strides, nullptr, nullptr, nullptr, 1, 1, pl.gq, p->D, p->dtype, st, false, w.qrows, nullptr);
+    if (e != hipSuccess) return e;
+    e = launch_permute(k, k_strides, w.kp, pool ? w.kc : nullptr, padded_k ? w.valid : nullptr, p->B, p->Hn, pl.gk, p->D,
+                       p->dtype, st, pl.direct_kv, nullptr, w.ktiles);
+    if (e != hipSuccess) return e;
+    if (!pl.direct_kv || padded_k)
+        e = launch_permute(v, v_strides, w.vp, nullptr, nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st, pl.direct_kv);
+    return e;
+}
+
+hipError_t attention_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, const void* q, const int64_t q_strides[3],
+                         const void* k, const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
+                         const int64_t o_strides[3], const int32_t* idx, const int32_t* lens, int idx_stride, float* lse,
+                         hipStream_t st) {
+    FwdLayout L;
+    L.q_rows = w.qrows;
+    L.k_tiles = w.ktiles;
+    L.k_edge = w.kp;
+    L.v_edge = w.vp;
+    for (int i = 0; i < 3; ++i) { L.q_st[i] = q_strides[i]; L.o_st[i] = o_strides[i]; }
+    if (pl.direct_kv) {
+        for (int i = 0; i < 3; ++i) { L.k_st[i] = k_strides[i]; L.v_st[i] = v_strides[i]; }
+        L.kw = pl.gk.w; L.kh = pl.gk.h; L.kH = pl.gk.H; L.kW = pl.gk.W;
+    } else {
+        L.k_st[0] = L.v_st[0] = (int64_t)p->Hn * pl.Skp * p->D;
+        L.k_st[1] = L.v_st[1] = pl.Skp * p->D;
+        L.k_st[2] = L.v_st[2] = p->D;
+        L.kw = 4; L.kh = 16; L.kH = 16; L.kW = 4;
+    }
+    return launch_fwd(q, pl.direct_kv ? k : w.kp, pl.direct_kv ? v : w.vp, idx, lens, kv_padded(p) ? w.valid : nullptr, o, lse,
+                      p->B, p->Hn, pl.Sqp, pl.Skp, pl.gq.chunk(), pl.gk.chunk(), idx_stride, p->sm_scale, p->dtype, st, &L,
+                      (int64_t)p->Tq * p->Hq * p->Wq, (int64_t)edge_count(pl.gk) * pl.gk.chunk() * p->D * pl.es);
+}
+
+int check_tensor(const void* x, const int64_t strides[3], const bsa_3d_params* p, const char* name) {
+    if (!x) return set_error(BSA_ERR_BAD_ARG, "%s is null", name);
+    BSA_TRY(check_strides(strides, p->D, p->dtype, name));
+    if (!aligned16(x)) return set_error(BSA_ERR_BAD_ARG, "%s must be 16-byte aligned", name);
+    return BSA_OK;
+}
+}  // namespace
+
+int bsa_thw_prepare(const bsa_3d_params* p, const void* k, const int64_t k_strides[3], const void* v,
+                    const int64_t v_strides[3], void* workspace, size_t workspace_bytes, void* stream) {
+    Plan pl;
+    Ws w;
+    BSA_TRY(make_plan(p, &pl));
+    if (!pl.direct_qo) return set_error(BSA_ERR_UNSUPPORTED, "thw_prepare: bf16 and fp16 only (fp32 runs through bsa_fwd_3d)");
+    BSA_TRY(carve(pl, workspace, workspace_bytes, "thw_prepare", &w));
+    BSA_TRY(check_tensor(k, k_strides, p, "k"));
+    BSA_TRY(check_tensor(v, v_strides, p, "v"));
+    BSA_TRY(check_kv_views(pl, k_strides, v_strides, "thw_prepare"));
+    const int64_t none[3] = {0, 0, p->D};
+    const hipError_t e = prepare_thw(pl, p, w, k, none, k, k_strides, v, v_strides, false, (hipStream_t)stream);
+    return e == hipSuccess ? BSA_OK : hip_fail(e, "thw_prepare");
+}
+
+int bsa_fwd_thw(const bsa_3d_params* p, const void* q, const int64_t q_strides[3], const void* k,
+                const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
+                const int64_t o_strides[3], const int32_t* idx, const int32_t* lens, int idx_stride, float* lse,
+                void* workspace, size_t workspace_bytes, void* stream) {
+    Plan pl;
+    Ws w;
+    BSA_TRY(make_plan(p, &pl));
+    if (!pl.direct_qo) return set_error(BSA_ERR_UNSUPPORTED, "fwd_thw: bf16 and fp16 only (fp32 runs through bsa_fwd_3d)");
+    BSA_TRY(carve(pl, workspace, workspace_bytes, "fwd_thw", &w));
+    BSA_TRY(check_tensor(q, q_strides, p, "q"));
+    BSA_TRY(check_tensor(k, k_strides, p, "k"));
+    BSA_TRY(check_tensor(v, v_strides, p, "v"));
+    BSA_TRY(check_tensor(o, o_strides, p, "o"));
+    BSA_TRY(check_kv_views(pl, k_strides, v_strides, "fwd_thw"));
+    if (!lens || idx_stride < 0 || (!idx && idx_stride > 0)) return set_error(BSA_ERR_BAD_ARG, "fwd_thw: selection is missing");
+    const hipError_t e = attention_thw(pl, p, w, q, q_strides, k, k_strides, v, v_strides, o, o_strides, idx, lens, idx_stride,
+                                       lse, (hipStream_t)stream);
+    return e == hipSuccess ? BSA_OK : hip_fail(e, "fwd_thw");
+}
+
 int bsa_fwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3], const void* k,
                const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
                const int64_t o_strides[3], void* workspace, size_t workspace_bytes, int32_t* idx_out,
                int32_t* lens_out, void* score_out, void* stream) {
     Plan pl;
+    Ws w;
     BSA_TRY(make_plan(p, &pl));
     if (!q || !k || !v || !o || !workspace) return set_error(BSA_ERR_BAD_ARG, "fwd_3d: null pointer");
-    if (workspace_bytes < pl.total)
-        return set_error(BSA_ERR_WORKSPACE, "fwd_3d: workspace of %zu bytes is smaller than the %zu required", workspace_bytes, pl.total);
-    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return set_error(BSA_ERR_BAD_ARG, "fwd_3d: workspace must be 256-byte aligned");
-    BSA_TRY(check_strides(q_strides, p->D, p->dtype, "q"));
-    BSA_TRY(check_strides(k_strides, p->D, p->dtype, "k"));
-    BSA_TRY(check_strides(v_strides, p->D, p->dtype, "v"));
-    BSA_TRY(check_strides(o_strides, p->D, p->dtype, "o"));
-    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
-        return set_error(BSA_ERR_BAD_ARG, "fwd_3d: q/k/v/o must be 16-byte aligned");
+    BSA_TRY(carve(pl, workspace, workspace_bytes, "fwd_3d", &w));
+    BSA_TRY(check_tensor(q, q_strides, p, "q"));
+    BSA_TRY(check_tensor(k, k_strides, p, "k"));
+    BSA_TRY(check_tensor(v, v_strides, p, "v"));
+    BSA_TRY(check_tensor(o, o_strides, p, "o"));
+    BSA_TRY(check_kv_views(pl, k_strides, v_strides, "fwd_3d"));
 
-    char* ws = static_cast<char*>(workspace);
-    void* qp = ws + pl.off_qp; void* kp = ws + pl.off_kp; void* vp = ws + pl.off_vp; void* op = ws + pl.off_op;
-    void* qc = ws + pl.off_qc; void* kc = ws + pl.off_kc; void* score = ws + pl.off_score;
-    int32_t* idx = reinterpret_cast<int32_t*>(ws + pl.off_idx);
-    int32_t* idx_sorted = reinterpret_cast<int32_t*>(ws + pl.off_idx_sorted);
-    int32_t* lens = reinterpret_cast<int32_t*>(ws + pl.off_lens);
-    uint64_t* valid = reinterpret_cast<uint64_t*>(ws + pl.off_valid);
-    const bool padded_k = (p->Tk % p->tk) || (p->Hk % p->hk) || (p->Wk % p->wk);
+    const bool padded_k = kv_padded(p);
     hipStream_t st = (hipStream_t)stream;
     hipError_t e;
 #define BSA_HIP(call, what) do { e = (call); if (e != hipSuccess) return hip_fail(e, what); } while (0)
-    int32_t* qrows = pl.direct_qo ? reinterpret_cast<int32_t*>(ws + pl.off_qrows) : nullptr;
-    uint32_t* ktiles = pl.direct_kv ? reinterpret_cast<uint32_t*>(ws + pl.off_ktiles) : nullptr;
-    BSA_HIP(launch_permute(q, q_strides, pl.direct_qo ? nullptr : qp, qc, nullptr, p->B, p->Hn, pl.gq, p->D, p->dtype, st, false, qrows, nullptr), "permute q");
-    if (pl.direct_kv && (k_strides[2] != v_strides[2] || !kv_direct_ok(pl.gk, k_strides[2] * pl.es)))
-        return set_error(BSA_ERR_UNSUPPORTED, "fwd_3d: k and v must share one token stride (got %lld and %lld elements) "
-                         "small enough for 32-bit offsets inside a tile; pass contiguous copies",
-                         (long long)k_strides[2], (long long)v_strides[2]);
-    BSA_HIP(launch_permute(k, k_strides, kp, kc, padded_k ? valid : nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st, pl.direct_kv, nullptr, ktiles), "permute k");
-    if (!pl.direct_kv || padded_k)
-        BSA_HIP(launch_permute(v, v_strides, vp, nullptr, nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st, pl.direct_kv), "permute v");
-    BSA_HIP(launch_score(qc, kc, score, p->B * p->Hn, pl.nbq, pl.nbk, p->D, p->dtype, st), "score");
+    if (pl.direct_qo) {
+        BSA_HIP(prepare_thw(pl, p, w, q, q_strides, k, k_strides, v, v_strides, true, st), "pool and prepare");
+    } else {
+        BSA_HIP(launch_permute(q, q_strides, w.qp, w.qc, nullptr, p->B, p->Hn, pl.gq, p->D, p->dtype, st), "permute q");
+        BSA_HIP(launch_permute(k, k_strides, w.kp, w.kc, padded_k ? w.valid : nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st), "permute k");
+        BSA_HIP(launch_permute(v, v_strides, w.vp, nullptr, nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st), "permute v");
+    }
+    BSA_HIP(launch_score(w.qc, w.kc, w.score, p->B * p->Hn, pl.nbq, pl.nbk, p->D, p->dtype, st), "score");
     // the attention kernel walks each list in ascending block order (L2 locality); the score
     // order is only produced when the caller asks for the selection
-    BSA_HIP(launch_topk(score, idx_out ? idx : nullptr, idx_sorted, lens, (int64_t)p->B * p->Hn * pl.nbq, pl.nbk, p->k_sel, p->dtype, st), "top-k");
+    BSA_HIP(launch_topk(w.score, idx_out ? w.idx : nullptr, w.idx_sorted, w.lens, (int64_t)p->B * p->Hn * pl.nbq, pl.nbk, p->k_sel, p->dtype, st), "top-k");
     if (pl.direct_qo) {
-        FwdLayout L;
-        L.q_rows = qrows;
-        L.k_tiles = ktiles;
-        L.k_edge = kp;
-        L.v_edge = vp;
-        for (int i = 0; i < 3; ++i) { L.q_st[i] = q_strides[i]; L.o_st[i] = o_strides[i]; }
-        if (pl.direct_kv) {
-            for (int i = 0; i < 3; ++i) { L.k_st[i] = k_strides[i]; L.v_st[i] = v_strides[i]; }
-            L.kw = pl.gk.w; L.kh = pl.gk.h; L.kH = pl.gk.H; L.kW = pl.gk.W;
-        } else {
-            L.k_st[0] = L.v_st[0] = (int64_t)p->Hn * pl.Skp * p->D;
-            L.k_st[1] = L.v_st[1] = pl.Skp * p->D;
-            L.k_st[2] = L.v_st[2] = p->D;
-            L.kw = 4; L.kh = 16; L.kH = 16; L.kW = 4;
-        }
-        BSA_HIP(launch_fwd(q, pl.direct_kv ? k : kp, pl.direct_kv ? v : vp, idx_sorted, lens, padded_k ? valid : nullptr, o, nullptr,
-                           p->B, p->Hn, pl.Sqp, pl.Skp, pl.gq.chunk(), pl.gk.chunk(), p->k_sel, p->sm_scale, p->dtype, st, &L,
-                           (int64_t)p->Tq * p->Hq * p->Wq, (int64_t)edge_count(pl.gk) * pl.gk.chunk() * p->D * pl.es), "attention");
+        BSA_HIP(attention_thw(pl, p, w, q, q_strides, k, k_strides, v, v_strides, o, o_strides, w.idx_sorted, w.lens, p->k_sel,
+                              nullptr, st), "attention");
     } else {
-        BSA_HIP(launch_fwd(qp, kp, vp, idx_sorted, lens, padded_k ? valid : nullptr, op, nullptr, p->B, p->Hn, pl.Sqp, pl.Skp,
+        BSA_HIP(launch_fwd(w.qp, w.kp, w.vp, w.idx_sorted, w.lens, padded_k ? w.valid : nullptr, w.op, nullptr, p->B, p->Hn, pl.Sqp, pl.Skp,
                            pl.gq.chunk(), pl.gk.chunk(), p->k_sel, p->sm_scale, p->dtype, st), "attention");
-        BSA_HIP(launch_unpermute(op, o, o_strides, p->B, p->Hn, pl.gq, p->D, p->dtype, st), "unpermute");
+        BSA_HIP(launch_unpermute(w.op, o, o_strides, p->B, p->Hn, pl.gq, p->D, p->dtype, st), "unpermute");
     }
     const size_t bh = (size_t)p->B * p->Hn;
     if (idx_out && p->k_sel > 0)
-        BSA_HIP(hipMemcpyAsync(idx_out, idx, bh * pl.nbq * p->k_sel * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy idx");
-    if (lens_out) BSA_HIP(hipMemcpyAsync(lens_out, lens, bh * pl.nbq * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy lens");
-    if (score_out) BSA_HIP(hipMemcpyAsync(score_out, score, bh * pl.nbq * (size_t)pl.nbk * pl.es, hipMemcpyDeviceToDevice, st), "copy score");
+        BSA_HIP(hipMemcpyAsync(idx_out, w.idx, bh * pl.nbq * p->k_sel * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy idx");
+    if (lens_out) BSA_HIP(hipMemcpyAsync(lens_out, w.lens, bh * pl.nbq * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy lens");
+    if (score_out) BSA_HIP(hipMemcpyAsync(score_out, w.score, bh * pl.nbq * (size_t)pl.nbk * pl.es, hipMemcpyDeviceToDevice, st), "copy score");
 #undef BSA_HIP
     return BSA_OK;
 }

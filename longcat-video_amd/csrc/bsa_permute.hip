@@ -73,20 +73,15 @@ __global__ __launch_bounds__(kThreads) void permute_kernel(
     }
     if (edge_only) {
         const int e = edge_index(g, blk);
-        if (e < 0) {
-            dbase = nullptr;
-            if (!POOL && tile_valid == nullptr) return;      // nothing to do for this chunk
-        } else {
-            dbase = dst + ((int64_t)bh * n_edge + e) * bs * D;
-        }
-    } else if (dst == nullptr) {
-        dbase = nullptr;
+        dbase = e < 0 ? nullptr : dst + ((int64_t)bh * n_edge + e) * bs * D;
     }
+    if (dst == nullptr) dbase = nullptr;
     float acc[EPV];
 #pragma unroll
     for (int i = 0; i < EPV; ++i) acc[i] = 0.f;
 
-    for (int r = rg; r < bs; r += RG) {
+    // the rows are only read when they are copied or pooled
+    for (int r = (POOL || dbase != nullptr) ? rg : bs; r < bs; r += RG) {
         const int wi = r % g.w, hi = (r / g.w) % g.h, ti = r / (g.w * g.h);
         const int tt = nt * g.t + ti, hh = nh * g.h + hi, ww = nw * g.w + wi;
         uint4 val = make_uint4(0, 0, 0, 0);

@@ -44,6 +44,9 @@ SIGNATURES = {
     "bsa_workspace_bytes": (C.c_size_t, [C.POINTER(Bsa3dParams)]),
     "bsa_fwd_3d": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
                         _p, C.c_size_t, _p, _p, _p, _p]),
+    "bsa_thw_prepare": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, C.c_size_t, _p]),
+    "bsa_fwd_thw": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
+                         _p, _p, _i, _p, _p, C.c_size_t, _p]),
     "bsa_rmsnorm": (_i, [_p, _p, _p, _i64, _i, _f, _i, _p]),
     "bsa_qk_norm_rope": (_i, [_p, _strides, _p, _strides, _p, _p, _p] + [_i] * 6 + [_f, _i, _p]),
     "bsa_linear_bf16": (_i, [_p, _p, _p, _p, _p, _i64, _i, _i, _p, C.c_size_t, _p]),

@@ -279,6 +279,64 @@ def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k,
     return (o, idx, lens, score) if want_selection else o
 
 
+class ThwAttention:
+    """Block-sparse attention over (T,H,W)-ordered tensors with a caller-supplied selection, in two
+    steps: the constructor prepares what depends on k and v (bsa_thw_prepare), every call runs the
+    attention kernel alone (bsa_fwd_thw).  bf16 / fp16."""
+
+    def __init__(self, k, v, latent_shape_q, latent_shape_k, chunk_3d_shape_q, chunk_3d_shape_k, sm_scale=None):
+        _need_gpu(k, v)
+        B, H, Sk, D = k.shape
+        self.gq = tuple(int(x) for x in latent_shape_q) + tuple(int(x) for x in chunk_3d_shape_q)
+        Tq, Hq, Wq, tq, hq, wq = self.gq
+        Tk, Hk, Wk = (int(x) for x in latent_shape_k)
+        tk, hk, wk = (int(x) for x in chunk_3d_shape_k)
+        assert Tk * Hk * Wk == Sk and v.shape == k.shape and v.dtype == k.dtype
+        self.lib = lib = _capi.load()
+        k, v = _rows_ok(k), _rows_ok(v)
+        if k.stride(2) != v.stride(2) or max(1, 64 // (wk * hk)) * Hk * Wk * k.stride(2) * k.element_size() >= 2 ** 32:
+            k, v = k.contiguous(), v.contiguous()      # one set of 32-bit in-tile offsets serves both
+        self.k, self.v = k, v
+        self.nbq = lib.bsa_padded_tokens(Tq, Hq, Wq, tq, hq, wq) // (tq * hq * wq)
+        scale = 1.0 / D ** 0.5 if sm_scale is None else float(sm_scale)
+        self.prm = _capi.Bsa3dParams(B, H, D, _code(k), Tq, Hq, Wq, Tk, Hk, Wk, tq, hq, wq, tk, hk, wk, 0, scale)
+        self.need = lib.bsa_workspace_bytes(C.byref(self.prm))
+        self.ws = torch.empty(max(self.need, 1), dtype=torch.uint8, device=k.device)
+        self.ks, self.vs = _capi.strides3(k.stride()[:3]), _capi.strides3(v.stride()[:3])
+        with torch.cuda.device(k.device):
+            _capi.check(lib.bsa_thw_prepare(C.byref(self.prm), _ptr(k), self.ks, _ptr(v), self.vs, _ptr(self.ws),
+                                            self.need, _stream(k)), "bsa_thw_prepare")
+
+    def __call__(self, q, block_indices, block_indices_lens, return_lse=False, out=None):
+        _need_gpu(q)
+        B, H, Sq, D = q.shape
+        Tq, Hq, Wq = self.gq[:3]
+        assert Tq * Hq * Wq == Sq and (B, H, D) == (self.k.shape[0], self.k.shape[1], self.k.shape[3]) and q.dtype == self.k.dtype
+        q = _rows_ok(q)
+        idx = block_indices.to(torch.int32).contiguous()
+        lens = block_indices_lens.to(torch.int32).contiguous()
+        assert idx.shape[:3] == (B, H, self.nbq) and lens.shape == (B, H, self.nbq)
+        o = torch.empty(B, H, Sq, D, dtype=q.dtype, device=q.device) if out is None else out
+        assert o.shape == (B, H, Sq, D) and o.dtype == q.dtype and o.stride(3) == 1
+        lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device) if return_lse else None
+        with torch.cuda.device(q.device):
+            _capi.check(self.lib.bsa_fwd_thw(
+                C.byref(self.prm), _ptr(q), _capi.strides3(q.stride()[:3]), _ptr(self.k), self.ks, _ptr(self.v), self.vs,
+                _ptr(o), _capi.strides3(o.stride()[:3]), _ptr(idx), _ptr(lens), idx.shape[3], _ptr(lse),
+                _ptr(self.ws), self.need, _stream(q)), "bsa_fwd_thw")
+        return (o, lse) if return_lse else o
+
+
+def attn_fwd_bsa_thw(q, k, v, latent_shape_q, latent_shape_k, chunk_3d_shape_q, chunk_3d_shape_k,
+                     block_indices, block_indices_lens, sm_scale=None, return_lse=False, out=None):
+    """What the reference does with three rearrange_THW_to_3d_block calls, attn_fwd_bsa_varlen_triton
+    and rearrange_3d_block_to_THW (bsa_interface.py:650-659, 290-341), without the permuted copies.
+    block_indices [B,H,nbq,n] / block_indices_lens [B,H,nbq] count chunks of the padded grids.
+    Returns o [B,H,Sq,D] (and lse [B,H,Sq] fp32, natural log, with return_lse)."""
+    return ThwAttention(k, v, latent_shape_q, latent_shape_k, chunk_3d_shape_q, chunk_3d_shape_k, sm_scale)(
+        q, block_indices, block_indices_lens, return_lse, out)
+
+
 @torch.library.custom_op("longcat_video_amd::flash_attn_bsa_3d", mutates_args=())
 def _bsa_3d_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, latent_shape_q: Sequence[int],
                latent_shape_k: Sequence[int], sparsity: float, chunk_3d_shape_q: Sequence[int],

@@ -159,3 +159,36 @@ def test_480p_two_heads_sampled_rows():
         sl = slice(m * 64, (m + 1) * 64)
         close(o[:, :, sl], want[:, :, sl], torch.bfloat16)
         assert torch.allclose(lse[:, :, sl], want_lse[:, :, sl], atol=2e-3)
+
+
+@pytest.mark.parametrize("latent,chunk", [
+    ((5, 9, 13), (4, 4, 4)),     # padded chunks in t, h and w
+    ((5, 6, 12), (4, 4, 8)),     # 128-slot chunks, one 64-slot tile of padding only
+    ((4, 8, 6), (4, 8, 2)),      # chunk shape without gathering: k and v copied in full
+])
+def test_thw_attention_equals_permute_attend_unpermute(latent, chunk):
+    """attn_fwd_bsa_thw reads q/k/v and writes o/lse in (T,H,W) order; the blocked-order kernel between
+    a permute and an unpermute (bsa_interface.py:650-659) must give the same bits, also for lists
+    of different lengths (an empty one included) in arbitrary order."""
+    bi = I()
+    S = int(np.prod(latent))
+    bs = int(np.prod(chunk))
+    q, k, v = (x.cuda() for x in seeded_qkv(41, 1, 2, S, S, 128, torch.bfloat16))
+    nb = int(np.prod(O.block_grid(latent, chunk)))
+    gen = torch.Generator().manual_seed(42)
+    n = max(nb // 2, 1)
+    idx = torch.stack([torch.randperm(nb, generator=gen)[:n] for _ in range(2 * nb)]).view(1, 2, nb, n).int().cuda()
+    lens = torch.randint(0, n + 1, (1, 2, nb), generator=gen).int().cuda()
+    lens[0, 0, 0] = 0
+    lens[0, 1, nb - 1] = n
+    qp, _, _ = bi._permute(q, latent, chunk)
+    kp, _, valid = bi._permute(k, latent, chunk, want_valid=True)
+    vp, _, _ = bi._permute(v, latent, chunk)
+    padded = any(a % c for a, c in zip(latent, chunk))
+    op, lse_p = bi.attn_fwd_bsa_varlen(qp, kp, vp, 0.11, idx, lens, bs, bs, tile_valid=valid if padded else None)
+    grid = O.block_grid(latent, chunk)
+    want = bi.rearrange_3d_block_to_THW(op, *grid, *chunk, 128, latent_shape=latent)
+    want_lse = O.rearrange_3d_block_to_thw(lse_p.cpu().unsqueeze(-1), latent, chunk)[..., 0]
+    got, lse = bi.attn_fwd_bsa_thw(q, k, v, latent, latent, chunk, chunk, idx, lens, sm_scale=0.11, return_lse=True)
+    assert torch.equal(got, want)
+    assert torch.equal(lse.cpu(), want_lse)
