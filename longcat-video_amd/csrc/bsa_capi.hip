@@ -288,11 +288,12 @@ hipError_t prepare_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, cons
     else    // tables only: one (batch, head) slice of workgroups, no row is read
         e = launch_permute(q, q_strides, nullptr, nullptr, nullptr, 1, 1, pl.gq, p->D, p->dtype, st, false, w.qrows, nullptr);
     if (e != hipSuccess) return e;
+    // gathering: the pass over k copies the edge chunks of v along with those of k
     e = launch_permute(k, k_strides, w.kp, pool ? w.kc : nullptr, padded_k ? w.valid : nullptr, p->B, p->Hn, pl.gk, p->D,
-                       p->dtype, st, pl.direct_kv, nullptr, w.ktiles);
+                       p->dtype, st, pl.direct_kv, nullptr, w.ktiles, pl.direct_kv && padded_k ? v : nullptr, v_strides, w.vp);
     if (e != hipSuccess) return e;
-    if (!pl.direct_kv || padded_k)
-        e = launch_permute(v, v_strides, w.vp, nullptr, nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st, pl.direct_kv);
+    if (!pl.direct_kv)
+        e = launch_permute(v, v_strides, w.vp, nullptr, nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st);
     return e;
 }
 

@@ -97,10 +97,12 @@ int set_error(int code, const char* fmt, ...);
 // edge_only: dst is [B*Hn][edge_count(g)][chunk][D] and only chunks with padded slots are copied
 // row_table ([S_padded] int32): token row of every blocked-order slot, -1 for padding.
 // tile_table ([S_padded/64] uint32): FwdLayout::k_tiles.  Both optional.
+// src2 / dst2 (edge_only): a second tensor on the same grid whose edge chunks are copied as well.
 hipError_t launch_permute(const void* src, const int64_t strides[3], void* dst, void* pooled,
                           uint64_t* tile_valid, int B, int Hn, const Grid3& g, int D, int dtype,
                           hipStream_t st, bool edge_only = false, int32_t* row_table = nullptr,
-                          uint32_t* tile_table = nullptr);
+                          uint32_t* tile_table = nullptr, const void* src2 = nullptr,
+                          const int64_t* strides2 = nullptr, void* dst2 = nullptr);
 hipError_t launch_unpermute(const void* src, void* dst, const int64_t strides[3], int B, int Hn,
                             const Grid3& g, int D, int dtype, hipStream_t st);
 hipError_t launch_mean_pool(const void* x, void* out, int B, int Hn, int64_t S, int block, int D,

@@ -44,7 +44,8 @@ template <typename T, bool POOL>
 __global__ __launch_bounds__(kThreads) void permute_kernel(
     const T* __restrict__ src, int64_t sB, int64_t sH, int64_t sS, T* __restrict__ dst,
     T* __restrict__ pooled, uint64_t* __restrict__ tile_valid, Grid3 g, int Hn, int D, int edge_only, int n_edge,
-    int32_t* __restrict__ row_table, uint32_t* __restrict__ tile_table) {
+    int32_t* __restrict__ row_table, uint32_t* __restrict__ tile_table,
+    const T* __restrict__ src2, int64_t s2B, int64_t s2H, int64_t s2S, T* __restrict__ dst2) {
     extern __shared__ float red[];
     constexpr int EPV = Piece<T>::EPV;
     const int blk = blockIdx.x;
@@ -80,17 +81,45 @@ __global__ __launch_bounds__(kThreads) void permute_kernel(
 #pragma unroll
     for (int i = 0; i < EPV; ++i) acc[i] = 0.f;
 
-    // the rows are only read when they are copied or pooled
-    for (int r = (POOL || dbase != nullptr) ? rg : bs; r < bs; r += RG) {
+    // The rows are only read when they are copied or pooled.  Four rows per thread are requested
+    // before the first one is used, so that a workgroup has its whole 64-slot chunk in flight.
+    auto fetch = [&](const T* base, int64_t stride_s, int r) -> uint4 {
         const int wi = r % g.w, hi = (r / g.w) % g.h, ti = r / (g.w * g.h);
         const int tt = nt * g.t + ti, hh = nh * g.h + hi, ww = nw * g.w + wi;
         uint4 val = make_uint4(0, 0, 0, 0);
-        if (tt < g.T && hh < g.H && ww < g.W) {
+        if (r < bs && tt < g.T && hh < g.H && ww < g.W) {
             const int64_t s = ((int64_t)tt * g.H + hh) * g.W + ww;
-            val = *reinterpret_cast<const uint4*>(sbase + s * sS + c * EPV);
+            val = *reinterpret_cast<const uint4*>(base + s * stride_s + c * EPV);
         }
-        if (dbase != nullptr) *reinterpret_cast<uint4*>(dbase + (int64_t)r * D + c * EPV) = val;
-        if (POOL) accumulate<T>(acc, val);
+        return val;
+    };
+    for (int r0 = (POOL || dbase != nullptr) ? rg : bs; r0 < bs; r0 += 4 * RG) {
+        uint4 val[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) val[j] = fetch(sbase, sS, r0 + j * RG);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int r = r0 + j * RG;
+            if (r < bs) {
+                if (dbase != nullptr) *reinterpret_cast<uint4*>(dbase + (int64_t)r * D + c * EPV) = val[j];
+                if (POOL) accumulate<T>(acc, val[j]);
+            }
+        }
+    }
+    // a second tensor on the same grid (v next to k): edge chunks only
+    if (src2 != nullptr && edge_only && dbase != nullptr) {
+        const T* sbase2 = src2 + (int64_t)b * s2B + (int64_t)hd * s2H;
+        T* dbase2 = dst2 + (dbase - dst);
+        for (int r0 = rg; r0 < bs; r0 += 4 * RG) {
+            uint4 val[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) val[j] = fetch(sbase2, s2S, r0 + j * RG);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int r = r0 + j * RG;
+                if (r < bs) *reinterpret_cast<uint4*>(dbase2 + (int64_t)r * D + c * EPV) = val[j];
+            }
+        }
     }
     if (tile_valid != nullptr && bh == 0) {
         // bit s of word i <=> slot 64*i+s of the blocked order holds a real token
@@ -163,17 +192,22 @@ inline size_t red_bytes(int D, int esize) {
 
 hipError_t launch_permute(const void* src, const int64_t st3[3], void* dst, void* pooled,
                           uint64_t* tile_valid, int B, int Hn, const Grid3& g, int D, int dtype,
-                          hipStream_t st, bool edge_only, int32_t* row_table, uint32_t* tile_table) {
+                          hipStream_t st, bool edge_only, int32_t* row_table, uint32_t* tile_table,
+                          const void* src2, const int64_t* st3_2, void* dst2) {
+    const int64_t zero3[3] = {0, 0, 0};
+    const int64_t* s2 = st3_2 ? st3_2 : zero3;
     dim3 grid(g.blocks(), B * Hn), block(kThreads);
     const size_t smem = pooled ? red_bytes(D, dtype_size(dtype)) : 0;
     const int eo = edge_only ? 1 : 0, ne = edge_only ? edge_count(g) : 0;
 #define BSA_LAUNCH(T)                                                                          \
     if (pooled)                                                                                \
         hipLaunchKernelGGL((permute_kernel<T, true>), grid, block, smem, st, (const T*)src,     \
-                           st3[0], st3[1], st3[2], (T*)dst, (T*)pooled, tile_valid, g, Hn, D, eo, ne, row_table, tile_table); \
+                           st3[0], st3[1], st3[2], (T*)dst, (T*)pooled, tile_valid, g, Hn, D, eo, ne, row_table, tile_table, \
+                           (const T*)src2, s2[0], s2[1], s2[2], (T*)dst2); \
     else                                                                                       \
         hipLaunchKernelGGL((permute_kernel<T, false>), grid, block, smem, st, (const T*)src,    \
-                           st3[0], st3[1], st3[2], (T*)dst, (T*)pooled, tile_valid, g, Hn, D, eo, ne, row_table, tile_table);
+                           st3[0], st3[1], st3[2], (T*)dst, (T*)pooled, tile_valid, g, Hn, D, eo, ne, row_table, tile_table, \
+                           (const T*)src2, s2[0], s2[1], s2[2], (T*)dst2);
     if (dtype == BSA_BF16) { BSA_LAUNCH(__bf16) }
     else if (dtype == BSA_F16) { BSA_LAUNCH(_Float16) }
     else { BSA_LAUNCH(float) }
