@@ -1,6 +1,6 @@
 """Benchmark of the block-sparse attention forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5]
 
 A step is one pass of the whole operator (chunk mean pooling of q and k, pooled
 scores, top-k, block-sparse flash attention that gathers its tiles from the
@@ -113,12 +113,83 @@ def cpu_baseline(torch, latent, sparsity, seed, rms, budget_s):
     }
 
 
+def run_c4(torch, args):
+    """BASELINE config 4: long-video continuation, grid 48x30x52 with 12 conditioning frames.  Two operator
+    calls per layer as in attention.py:124-135, writing into one output buffer."""
+    from longcat_video_amd.block_sparse_attention import bsa_interface as I
+    T, Hh, W, cond = 48, 30, 52, 12
+    S, n = T * Hh * W, cond * Hh * W
+    q, k, v = make_inputs(torch, (T, Hh, W), 3, False)
+    out = torch.empty(1, S, HEADS, D, dtype=torch.bfloat16, device="cuda").permute(0, 2, 1, 3)
+
+    def step():
+        I._bsa_3d(q[:, :, :n], k[:, :, :n], v[:, :, :n], (cond, Hh, W), (cond, Hh, W), 0.875, CHUNK, CHUNK, out=out[:, :, :n])
+        I._bsa_3d(q[:, :, n:], k, v, (T - cond, Hh, W), (T, Hh, W), 0.875, CHUNK, CHUNK, out=out[:, :, n:])
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    pairs = HEADS * (312 * 39 + 936 * 156)
+    flop = pairs * 4 * 64 * 64 * D
+    print(json.dumps({
+        "metric": "BSA fwd ms/layer + sparse TFLOPS, long-video continuation (cond/noise split)", "value": round(flop / ms / 1e9, 2),
+        "unit": "TFLOP/s (sparse-actual, both operator calls)", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic N(0,1) q/k/v, seeded on the GPU",
+        "config": {"workload": "c4: 32 heads x 128, grid 48x30x52 (74880 tokens), 12 conditioning frames, density 1/8",
+                   "block_pairs": pairs},
+        "pct_of_bf16_peak_whole_operator": round(100 * flop / ms / 1e9 / PEAK_BF16_TFLOPS, 2)}))
+
+
+def run_c5(torch, args):
+    """BASELINE config 5: the attention sub-chain of one DiT block at 720p: RMSNorm -> QKV projection ->
+    per-head RMSNorm + 3-D RoPE -> block-sparse attention -> output projection + residual (dim 4096)."""
+    from longcat_video_amd.modules import attention as M
+    latent = WORKLOADS["c3"][0]
+    N, C = latent[0] * latent[1] * latent[2], HEADS * D
+    g = torch.Generator(device="cuda").manual_seed(4)
+    x = torch.randn(1, N, C, generator=g, device="cuda").bfloat16()
+    attn = M.Attention(C, HEADS, enable_bsa=True,
+                       bsa_params=dict(sparsity=0.9375, chunk_3d_shape_q=list(CHUNK), chunk_3d_shape_k=list(CHUNK))).cuda().bfloat16()
+    for prm in attn.parameters():
+        prm.data = (torch.randn(prm.shape, generator=g, device="cuda") * 0.02).bfloat16() if prm.dim() > 1 else torch.zeros_like(prm)
+    attn.q_norm.weight.data.fill_(1.0)
+    attn.k_norm.weight.data.fill_(1.0)
+    w_pre = torch.ones(C, dtype=torch.bfloat16, device="cuda")
+    for _ in range(args.warmup):
+        M.attention_block_forward(x, w_pre, attn, latent)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        y = M.attention_block_forward(x, w_pre, attn, latent)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    assert torch.isfinite(y.float()).all()
+    bsa_flop = HEADS * 1440 * 90 * 4 * 64 * 64 * D
+    gemm_flop = 2 * N * C * 3 * C + 2 * N * C * C
+    ms_qkv = time_events(torch, lambda: M.linear_bf16(x, attn.qkv.weight, attn.qkv.bias), 5, 2)
+    print(json.dumps({
+        "metric": "attention sub-chain of a DiT block, ms/layer + TFLOPS (GEMMs + sparse-actual attention)",
+        "value": round((bsa_flop + gemm_flop) / ms / 1e9, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic N(0,1) activations, N(0,0.02) weights, zero biases, unit norm weights",
+        "config": {"workload": "c5: x [1, 86400, 4096] bf16, 32 heads x 128, grid 24x45x80, density 1/16"},
+        "qkv_gemm_ms": round(ms_qkv, 4), "qkv_gemm_tflops": round(2 * N * C * 3 * C / ms_qkv / 1e9, 1),
+        "pct_of_bf16_peak": round(100 * (bsa_flop + gemm_flop) / ms / 1e9 / PEAK_BF16_TFLOPS, 2)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4", "c5"],
+                    help="c3 is the headline (default); c2 the same operator at 480p; c4 and c5 print a reduced line "
+                         "for the cond/noise split and for the attention module")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the CPU baseline's attention sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -132,6 +203,10 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (there is no CPU path to measure)")
     torch.cuda.set_device(0)
+    if args.workload == "c4":
+        return run_c4(torch, args)
+    if args.workload == "c5":
+        return run_c5(torch, args)
     latent, sparsity, seed, rms, desc = WORKLOADS[args.workload]
     q, k, v = make_inputs(torch, latent, seed, rms)
     prm = dict(sparsity=sparsity, chunk_3d_shape_q=list(CHUNK), chunk_3d_shape_k=list(CHUNK))

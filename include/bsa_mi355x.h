@@ -220,8 +220,9 @@ int bsa_qk_norm_rope(void* q, const int64_t q_strides[3], void* k, const int64_t
                      int B, int Hn, int T, int H, int W, int D, float eps, int dtype, void* stream);
 
 /* out[M,N] = x[M,K] . w[N,K]^T (+ bias[N]) (+ residual[M,N]), bf16 in/out, fp32 accumulate, on MFMA
- * through hipBLASLt.  Replaces the nn.Linear calls attention.py:111 and :142.  `workspace` may be
- * null with workspace_bytes 0.  Creates one process-wide hipBLASLt handle on first use. */
+ * through hipBLASLt.  Replaces the nn.Linear calls attention.py:111 and :142.  `workspace`: at least
+ * 32 MiB of device memory (BSA_ERR_WORKSPACE otherwise); its contents do not matter.  Creates one
+ * process-wide hipBLASLt handle on first use. */
 int bsa_linear_bf16(const void* x, const void* w, const void* bias, const void* residual, void* out,
                     int64_t M, int N, int K, void* workspace, size_t workspace_bytes, void* stream);
 

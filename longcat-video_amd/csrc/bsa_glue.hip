@@ -166,7 +166,10 @@ int bsa_linear_bf16(const void* x, const void* w, const void* bias, const void* 
                     int K, void* workspace, size_t workspace_bytes, void* stream) {
     if (!x || !w || !out) return set_error(BSA_ERR_BAD_ARG, "linear: null pointer");
     if (M <= 0 || N <= 0 || K <= 0) return set_error(BSA_ERR_BAD_ARG, "linear: sizes must be positive");
-    if (workspace_bytes > 0 && !workspace) return set_error(BSA_ERR_BAD_ARG, "linear: workspace is null");
+    // hipBLASLt has been seen to write through the workspace pointer for large problems even when it was
+    // told that there is none, so a workspace is mandatory
+    if (!workspace || workspace_bytes < ((size_t)32 << 20))
+        return set_error(BSA_ERR_WORKSPACE, "linear: a workspace of at least 32 MiB is required (got %zu bytes)", workspace_bytes);
     LtState& st = lt_state();
     std::lock_guard<std::mutex> lock(st.mu);
     if (!st.handle && hipblasLtCreate(&st.handle) != HIPBLAS_STATUS_SUCCESS)
@@ -200,12 +203,15 @@ int bsa_linear_bf16(const void* x, const void* w, const void* bias, const void* 
         BSA_LT(hipblasLtMatmulPreferenceCreate(&pref));
         const uint64_t wsb = workspace_bytes;
         BSA_LT(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &wsb, sizeof(wsb)));
-        hipblasLtMatmulHeuristicResult_t heur;
-        int found = 0;
-        BSA_LT(hipblasLtMatmulAlgoGetHeuristic(st.handle, desc, la, lb, lc, lc, pref, 1, &heur, &found));
-        if (found == 0) { rc = set_error(BSA_ERR_UNSUPPORTED, "linear: no GEMM algorithm for M=%lld N=%d K=%d", (long long)M, N, K); goto done; }
+        hipblasLtMatmulHeuristicResult_t heur[8];
+        int found = 0, pick = -1;
+        BSA_LT(hipblasLtMatmulAlgoGetHeuristic(st.handle, desc, la, lb, lc, lc, pref, 8, heur, &found));
+        // never hand the library less workspace than the algorithm says it uses
+        for (int i = 0; i < found && pick < 0; ++i)
+            if (heur[i].state == HIPBLAS_STATUS_SUCCESS && heur[i].workspaceSize <= workspace_bytes) pick = i;
+        if (pick < 0) { rc = set_error(BSA_ERR_UNSUPPORTED, "linear: no GEMM algorithm for M=%lld N=%d K=%d within %zu bytes of workspace", (long long)M, N, K, workspace_bytes); goto done; }
         BSA_LT(hipblasLtMatmul(st.handle, desc, &alpha, w, la, x, lb, &beta, residual ? residual : out, lc, out, lc,
-                               &heur.algo, workspace, workspace_bytes, (hipStream_t)stream));
+                               &heur[pick].algo, workspace, workspace_bytes, (hipStream_t)stream));
     }
 done:
     if (pref) hipblasLtMatmulPreferenceDestroy(pref);

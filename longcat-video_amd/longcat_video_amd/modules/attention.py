@@ -59,7 +59,8 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
 
 
 def linear_bf16(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
-                residual: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                residual: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ weight.T + bias (+ residual)`` for bf16 tensors, weight in nn.Linear layout [out, in]."""
     if not x.is_cuda:
         raise RuntimeError("the engine runs on the GPU only")
@@ -71,7 +72,9 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
     x2 = x.reshape(-1, K).contiguous()
     w = weight.to(torch.bfloat16).contiguous()
     b = None if bias is None else bias.to(torch.bfloat16).contiguous()
-    out = torch.empty(x2.shape[0], N, dtype=torch.bfloat16, device=x.device)
+    if out is None:
+        out = torch.empty(x2.shape[0], N, dtype=torch.bfloat16, device=x.device)
+    assert out.shape == (x2.shape[0], N) and out.dtype == torch.bfloat16 and out.is_contiguous()
     r = None
     if residual is not None:
         r = residual.reshape(-1, N).contiguous()
