@@ -219,6 +219,19 @@ int bsa_qk_norm_rope(void* q, const int64_t q_strides[3], void* k, const int64_t
                      const void* q_weight, const void* k_weight, const float* rope_table,
                      int B, int Hn, int T, int H, int W, int D, float eps, int dtype, void* stream);
 
+/* One tensor of the same chain, with every step optional and an optional move to another layout:
+ *   dst = rope(norm(src)).  weight == NULL skips the RMSNorm, rope_table == NULL skips the rotation, both
+ *   NULL copies.  src / dst [B, Hn, T*H*W, 128] with element strides {B, Hn, S}; src == dst with equal
+ *   strides works in place.  The token at grid position (t, h, w) is rotated by frame t_offset + t of a
+ *   table built for table_T frames (layout as in bsa_qk_norm_rope with T = table_T).
+ * Serves the plain forward (q, k, v moved from the token-major projection output into per-head contiguous
+ * tensors while q and k are normalised and rotated), return_kv (attention.py:118-119: k after the norm,
+ * before the rotation) and forward_with_kv_cache (attention.py:166-171: cached keys and new queries are
+ * rotated on a grid of T + num_cond_latents frames, the queries starting at frame num_cond_latents). */
+int bsa_norm_rope(const void* src, const int64_t src_strides[3], void* dst, const int64_t dst_strides[3],
+                  const void* weight, const float* rope_table, int B, int Hn, int T, int H, int W,
+                  int t_offset, int table_T, int D, float eps, int dtype, void* stream);
+
 /* out[M,N] = x[M,K] . w[N,K]^T (+ bias[N]) (+ residual[M,N]), bf16 in/out, fp32 accumulate, on MFMA
  * through hipBLASLt.  Replaces the nn.Linear calls attention.py:111 and :142.  `workspace`: at least
  * 32 MiB of device memory (BSA_ERR_WORKSPACE otherwise); its contents do not matter.  Creates one

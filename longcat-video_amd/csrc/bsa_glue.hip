@@ -42,65 +42,82 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* __restrict__
     }
 }
 
-// ------------------------------------------------- per-head QK RMSNorm + RoPE
+// ------------------------------------------------- per-head RMSNorm + RoPE
 // One row = one (token, head) vector of D = 128 elements, handled by 16 lanes
 // (8 elements each, i.e. 4 interleaved rotation pairs per lane).
 // x -> bf16(x * rsqrt(mean(x^2)+eps)) -> bf16(. * w) -> fp32 x*cos + rot(x)*sin -> bf16
 // with rot(x)[2i] = -x[2i+1], rot(x)[2i+1] = x[2i]; the d axis is split
 // (t: D - 4*(D/6), h: 2*(D/6), w: 2*(D/6)) and pair i of an axis turns by pos * freq_i.
-// tab holds cos_t[T][nt], sin_t[T][nt], cos_h[H][nh], sin_h[H][nh], cos_w[W][nw], sin_w[W][nw] (fp32).
+// tab holds cos_t[Ttab][nt], sin_t[Ttab][nt], cos_h[H][nh], sin_h[H][nh], cos_w[W][nw], sin_w[W][nw]
+// (fp32); the token at grid position (ti, hi, wi) uses row t0 + ti of the t tables.
+// Either step can be left out (w == nullptr: no norm; tab == nullptr: no rotation), and the result
+// may go to another tensor with other strides, so the same pass also moves q, k, v from the
+// token-major layout of the QKV projection into per-head contiguous tensors.
+// head_fastest: consecutive rows walk the heads of one token (the order in which a token-major
+// source lies in memory); otherwise the tokens of one head.
 template <typename T>
-__global__ __launch_bounds__(256) void qk_norm_rope_kernel(T* __restrict__ q, int64_t qsB, int64_t qsH, int64_t qsS,
-                                                           T* __restrict__ k, int64_t ksB, int64_t ksH, int64_t ksS,
-                                                           const T* __restrict__ qw, const T* __restrict__ kw,
-                                                           const float* __restrict__ tab, int B, int Hn, int Tn,
-                                                           int Hg, int Wg, float eps) {
+__global__ __launch_bounds__(256) void norm_rope_kernel(const T* __restrict__ src, int64_t sB, int64_t sH, int64_t sS,
+                                                        T* __restrict__ dst, int64_t dB, int64_t dH, int64_t dS,
+                                                        const T* __restrict__ w, const float* __restrict__ tab, int B,
+                                                        int Hn, int Tn, int Hg, int Wg, int t0, int Ttab, float eps,
+                                                        int head_fastest) {
     constexpr int D = 128;
     constexpr int nt = (D - 4 * (D / 6)) / 2, nh = (D / 6), nw = (D / 6);   // pairs per axis: 22, 21, 21
     const int sub = threadIdx.x & 15;
     const int64_t S = (int64_t)Tn * Hg * Wg;
-    const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);      // over B*Hn*S rows, and q then k
-    const int64_t nrows = (int64_t)B * Hn * S;
-    if (row >= 2 * nrows) return;
-    const bool is_k = row >= nrows;
-    const int64_t r = is_k ? row - nrows : row;
-    const int64_t s = r % S;
-    const int hd = (int)((r / S) % Hn), b = (int)(r / (S * Hn));
-    T* p = is_k ? k + b * ksB + hd * ksH + s * ksS : q + b * qsB + hd * qsH + s * qsS;
-    const T* wv = is_k ? kw : qw;
-    const int wi = (int)(s % Wg), hi = (int)((s / Wg) % Hg), ti = (int)(s / ((int64_t)Wg * Hg));
+    const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    if (row >= (int64_t)B * Hn * S) return;
+    int64_t s;
+    int hd, b;
+    if (head_fastest) { hd = (int)(row % Hn); s = (row / Hn) % S; b = (int)(row / (S * Hn)); }
+    else { s = row % S; hd = (int)((row / S) % Hn); b = (int)(row / (S * Hn)); }
+    const T* p = src + b * sB + hd * sH + s * sS;
+    T* o = dst + b * dB + hd * dH + s * dS;
 
     const uint4 raw = *reinterpret_cast<const uint4*>(p + sub * 8);
-    const uint4 wraw = *reinterpret_cast<const uint4*>(wv + sub * 8);
-    const T* e = reinterpret_cast<const T*>(&raw);
-    const T* we = reinterpret_cast<const T*>(&wraw);
-    float f[8];
-    float ss = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) { f[i] = (float)e[i]; ss = fmaf(f[i], f[i], ss); }
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
-    const float rs = rsqrtf(ss / (float)D + eps);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = (float)(T)((float)(T)(f[i] * rs) * (float)we[i]);
-
-    const float* cos_t = tab;                 const float* sin_t = cos_t + (int64_t)Tn * nt;
-    const float* cos_h = sin_t + (int64_t)Tn * nt; const float* sin_h = cos_h + (int64_t)Hg * nh;
-    const float* cos_w = sin_h + (int64_t)Hg * nh; const float* sin_w = cos_w + (int64_t)Wg * nw;
-    T res[8];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int pair = sub * 4 + j;          // 0..63
-        float c, sn;
-        if (pair < nt) { c = cos_t[ti * nt + pair]; sn = sin_t[ti * nt + pair]; }
-        else if (pair < nt + nh) { c = cos_h[hi * nh + pair - nt]; sn = sin_h[hi * nh + pair - nt]; }
-        else { c = cos_w[wi * nw + pair - nt - nh]; sn = sin_w[wi * nw + pair - nt - nh]; }
-        const float x0 = f[2 * j], x1 = f[2 * j + 1];
-        // two products, then one add, each rounded: the order of operations of the eager expression
-        res[2 * j] = (T)__fadd_rn(__fmul_rn(x0, c), __fmul_rn(-x1, sn));
-        res[2 * j + 1] = (T)__fadd_rn(__fmul_rn(x1, c), __fmul_rn(x0, sn));
+    if (w == nullptr && tab == nullptr) {                 // plain move
+        *reinterpret_cast<uint4*>(o + sub * 8) = raw;
+        return;
     }
-    *reinterpret_cast<uint4*>(p + sub * 8) = *reinterpret_cast<const uint4*>(res);
+    const T* e = reinterpret_cast<const T*>(&raw);
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = (float)e[i];
+    if (w != nullptr) {
+        const uint4 wraw = *reinterpret_cast<const uint4*>(w + sub * 8);
+        const T* we = reinterpret_cast<const T*>(&wraw);
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+        const float rs = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (float)(T)((float)(T)(f[i] * rs) * (float)we[i]);
+    }
+    T res[8];
+    if (tab != nullptr) {
+        const int wi = (int)(s % Wg), hi = (int)((s / Wg) % Hg), ti = t0 + (int)(s / ((int64_t)Wg * Hg));
+        const float* cos_t = tab;                        const float* sin_t = cos_t + (int64_t)Ttab * nt;
+        const float* cos_h = sin_t + (int64_t)Ttab * nt; const float* sin_h = cos_h + (int64_t)Hg * nh;
+        const float* cos_w = sin_h + (int64_t)Hg * nh;   const float* sin_w = cos_w + (int64_t)Wg * nw;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int pair = sub * 4 + j;          // 0..63
+            float c, sn;
+            if (pair < nt) { c = cos_t[ti * nt + pair]; sn = sin_t[ti * nt + pair]; }
+            else if (pair < nt + nh) { c = cos_h[hi * nh + pair - nt]; sn = sin_h[hi * nh + pair - nt]; }
+            else { c = cos_w[wi * nw + pair - nt - nh]; sn = sin_w[wi * nw + pair - nt - nh]; }
+            const float x0 = f[2 * j], x1 = f[2 * j + 1];
+            // two products, then one add, each rounded: the order of operations of the eager expression
+            res[2 * j] = (T)__fadd_rn(__fmul_rn(x0, c), __fmul_rn(-x1, sn));
+            res[2 * j + 1] = (T)__fadd_rn(__fmul_rn(x1, c), __fmul_rn(x0, sn));
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) res[i] = (T)f[i];
+    }
+    *reinterpret_cast<uint4*>(o + sub * 8) = *reinterpret_cast<const uint4*>(res);
 }
 
 // ------------------------------------------------------------- linear (GEMM)
@@ -134,32 +151,46 @@ int bsa_rmsnorm(const void* x, const void* weight, void* out, int64_t rows, int 
     return e == hipSuccess ? BSA_OK : set_error(BSA_ERR_HIP, "rmsnorm launch: %s", hipGetErrorString(e));
 }
 
+int bsa_norm_rope(const void* src, const int64_t src_strides[3], void* dst, const int64_t dst_strides[3],
+                  const void* weight, const float* rope_table, int B, int Hn, int T, int H, int W, int t_offset,
+                  int table_T, int D, float eps, int dtype, void* stream) {
+    if (!src || !dst || !src_strides || !dst_strides) return set_error(BSA_ERR_BAD_ARG, "norm_rope: null pointer");
+    if (D != 128) return set_error(BSA_ERR_UNSUPPORTED, "norm_rope: head dim %d is not built (only 128)", D);
+    if (B <= 0 || Hn <= 0 || T <= 0 || H <= 0 || W <= 0) return set_error(BSA_ERR_BAD_ARG, "norm_rope: sizes must be positive");
+    if (rope_table && (t_offset < 0 || table_T < t_offset + T))
+        return set_error(BSA_ERR_SHAPE, "norm_rope: frames %d..%d lie outside a table of %d frames", t_offset, t_offset + T, table_T);
+    for (int i = 0; i < 3; ++i)
+        if (src_strides[i] < 0 || dst_strides[i] < 0 || (src_strides[i] * 2) % 16 || (dst_strides[i] * 2) % 16)
+            return set_error(BSA_ERR_BAD_ARG, "norm_rope: strides must keep rows 16-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(weight)) & 15u)
+        return set_error(BSA_ERR_BAD_ARG, "norm_rope: pointers must be 16-byte aligned");
+    if (!(eps >= 0.f)) return set_error(BSA_ERR_BAD_ARG, "norm_rope: eps must be non-negative");
+    const int64_t rows = (int64_t)B * Hn * T * H * W;
+    if ((rows + 15) / 16 > 0x7fffffffLL) return set_error(BSA_ERR_UNSUPPORTED, "norm_rope: too many rows");
+    const dim3 grid((unsigned)((rows + 15) / 16)), block(256);
+    const int head_fastest = src_strides[1] < src_strides[2] ? 1 : 0;
+    if (dtype == BSA_BF16)
+        hipLaunchKernelGGL((norm_rope_kernel<__bf16>), grid, block, 0, (hipStream_t)stream, (const __bf16*)src, src_strides[0],
+                           src_strides[1], src_strides[2], (__bf16*)dst, dst_strides[0], dst_strides[1], dst_strides[2],
+                           (const __bf16*)weight, rope_table, B, Hn, T, H, W, t_offset, table_T, eps, head_fastest);
+    else if (dtype == BSA_F16)
+        hipLaunchKernelGGL((norm_rope_kernel<_Float16>), grid, block, 0, (hipStream_t)stream, (const _Float16*)src, src_strides[0],
+                           src_strides[1], src_strides[2], (_Float16*)dst, dst_strides[0], dst_strides[1], dst_strides[2],
+                           (const _Float16*)weight, rope_table, B, Hn, T, H, W, t_offset, table_T, eps, head_fastest);
+    else
+        return set_error(BSA_ERR_UNSUPPORTED, "norm_rope: dtype %d is not built (bf16, fp16)", dtype);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? BSA_OK : set_error(BSA_ERR_HIP, "norm_rope launch: %s", hipGetErrorString(e));
+}
+
 int bsa_qk_norm_rope(void* q, const int64_t q_strides[3], void* k, const int64_t k_strides[3], const void* q_weight,
                      const void* k_weight, const float* rope_table, int B, int Hn, int T, int H, int W, int D,
                      float eps, int dtype, void* stream) {
     if (!q || !k || !q_weight || !k_weight || !rope_table || !q_strides || !k_strides)
         return set_error(BSA_ERR_BAD_ARG, "qk_norm_rope: null pointer");
-    if (D != 128) return set_error(BSA_ERR_UNSUPPORTED, "qk_norm_rope: head dim %d is not built (only 128)", D);
-    if (B <= 0 || Hn <= 0 || T <= 0 || H <= 0 || W <= 0) return set_error(BSA_ERR_BAD_ARG, "qk_norm_rope: sizes must be positive");
-    for (int i = 0; i < 3; ++i)
-        if (q_strides[i] < 0 || k_strides[i] < 0 || (q_strides[i] * 2) % 16 || (k_strides[i] * 2) % 16)
-            return set_error(BSA_ERR_BAD_ARG, "qk_norm_rope: strides must keep rows 16-byte aligned");
-    if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(q_weight) |
-         reinterpret_cast<uintptr_t>(k_weight)) & 15u)
-        return set_error(BSA_ERR_BAD_ARG, "qk_norm_rope: pointers must be 16-byte aligned");
-    const int64_t rows = 2 * (int64_t)B * Hn * T * H * W;
-    if ((rows + 15) / 16 > 0x7fffffffLL) return set_error(BSA_ERR_UNSUPPORTED, "qk_norm_rope: too many rows");
-    const dim3 grid((unsigned)((rows + 15) / 16)), block(256);
-    if (dtype == BSA_BF16)
-        hipLaunchKernelGGL((qk_norm_rope_kernel<__bf16>), grid, block, 0, (hipStream_t)stream, (__bf16*)q, q_strides[0], q_strides[1], q_strides[2],
-                           (__bf16*)k, k_strides[0], k_strides[1], k_strides[2], (const __bf16*)q_weight, (const __bf16*)k_weight, rope_table, B, Hn, T, H, W, eps);
-    else if (dtype == BSA_F16)
-        hipLaunchKernelGGL((qk_norm_rope_kernel<_Float16>), grid, block, 0, (hipStream_t)stream, (_Float16*)q, q_strides[0], q_strides[1], q_strides[2],
-                           (_Float16*)k, k_strides[0], k_strides[1], k_strides[2], (const _Float16*)q_weight, (const _Float16*)k_weight, rope_table, B, Hn, T, H, W, eps);
-    else
-        return set_error(BSA_ERR_UNSUPPORTED, "qk_norm_rope: dtype %d is not built (bf16, fp16)", dtype);
-    const hipError_t e = hipGetLastError();
-    return e == hipSuccess ? BSA_OK : set_error(BSA_ERR_HIP, "qk_norm_rope launch: %s", hipGetErrorString(e));
+    const int rc = bsa_norm_rope(q, q_strides, q, q_strides, q_weight, rope_table, B, Hn, T, H, W, 0, T, D, eps, dtype, stream);
+    if (rc != BSA_OK) return rc;
+    return bsa_norm_rope(k, k_strides, k, k_strides, k_weight, rope_table, B, Hn, T, H, W, 0, T, D, eps, dtype, stream);
 }
 
 int bsa_linear_bf16(const void* x, const void* w, const void* bias, const void* residual, void* out, int64_t M, int N,

@@ -11,11 +11,13 @@ C-ABI of the engine:
     block-sparse attention               bsa_fwd_3d        (attention.py:58-67, :124-137)
     x = Linear(o)                        bsa_linear_bf16   (attention.py:139-142)
 
-q, k, v stay strided views of the projection output and the attention output is
-written token-major, so none of the reference's ``.contiguous()`` / transpose
-copies (attention.py:127-135, :140-141) exist here.  Only the block-sparse branch
-is built: dense back ends (flash-attn, xformers) and the KV-cache variant
-(attention.py:149-181) raise ``NotImplementedError``.
+q, k and v are moved from the token-major projection output into per-head
+contiguous tensors by the same pass that normalises and rotates q and k (the
+attention kernel fetches K/V tiles faster from 256-byte-dense heads than from
+rows 24 KB apart), and the attention output is written token-major, so none of
+the reference's ``.contiguous()`` / ``cat`` / transpose copies (attention.py:127-135,
+:140-141, :166-171) exist here.  Only the block-sparse branch is built: dense back
+ends (flash-attn, xformers) raise ``NotImplementedError``.
 """
 from __future__ import annotations
 
@@ -126,6 +128,31 @@ def qk_norm_rope_(q: torch.Tensor, k: torch.Tensor, q_weight, k_weight, grid_siz
             _ptr(tab), B, H, T, Hg, Wg, D, float(eps), code, _stream(q)), "qk_norm_rope")
 
 
+def norm_rope(src: torch.Tensor, dst: torch.Tensor, weight=None, grid_size=None, eps: float = 1e-6,
+              t_offset: int = 0, table_grid=None) -> torch.Tensor:
+    """dst = rope(norm(src)) on [B,H,S,128] tensors or views (contiguous D); `weight` None skips the RMSNorm,
+    `grid_size` None skips the rotation, both None copies.  `table_grid`: the grid the rotation angles are
+    laid out on when src covers only the frames t_offset .. t_offset + T of it."""
+    B, H, S, D = src.shape
+    assert dst.shape == src.shape and dst.dtype == src.dtype and src.stride(3) == 1 and dst.stride(3) == 1
+    code = {torch.bfloat16: _capi.BSA_BF16, torch.float16: _capi.BSA_F16}.get(src.dtype)
+    if code is None:
+        raise NotImplementedError("norm_rope: dtype %s is not built (bf16, fp16)" % src.dtype)
+    tab, T, Hg, Wg, table_T = None, S, 1, 1, S
+    if grid_size is not None:
+        T, Hg, Wg = (int(g) for g in grid_size)
+        assert S == T * Hg * Wg
+        table_grid = tuple(int(g) for g in (table_grid if table_grid is not None else grid_size))
+        assert table_grid[1:] == (Hg, Wg)
+        tab, table_T = rope_table(table_grid, D, src.device), table_grid[0]
+    w = None if weight is None else weight.to(src.dtype).contiguous()
+    with torch.cuda.device(src.device):
+        _capi.check(_capi.load().bsa_norm_rope(
+            _ptr(src), _capi.strides3(src.stride()[:3]), _ptr(dst), _capi.strides3(dst.stride()[:3]), _ptr(w), _ptr(tab),
+            B, H, T, Hg, Wg, int(t_offset), table_T, D, float(eps), code, _stream(src)), "norm_rope")
+    return dst
+
+
 class Attention(nn.Module):
     def __init__(
         self,
@@ -176,17 +203,27 @@ class Attention(nn.Module):
         return _bsa_3d(q, k, v, (Tq, Hh, W), (Tk, Hh, W), float(prm["sparsity"]), prm["chunk_3d_shape_q"],
                        prm["chunk_3d_shape_k"], out=out)
 
+    def _project_qkv(self, x):
+        B, N, C = x.shape
+        qkv = linear_bf16(x, self.qkv.weight, self.qkv.bias)                      # [B, N, 3C]
+        return qkv.view(B, N, 3, self.num_heads, self.head_dim).permute(2, 0, 3, 1, 4).unbind(0)   # strided [B,H,N,D] views
+
     @torch.no_grad()
     def forward(self, x: torch.Tensor, shape=None, num_cond_latents=None, return_kv=False,
-                residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+                residual: Optional[torch.Tensor] = None):
         """attention.py:107-147.  `residual` (extension): added to the projection output inside the GEMM."""
-        if return_kv:
-            raise NotImplementedError("the KV-cache variant is not built")
         B, N, C = x.shape
         Hn, D = self.num_heads, self.head_dim
-        qkv = linear_bf16(x, self.qkv.weight, self.qkv.bias)                      # [B, N, 3C]
-        q, k, v = qkv.view(B, N, 3, Hn, D).permute(2, 0, 3, 1, 4).unbind(0)       # strided [B, H, N, D] views
-        qk_norm_rope_(q, k, self.q_norm.weight, self.k_norm.weight, shape, self.q_norm.eps)
+        qs, ks, vs = self._project_qkv(x)
+        new = lambda: torch.empty(B, Hn, N, D, dtype=x.dtype, device=x.device)
+        eps = self.q_norm.eps
+        q = norm_rope(qs, new(), self.q_norm.weight, shape, eps=eps)
+        v = norm_rope(vs, new())                                                  # plain move
+        if return_kv:
+            k_cache = norm_rope(ks, new(), self.k_norm.weight, eps=eps)           # attention.py:118-119
+            k = norm_rope(k_cache, new(), None, shape)
+        else:
+            k = norm_rope(ks, new(), self.k_norm.weight, shape, eps=eps)
 
         o = torch.empty(B, N, Hn, D, dtype=x.dtype, device=x.device)             # token-major: reshape below is free
         ov = o.permute(0, 2, 1, 3)                                                # [B, H, N, D] view
@@ -196,10 +233,44 @@ class Attention(nn.Module):
             self._process_attn(q[:, :, n:], k, v, shape, out=ov[:, :, n:])                       # attention.py:132-133
         else:
             self._process_attn(q, k, v, shape, out=ov)
-        return linear_bf16(o.view(B, N, C), self.proj.weight, self.proj.bias, residual=residual)
+        y = linear_bf16(o.view(B, N, C), self.proj.weight, self.proj.bias, residual=residual)
+        if return_kv:
+            return y, (k_cache, v.clone())
+        return y
 
-    def forward_with_kv_cache(self, *args, **kwargs):
-        raise NotImplementedError("the KV-cache variant (attention.py:149-181) is not built")
+    @torch.no_grad()
+    def forward_with_kv_cache(self, x: torch.Tensor, shape=None, num_cond_latents=None, kv_cache=None,
+                              residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """attention.py:149-181: the new tokens attend to the cached conditioning keys/values followed by
+        their own.  The cache holds keys after the norm and before the rotation; cached and new keys are
+        rotated together on a grid of T + num_cond_latents frames, the queries sit at its last T frames."""
+        B, N, C = x.shape
+        Hn, D = self.num_heads, self.head_dim
+        T, Hg, Wg = (int(g) for g in shape)
+        k_cache, v_cache = kv_cache
+        assert k_cache.shape[0] == v_cache.shape[0] and k_cache.shape[0] in [1, B]
+        if not (num_cond_latents is not None and num_cond_latents > 0):
+            # the reference leaves k_full undefined on this path (attention.py:165-173)
+            raise ValueError("forward_with_kv_cache needs num_cond_latents > 0")
+        n_c = k_cache.shape[2]
+        assert n_c == num_cond_latents * Hg * Wg and N == T * Hg * Wg
+        qs, ks, vs = self._project_qkv(x)
+        eps = self.q_norm.eps
+        grid_full = (T + num_cond_latents, Hg, Wg)
+        k_full = torch.empty(B, Hn, n_c + N, D, dtype=x.dtype, device=x.device)
+        v_full = torch.empty_like(k_full)
+        kc = k_cache.to(x.device).expand(B, -1, -1, -1)                            # attention.py:162-164
+        vc = v_cache.to(x.device).expand(B, -1, -1, -1)
+        # cached keys: rotation only, frames 0 .. num_cond; new keys: norm + rotation at frames num_cond ..
+        norm_rope(kc, k_full[:, :, :n_c], None, (num_cond_latents, Hg, Wg), table_grid=grid_full)
+        norm_rope(ks, k_full[:, :, n_c:], self.k_norm.weight, shape, eps=eps, t_offset=num_cond_latents, table_grid=grid_full)
+        norm_rope(vc, v_full[:, :, :n_c])
+        norm_rope(vs, v_full[:, :, n_c:])
+        q = norm_rope(qs, torch.empty(B, Hn, N, D, dtype=x.dtype, device=x.device), self.q_norm.weight, shape, eps=eps,
+                      t_offset=num_cond_latents, table_grid=grid_full)
+        o = torch.empty(B, N, Hn, D, dtype=x.dtype, device=x.device)
+        self._process_attn(q, k_full, v_full, shape, out=o.permute(0, 2, 1, 3))
+        return linear_bf16(o.view(B, N, C), self.proj.weight, self.proj.bias, residual=residual)
 
 
 @torch.no_grad()

@@ -413,3 +413,38 @@ def attention_module_forward(x, w_qkv, b_qkv, w_proj, b_proj, q_norm_w, k_norm_w
         o, *_ = flash_attn_bsa_3d(q, k, v, shape, shape, **bsa_params)
     o = o.to(dt).transpose(1, 2).reshape(B, N, C)
     return (o.float() @ w_proj.float().t() + b_proj.float()).to(dt)
+
+
+def attention_module_kv(x, w_qkv, b_qkv, q_norm_w, k_norm_w, num_heads: int):
+    """attn:110-119 with return_kv: the cache holds k after the RMSNorm and before the rotation, and v."""
+    B, N, C = x.shape
+    D = C // num_heads
+    qkv = (x.float() @ w_qkv.float().t() + b_qkv.float()).to(x.dtype)
+    _, k, v = qkv.view(B, N, 3, num_heads, D).permute(2, 0, 3, 1, 4).unbind(0)
+    return rms_norm_fp32(k, k_norm_w).clone(), v.clone()
+
+
+def attention_module_forward_with_kv_cache(x, w_qkv, b_qkv, w_proj, b_proj, q_norm_w, k_norm_w, shape,
+                                           num_heads: int, bsa_params: dict, num_cond_latents: int, kv_cache):
+    """attn:149-181 (Attention.forward_with_kv_cache), BSA branch.  x holds the T*H*W new tokens; the
+    cache holds num_cond_latents frames.  Keys: cat(cache, new) rotated on a grid of T + num_cond frames
+    (attn:166-170); queries: the last N positions of that grid (attn:168-171); attention with
+    Tq = T and Tk = T + num_cond (attn:173, 60-61)."""
+    B, N, C = x.shape
+    D = C // num_heads
+    dt = x.dtype
+    T, Hh, W = shape
+    qkv = (x.float() @ w_qkv.float().t() + b_qkv.float()).to(dt)
+    q, k, v = qkv.view(B, N, 3, num_heads, D).permute(2, 0, 3, 1, 4).unbind(0)
+    q, k = rms_norm_fp32(q, q_norm_w), rms_norm_fp32(k, k_norm_w)
+    k_cache, v_cache = kv_cache
+    if k_cache.shape[0] == 1:
+        k_cache, v_cache = k_cache.repeat(B, 1, 1, 1), v_cache.repeat(B, 1, 1, 1)
+    k_full = torch.cat([k_cache, k], dim=2)
+    v_full = torch.cat([v_cache, v], dim=2)
+    ang = rope_3d_angles((T + num_cond_latents, Hh, W), D)
+    k_full = rope_3d_apply(k_full, ang)
+    q = rope_3d_apply(q, ang[-N:])
+    o, *_ = flash_attn_bsa_3d(q, k_full, v_full, (T, Hh, W), (T + num_cond_latents, Hh, W), **bsa_params)
+    o = o.to(dt).transpose(1, 2).reshape(B, N, C)
+    return (o.float() @ w_proj.float().t() + b_proj.float()).to(dt)

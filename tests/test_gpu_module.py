@@ -142,13 +142,70 @@ def test_attention_block_with_pre_norm_and_residual():
     assert d.max() <= 4e-2 and d.mean() <= 4e-3, (d.max(), d.mean())
 
 
+def test_return_kv_and_forward_with_kv_cache():
+    """attention.py:118-119 and :149-181: a first pass over the conditioning frames returns the cache
+    (keys after the norm, before the rotation); a second pass over the new frames attends to cache + new."""
+    cond, T, Hh, W = 4, 8, 8, 8
+    m = make_module(sparsity=0.5, seed=9)
+    g = torch.Generator().manual_seed(10)
+    x_cond = torch.randn(1, cond * Hh * W, 512, generator=g).bfloat16()
+    x_new = torch.randn(2, T * Hh * W, 512, generator=g).bfloat16()      # the cache of batch 1 serves batch 2
+    sd = {k: v.detach().cpu() for k, v in m.state_dict().items()}
+    prm = dict(sparsity=0.5, chunk_3d_shape_q=(4, 4, 4), chunk_3d_shape_k=(4, 4, 4))
+    mc = m.cuda()
+    y, (k_cache, v_cache) = mc(x_cond.cuda(), shape=(cond, Hh, W), return_kv=True)
+    assert torch.equal(y, mc(x_cond.cuda(), shape=(cond, Hh, W)))          # the cache is a by-product
+    want_k, want_v = O.attention_module_kv(x_cond, sd["qkv.weight"], sd["qkv.bias"], sd["q_norm.weight"],
+                                           sd["k_norm.weight"], m.num_heads)
+    assert k_cache.shape == (1, 4, cond * Hh * W, 128) and k_cache.is_contiguous()
+    dk = (k_cache.cpu().float() - want_k.float()).abs()
+    assert torch.all(dk <= want_k.float().abs() * 3 * BF16_ULP + 0.02) and (dk > 0).float().mean() < 0.05
+    dv = (v_cache.cpu().float() - want_v.float()).abs()
+    assert torch.all(dv <= want_v.float().abs() * BF16_ULP + 2e-3)
+    # second pass: judged against the oracle fed with the GPU's own cache
+    want = O.attention_module_forward_with_kv_cache(
+        x_new, sd["qkv.weight"], sd["qkv.bias"], sd["proj.weight"], sd["proj.bias"], sd["q_norm.weight"],
+        sd["k_norm.weight"], (T, Hh, W), m.num_heads, prm, cond, (k_cache.cpu(), v_cache.cpu()))
+    got = mc.forward_with_kv_cache(x_new.cuda(), shape=(T, Hh, W), num_cond_latents=cond, kv_cache=(k_cache, v_cache)).cpu()
+    assert got.shape == (2, T * Hh * W, 512)
+    d = (got.float() - want.float()).abs()
+    assert d.max() <= 2e-2 and d.mean() <= 2e-3, (d.max(), d.mean())
+
+
+def test_norm_rope_steps_and_frame_offset():
+    """bsa_norm_rope: each step alone, the move into another layout, and rotation of a slice of frames on
+    a larger grid (the position a new token gets in forward_with_kv_cache)."""
+    g = torch.Generator().manual_seed(11)
+    B, H, grid = 2, 3, (6, 4, 5)
+    S = grid[0] * grid[1] * grid[2]
+    x = torch.randn(B, S, H, 128, generator=g).bfloat16().permute(0, 2, 1, 3)     # token-major storage
+    w = (1 + 0.1 * torch.randn(128, generator=g)).bfloat16()
+    dx = x.cuda()
+    new = lambda: torch.empty(B, H, S, 128, dtype=torch.bfloat16, device="cuda")
+    moved = M().norm_rope(dx, new())
+    assert moved.is_contiguous() and torch.equal(moved.cpu(), x)
+    normed = M().norm_rope(dx, new(), w.cuda())
+    want_n = O.rms_norm_fp32(x, w)
+    assert torch.all((normed.cpu().float() - want_n.float()).abs() <= want_n.float().abs() * BF16_ULP + 1e-6)
+    ang = O.rope_3d_angles(grid, 128)
+    roped = M().norm_rope(normed, new(), None, grid)
+    want_r = O.rope_3d_apply(normed.cpu(), ang)
+    assert torch.all((roped.cpu().float() - want_r.float()).abs() <= want_r.float().abs() * BF16_ULP + 1e-2)
+    both = M().norm_rope(dx, new(), w.cuda(), grid)
+    assert torch.equal(both, roped)                          # the fused pass rounds at the same points
+    # frames 2..6 of the grid, handed over as a tensor of 4 frames
+    part = normed[:, :, 2 * 20:].contiguous()
+    off = M().norm_rope(part, torch.empty_like(part), None, (4, 4, 5), t_offset=2, table_grid=grid)
+    assert torch.equal(off, roped[:, :, 2 * 20:])
+    with pytest.raises(AssertionError):
+        M().norm_rope(part, torch.empty_like(part), None, (4, 4, 5), t_offset=3, table_grid=grid)
+
+
 def test_unbuilt_branches_raise():
     m = make_module().cuda()
     x = torch.zeros(1, 256, 512, dtype=torch.bfloat16, device="cuda")
-    with pytest.raises(NotImplementedError):
-        m(x, shape=(4, 8, 8), return_kv=True)
-    with pytest.raises(NotImplementedError):
-        m.forward_with_kv_cache(x)
+    with pytest.raises(ValueError):
+        m.forward_with_kv_cache(x, shape=(4, 8, 8), kv_cache=(x.view(1, 4, 256, 128), x.view(1, 4, 256, 128)))
     m.enable_bsa = False
     with pytest.raises(NotImplementedError):
         m(x, shape=(4, 8, 8))

@@ -55,3 +55,31 @@ def test_rope_pairs_are_interleaved():
     x = torch.tensor([1.0, 2.0, 3.0, 4.0]).view(1, 1, 1, 4)
     y = O.rope_3d_apply(x, ang)
     assert torch.allclose(y.flatten(), torch.tensor([-2.0, 1.0, 3.0, 4.0]), atol=1e-6)
+
+
+def test_kv_cache_forward_equals_the_noise_rows_of_the_split_forward():
+    """attn:149-181 against attn:107-147: running the conditioning frames first (return_kv) and the new
+    frames against the cache must reproduce, bit for bit, the noise rows of one forward over all frames
+    with num_cond_latents set: the same keys are normalised, rotated at the same grid positions and
+    selected from the same pooled scores in both routes."""
+    g = torch.Generator().manual_seed(3)
+    heads, C, cond, T, Hh, W = 2, 256, 4, 4, 4, 8
+    n_c, n_new = cond * Hh * W, T * Hh * W
+    x = torch.randn(1, n_c + n_new, C, generator=g).bfloat16()
+    w_qkv = (torch.randn(3 * C, C, generator=g) * 0.05).bfloat16()
+    b_qkv = (torch.randn(3 * C, generator=g) * 0.05).bfloat16()
+    w_proj = (torch.randn(C, C, generator=g) * 0.05).bfloat16()
+    b_proj = (torch.randn(C, generator=g) * 0.05).bfloat16()
+    qw = (1 + 0.1 * torch.randn(128, generator=g)).bfloat16()
+    kw = (1 + 0.1 * torch.randn(128, generator=g)).bfloat16()
+    prm = dict(sparsity=0.5, chunk_3d_shape_q=(4, 4, 4), chunk_3d_shape_k=(4, 4, 4))
+    full = O.attention_module_forward(x, w_qkv, b_qkv, w_proj, b_proj, qw, kw, (T + cond, Hh, W), heads, prm, cond)
+    cache = O.attention_module_kv(x[:, :n_c], w_qkv, b_qkv, qw, kw, heads)
+    assert cache[0].shape == (1, heads, n_c, 128)
+    got = O.attention_module_forward_with_kv_cache(x[:, n_c:], w_qkv, b_qkv, w_proj, b_proj, qw, kw, (T, Hh, W), heads,
+                                                   prm, cond, cache)
+    assert torch.equal(got, full[:, n_c:])
+    # the cache is position-free: its keys are not rotated yet
+    k_plain = O.rms_norm_fp32((x[:, :n_c].float() @ w_qkv.float().t() + b_qkv.float()).bfloat16()
+                              .view(1, n_c, 3, heads, 128)[:, :, 1].transpose(1, 2), kw)
+    assert torch.equal(cache[0], k_plain)
