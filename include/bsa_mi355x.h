@@ -208,6 +208,18 @@ int bsa_fwd_thw(const bsa_3d_params* p,
 int bsa_rmsnorm(const void* x, const void* weight, void* out, int64_t rows, int dim, float eps,
                 int dtype, void* stream);
 
+/* The adaLN wrapper of the self-attention branch of a DiT block (longcat_video/modules/longcat_video_dit.py:
+ * 82-103), bf16 / fp16, rows of `dim` elements, `rows_per_group` consecutive rows (the tokens of one latent
+ * frame) sharing one fp32 row of shift / scale / gate:
+ *   bsa_layernorm_modulate: out = cast(layer_norm(float(x)) * (scale + 1) + shift), LayerNorm without affine
+ *     parameters, biased variance, everything in fp32, one rounding.  Replaces modulate_fp32(mod_norm_attn, ...)
+ *     (blocks.py:56-69, 126-134; longcat_video_dit.py:88).  dim <= 8192.
+ *   bsa_gated_residual: out = cast(float(x) + gate * float(y)).  Replaces longcat_video_dit.py:101-103. */
+int bsa_layernorm_modulate(const void* x, const float* shift, const float* scale, void* out, int64_t rows,
+                           int rows_per_group, int dim, float eps, int dtype, void* stream);
+int bsa_gated_residual(const void* x, const void* y, const float* gate, void* out, int64_t rows,
+                       int rows_per_group, int dim, int dtype, void* stream);
+
 /* In-place per-head RMSNorm (blocks.py:42-53, called attention.py:116) followed by 3-D RoPE
  * (longcat_video/modules/rope_3d.py:99-120, called attention.py:121) on q and k.
  *   q, k  [B, Hn, T*H*W, 128] with element strides {B, Hn, S} (views of the QKV projection are fine)

@@ -42,6 +42,89 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* __restrict__
     }
 }
 
+// --------------------------------------- LayerNorm (no affine) + adaLN modulate
+// out = T(((x - mean) * rsqrt(var + eps)) * (scale + 1) + shift), everything in fp32 with one rounding at
+// the end; mean and the biased variance over the row (two passes over registers).  shift / scale are fp32
+// rows shared by `rows_per_group` consecutive rows (one latent frame).  One wavefront per row, dim <= 8192.
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_modulate_kernel(const T* __restrict__ x, const float* __restrict__ shift,
+                                                                 const float* __restrict__ scale, T* __restrict__ out,
+                                                                 int64_t rows, int rows_per_group, int dim, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* xr = x + row * dim;
+    const float* sh = shift + (row / rows_per_group) * dim;
+    const float* sc = scale + (row / rows_per_group) * dim;
+    uint4 raw[16];                     // the row stays in registers in its storage type
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int d = j * 512 + lane * 8;
+        if (d < dim) {
+            raw[j] = *reinterpret_cast<const uint4*>(xr + d);
+            const T* e = reinterpret_cast<const T*>(&raw[j]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sum += (float)e[i];
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+    const float mean = sum / (float)dim;
+    float sq = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+        if (j * 512 + lane * 8 < dim) {
+            const T* e = reinterpret_cast<const T*>(&raw[j]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { const float c = (float)e[i] - mean; sq = fmaf(c, c, sq); }
+        }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
+    const float rstd = rsqrtf(sq / (float)dim + eps);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int d = j * 512 + lane * 8;
+        if (d < dim) {
+            const float4 s0 = *reinterpret_cast<const float4*>(sc + d), s1 = *reinterpret_cast<const float4*>(sc + d + 4);
+            const float4 h0 = *reinterpret_cast<const float4*>(sh + d), h1 = *reinterpret_cast<const float4*>(sh + d + 4);
+            const float scl[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+            const float sft[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
+            const T* e = reinterpret_cast<const T*>(&raw[j]);
+            T res[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float n = __fmul_rn((float)e[i] - mean, rstd);
+                res[i] = (T)__fadd_rn(__fmul_rn(n, __fadd_rn(scl[i], 1.0f)), sft[i]);     // x * (scale + 1) + shift
+            }
+            *reinterpret_cast<uint4*>(out + row * dim + d) = *reinterpret_cast<const uint4*>(res);
+        }
+    }
+}
+
+// out = T(float(x) + gate * float(y)), gate fp32 per group of rows (one latent frame).
+template <typename T>
+__global__ __launch_bounds__(256) void gated_residual_kernel(const T* __restrict__ x, const T* __restrict__ y,
+                                                             const float* __restrict__ gate, T* __restrict__ out,
+                                                             int64_t rows, int rows_per_group, int dim) {
+    const int per_row = dim / 8;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * per_row) return;
+    const int64_t row = i / per_row;
+    const int d = (int)(i % per_row) * 8;
+    const uint4 xr = *reinterpret_cast<const uint4*>(x + row * dim + d);
+    const uint4 yr = *reinterpret_cast<const uint4*>(y + row * dim + d);
+    const float* g = gate + (row / rows_per_group) * dim + d;
+    const float4 g0 = *reinterpret_cast<const float4*>(g), g1 = *reinterpret_cast<const float4*>(g + 4);
+    const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+    const T* xe = reinterpret_cast<const T*>(&xr);
+    const T* ye = reinterpret_cast<const T*>(&yr);
+    T res[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) res[k] = (T)__fadd_rn((float)xe[k], __fmul_rn(gv[k], (float)ye[k]));
+    *reinterpret_cast<uint4*>(out + row * dim + d) = *reinterpret_cast<const uint4*>(res);
+}
+
 // ------------------------------------------------- per-head RMSNorm + RoPE
 // One row = one (token, head) vector of D = 128 elements, handled by 16 lanes
 // (8 elements each, i.e. 4 interleaved rotation pairs per lane).
@@ -149,6 +232,47 @@ int bsa_rmsnorm(const void* x, const void* weight, void* out, int64_t rows, int 
         return set_error(BSA_ERR_UNSUPPORTED, "rmsnorm: dtype %d is not built (bf16, fp16)", dtype);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? BSA_OK : set_error(BSA_ERR_HIP, "rmsnorm launch: %s", hipGetErrorString(e));
+}
+
+int bsa_layernorm_modulate(const void* x, const float* shift, const float* scale, void* out, int64_t rows,
+                           int rows_per_group, int dim, float eps, int dtype, void* stream) {
+    if (!x || !shift || !scale || !out) return set_error(BSA_ERR_BAD_ARG, "layernorm_modulate: null pointer");
+    if (rows <= 0 || rows_per_group <= 0 || rows % rows_per_group != 0)
+        return set_error(BSA_ERR_SHAPE, "layernorm_modulate: %lld rows do not split into groups of %d", (long long)rows, rows_per_group);
+    if (dim <= 0 || dim % 8 != 0 || dim > 8192) return set_error(BSA_ERR_UNSUPPORTED, "layernorm_modulate: dim %d (multiples of 8 up to 8192)", dim);
+    if (!(eps >= 0.f)) return set_error(BSA_ERR_BAD_ARG, "layernorm_modulate: eps must be non-negative");
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(shift) | reinterpret_cast<uintptr_t>(scale) | reinterpret_cast<uintptr_t>(out)) & 15u)
+        return set_error(BSA_ERR_BAD_ARG, "layernorm_modulate: pointers must be 16-byte aligned");
+    const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    if (dtype == BSA_BF16)
+        hipLaunchKernelGGL((layernorm_modulate_kernel<__bf16>), grid, block, 0, (hipStream_t)stream, (const __bf16*)x, shift, scale, (__bf16*)out, rows, rows_per_group, dim, eps);
+    else if (dtype == BSA_F16)
+        hipLaunchKernelGGL((layernorm_modulate_kernel<_Float16>), grid, block, 0, (hipStream_t)stream, (const _Float16*)x, shift, scale, (_Float16*)out, rows, rows_per_group, dim, eps);
+    else
+        return set_error(BSA_ERR_UNSUPPORTED, "layernorm_modulate: dtype %d is not built (bf16, fp16)", dtype);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? BSA_OK : set_error(BSA_ERR_HIP, "layernorm_modulate launch: %s", hipGetErrorString(e));
+}
+
+int bsa_gated_residual(const void* x, const void* y, const float* gate, void* out, int64_t rows, int rows_per_group,
+                       int dim, int dtype, void* stream) {
+    if (!x || !y || !gate || !out) return set_error(BSA_ERR_BAD_ARG, "gated_residual: null pointer");
+    if (rows <= 0 || rows_per_group <= 0 || rows % rows_per_group != 0)
+        return set_error(BSA_ERR_SHAPE, "gated_residual: %lld rows do not split into groups of %d", (long long)rows, rows_per_group);
+    if (dim <= 0 || dim % 8 != 0) return set_error(BSA_ERR_UNSUPPORTED, "gated_residual: dim %d must be a multiple of 8", dim);
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(out)) & 15u)
+        return set_error(BSA_ERR_BAD_ARG, "gated_residual: pointers must be 16-byte aligned");
+    const int64_t n = rows * (dim / 8);
+    if ((n + 255) / 256 > 0x7fffffffLL) return set_error(BSA_ERR_UNSUPPORTED, "gated_residual: too many elements");
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    if (dtype == BSA_BF16)
+        hipLaunchKernelGGL((gated_residual_kernel<__bf16>), grid, block, 0, (hipStream_t)stream, (const __bf16*)x, (const __bf16*)y, gate, (__bf16*)out, rows, rows_per_group, dim);
+    else if (dtype == BSA_F16)
+        hipLaunchKernelGGL((gated_residual_kernel<_Float16>), grid, block, 0, (hipStream_t)stream, (const _Float16*)x, (const _Float16*)y, gate, (_Float16*)out, rows, rows_per_group, dim);
+    else
+        return set_error(BSA_ERR_UNSUPPORTED, "gated_residual: dtype %d is not built (bf16, fp16)", dtype);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? BSA_OK : set_error(BSA_ERR_HIP, "gated_residual launch: %s", hipGetErrorString(e));
 }
 
 int bsa_norm_rope(const void* src, const int64_t src_strides[3], void* dst, const int64_t dst_strides[3],

@@ -48,6 +48,8 @@ SIGNATURES = {
     "bsa_fwd_thw": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
                          _p, _p, _i, _p, _p, C.c_size_t, _p]),
     "bsa_rmsnorm": (_i, [_p, _p, _p, _i64, _i, _f, _i, _p]),
+    "bsa_layernorm_modulate": (_i, [_p, _p, _p, _p, _i64, _i, _i, _f, _i, _p]),
+    "bsa_gated_residual": (_i, [_p, _p, _p, _p, _i64, _i, _i, _i, _p]),
     "bsa_norm_rope": (_i, [_p, _strides, _p, _strides, _p, _p] + [_i] * 8 + [_f, _i, _p]),
     "bsa_qk_norm_rope": (_i, [_p, _strides, _p, _strides, _p, _p, _p] + [_i] * 6 + [_f, _i, _p]),
     "bsa_linear_bf16": (_i, [_p, _p, _p, _p, _p, _i64, _i, _i, _p, C.c_size_t, _p]),

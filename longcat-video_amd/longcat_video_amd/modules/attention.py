@@ -280,3 +280,70 @@ def attention_block_forward(x: torch.Tensor, pre_norm_weight: torch.Tensor, attn
     -> residual: the attention sub-chain of one DiT block as BASELINE config 5 words it."""
     y = rms_norm(x, pre_norm_weight, eps)
     return attn(y, shape=shape, num_cond_latents=num_cond_latents, residual=x)
+
+
+# ---------------------------------------------------------------------------
+# adaLN wrapper of the self-attention branch of a DiT block
+# ---------------------------------------------------------------------------
+def _frames(x: torch.Tensor, mod: torch.Tensor, name: str):
+    B, N, C = x.shape
+    assert mod.dtype == torch.float32, "%s must be fp32 (blocks.py:129)" % name
+    assert mod.dim() == 4 and mod.shape[0] == B and mod.shape[2] == 1 and mod.shape[3] == C, \
+        "%s must be [B, T, 1, C]" % name
+    T = mod.shape[1]
+    assert N % T == 0
+    return mod.contiguous(), N // T
+
+
+def layernorm_modulate(x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """modulate_fp32(LayerNorm_FP32(no affine), x.view(B,T,-1,C), shift, scale).view(B,N,C)
+    (blocks.py:56-69, 126-134 as called at longcat_video_dit.py:88).  x [B,N,C] bf16/fp16; shift, scale [B,T,1,C] fp32."""
+    if not x.is_cuda:
+        raise RuntimeError("the engine runs on the GPU only")
+    code = {torch.bfloat16: _capi.BSA_BF16, torch.float16: _capi.BSA_F16}.get(x.dtype)
+    if code is None:
+        raise NotImplementedError("layernorm_modulate: dtype %s is not built (bf16, fp16)" % x.dtype)
+    shift, per = _frames(x, shift, "shift")
+    scale, _ = _frames(x, scale, "scale")
+    x = x.contiguous()
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        _capi.check(_capi.load().bsa_layernorm_modulate(_ptr(x), _ptr(shift), _ptr(scale), _ptr(out), x.shape[0] * x.shape[1],
+                                                        per, x.shape[2], float(eps), code, _stream(x)), "layernorm_modulate")
+    return out
+
+
+def gated_residual(x: torch.Tensor, gate: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """(x + gate * y.view(B,-1,N//T,C)).to(x.dtype) of longcat_video_dit.py:101-103; gate [B,T,1,C] fp32."""
+    if not x.is_cuda:
+        raise RuntimeError("the engine runs on the GPU only")
+    code = {torch.bfloat16: _capi.BSA_BF16, torch.float16: _capi.BSA_F16}.get(x.dtype)
+    if code is None:
+        raise NotImplementedError("gated_residual: dtype %s is not built (bf16, fp16)" % x.dtype)
+    gate, per = _frames(x, gate, "gate")
+    assert y.shape == x.shape and y.dtype == x.dtype
+    x, y = x.contiguous(), y.contiguous()
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        _capi.check(_capi.load().bsa_gated_residual(_ptr(x), _ptr(y), _ptr(gate), _ptr(out), x.shape[0] * x.shape[1], per,
+                                                    x.shape[2], code, _stream(x)), "gated_residual")
+    return out
+
+
+@torch.no_grad()
+def dit_self_attention_branch(x: torch.Tensor, shift_msa: torch.Tensor, scale_msa: torch.Tensor, gate_msa: torch.Tensor,
+                              attn: Attention, latent_shape, num_cond_latents=None, return_kv=False, kv_cache=None):
+    """The self-attention branch of LongCatSingleStreamBlock.forward (longcat_video_dit.py:88-103):
+    x + gate * attn(modulate(LayerNorm(x), shift, scale)), with the block's three attention routes
+    (plain / return_kv / kv_cache).  The modulation vectors come from the caller (adaLN_modulation is a
+    small fp32 linear layer outside this path)."""
+    x_m = layernorm_modulate(x, shift_msa, scale_msa)
+    new_cache = None
+    if kv_cache is not None:
+        x_s = attn.forward_with_kv_cache(x_m, shape=latent_shape, num_cond_latents=num_cond_latents, kv_cache=kv_cache)
+    elif return_kv:
+        x_s, new_cache = attn(x_m, shape=latent_shape, num_cond_latents=num_cond_latents, return_kv=True)
+    else:
+        x_s = attn(x_m, shape=latent_shape, num_cond_latents=num_cond_latents)
+    out = gated_residual(x, gate_msa, x_s)
+    return (out, new_cache) if return_kv else out

@@ -448,3 +448,24 @@ def attention_module_forward_with_kv_cache(x, w_qkv, b_qkv, w_proj, b_proj, q_no
     o, *_ = flash_attn_bsa_3d(q, k_full, v_full, (T, Hh, W), (T + num_cond_latents, Hh, W), **bsa_params)
     o = o.to(dt).transpose(1, 2).reshape(B, N, C)
     return (o.float() @ w_proj.float().t() + b_proj.float()).to(dt)
+
+
+def layernorm_modulate_fp32(x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """modulate_fp32 (blocks.py:126-134) around LayerNorm_FP32 without affine parameters (blocks.py:56-69), as
+    called at longcat_video_dit.py:88: x [B,N,C] viewed as [B,T,N/T,C]; shift, scale [B,T,1,C] fp32; the
+    statistics, the product with (scale + 1) and the sum are fp32, one rounding to x.dtype."""
+    B, N, C = x.shape
+    T = shift.shape[1]
+    xf = x.float().view(B, T, N // T, C)
+    mean = xf.mean(-1, keepdim=True)
+    var = ((xf - mean) ** 2).mean(-1, keepdim=True)
+    n = (xf - mean) * torch.rsqrt(var + eps)
+    return (n * (scale.float() + 1) + shift.float()).to(x.dtype).view(B, N, C)
+
+
+def gated_residual_fp32(x: torch.Tensor, gate: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """longcat_video_dit.py:101-103: x + gate * y in fp32 (gate [B,T,1,C] fp32), one rounding to x.dtype."""
+    B, N, C = x.shape
+    T = gate.shape[1]
+    out = x.float().view(B, T, N // T, C) + gate.float() * y.float().view(B, T, N // T, C)
+    return out.view(B, N, C).to(x.dtype)

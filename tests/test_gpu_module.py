@@ -201,6 +201,44 @@ def test_norm_rope_steps_and_frame_offset():
         M().norm_rope(part, torch.empty_like(part), None, (4, 4, 5), t_offset=3, table_grid=grid)
 
 
+def test_layernorm_modulate_and_gated_residual():
+    g = torch.Generator().manual_seed(12)
+    B, T, per, C = 2, 3, 40, 512
+    x = (torch.randn(B, T * per, C, generator=g) * 2 + 0.5).bfloat16()
+    y = torch.randn(B, T * per, C, generator=g).bfloat16()
+    shift = torch.randn(B, T, 1, C, generator=g)
+    scale = torch.randn(B, T, 1, C, generator=g) * 0.2
+    gate = torch.randn(B, T, 1, C, generator=g)
+    got = M().layernorm_modulate(x.cuda(), shift.cuda(), scale.cuda()).cpu()
+    want = O.layernorm_modulate_fp32(x, shift, scale)
+    d = (got.float() - want.float()).abs()
+    assert torch.all(d <= want.float().abs() * BF16_ULP + 1e-6) and (d > 0).float().mean() < 0.01   # fp32 statistics differ in the last bit at most
+    assert torch.equal(M().gated_residual(x.cuda(), gate.cuda(), y.cuda()).cpu(), O.gated_residual_fp32(x, gate, y))
+    wide = torch.randn(1, 8, 4096, generator=g).bfloat16()                     # the model's width
+    z = torch.zeros(1, 2, 1, 4096)
+    got = M().layernorm_modulate(wide.cuda(), z.cuda(), z.cuda()).cpu()
+    want = O.layernorm_modulate_fp32(wide, z, z)
+    assert torch.all((got.float() - want.float()).abs() <= want.float().abs() * BF16_ULP + 1e-6)
+    with pytest.raises(AssertionError):
+        M().layernorm_modulate(x.cuda(), shift.cuda().bfloat16(), scale.cuda())
+
+
+def test_dit_self_attention_branch():
+    """longcat_video_dit.py:88-103: LayerNorm + modulate, attention, gated residual."""
+    shape = (4, 8, 8)
+    m = make_module(sparsity=0.5, seed=13)
+    g = torch.Generator().manual_seed(14)
+    x = torch.randn(1, 256, 512, generator=g).bfloat16()
+    shift = torch.randn(1, 4, 1, 512, generator=g) * 0.1
+    scale = torch.randn(1, 4, 1, 512, generator=g) * 0.1
+    gate = torch.randn(1, 4, 1, 512, generator=g)
+    x_m = O.layernorm_modulate_fp32(x, shift, scale)
+    want = O.gated_residual_fp32(x, gate, module_reference(m, x_m, shape))
+    got = M().dit_self_attention_branch(x.cuda(), shift.cuda(), scale.cuda(), gate.cuda(), m.cuda(), shape).cpu()
+    d = (got.float() - want.float()).abs()
+    assert d.max() <= 6e-2 and d.mean() <= 4e-3, (d.max(), d.mean())
+
+
 def test_unbuilt_branches_raise():
     m = make_module().cuda()
     x = torch.zeros(1, 256, 512, dtype=torch.bfloat16, device="cuda")

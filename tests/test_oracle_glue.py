@@ -83,3 +83,39 @@ def test_kv_cache_forward_equals_the_noise_rows_of_the_split_forward():
     k_plain = O.rms_norm_fp32((x[:, :n_c].float() @ w_qkv.float().t() + b_qkv.float()).bfloat16()
                               .view(1, n_c, 3, heads, 128)[:, :, 1].transpose(1, 2), kw)
     assert torch.equal(cache[0], k_plain)
+
+
+def test_layernorm_modulate_against_the_library_routine():
+    """The oracle's LayerNorm must be torch's F.layer_norm (what LayerNorm_FP32 calls, blocks.py:60-66); the
+    modulation is checked on closed forms: zero shift/scale is the plain norm, and a constant row maps to shift."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(5)
+    B, T, per, C = 2, 3, 5, 64
+    x = (torch.randn(B, T * per, C, generator=g) * 3 + 1).bfloat16()
+    shift = torch.randn(B, T, 1, C, generator=g)
+    scale = torch.randn(B, T, 1, C, generator=g) * 0.1
+    zero = torch.zeros(B, T, 1, C)
+    plain = O.layernorm_modulate_fp32(x, zero, zero)
+    assert torch.equal(plain, F.layer_norm(x.float(), (C,), None, None, 1e-6).to(torch.bfloat16))
+    want = (F.layer_norm(x.float(), (C,), None, None, 1e-6).view(B, T, per, C) * (scale + 1) + shift).to(torch.bfloat16)
+    assert torch.equal(O.layernorm_modulate_fp32(x, shift, scale), want.view(B, T * per, C))
+    const = torch.full((B, T * per, C), 2.5).bfloat16()
+    assert torch.equal(O.layernorm_modulate_fp32(const, shift, scale),
+                       shift.expand(B, T, per, C).reshape(B, T * per, C).to(torch.bfloat16))
+    # every frame uses its own row of shift / scale
+    s2 = shift.clone()
+    s2[:, 1] += 1.0
+    d = (O.layernorm_modulate_fp32(x, s2, scale).float() - O.layernorm_modulate_fp32(x, shift, scale).float()).view(B, T, per, C)
+    assert torch.all(d[:, 0] == 0) and torch.all(d[:, 2] == 0) and torch.all((d[:, 1] - 1).abs() < 0.05)
+
+
+def test_gated_residual_closed_forms():
+    g = torch.Generator().manual_seed(6)
+    B, T, per, C = 1, 2, 4, 32
+    x = torch.randn(B, T * per, C, generator=g).bfloat16()
+    y = torch.randn(B, T * per, C, generator=g).bfloat16()
+    assert torch.equal(O.gated_residual_fp32(x, torch.zeros(B, T, 1, C), y), x)
+    assert torch.equal(O.gated_residual_fp32(torch.zeros_like(x), torch.ones(B, T, 1, C), y), y)
+    gate = torch.randn(B, T, 1, C, generator=g)
+    want = (x.float() + gate.expand(B, T, per, C).reshape(B, T * per, C) * y.float()).bfloat16()
+    assert torch.equal(O.gated_residual_fp32(x, gate, y), want)
