@@ -31,42 +31,68 @@ template <> struct Vec8<__bf16> { typedef bf16x8 type; };
 template <> struct Vec8<_Float16> { typedef f16x8 type; };
 
 // ---------------------------------------------------------------- score GEMM
-// Workgroup = 4 wavefronts = a 64x64 score tile; each wavefront one 32x32 MFMA
-// tile.  Operands come straight from global memory (the pooled tensors are a
-// few hundred KB per head and stay in L2): lane l supplies row l%32, and the 8
-// consecutive d values 16*s + 8*(l/32) .. +8 of k-step s, for both operands.
+// Workgroup = 4 wavefronts = 128 score rows x up to kScoreCols columns; each wavefront keeps its 32
+// query rows (all 128 d, the A operand) in registers and walks the column tiles, fetching the B
+// fragments of the next tile while the 8 MFMAs of the current one run.  Operands come straight from
+// global memory (the pooled tensors are a few MB and stay in L2; the four wavefronts ask for the same
+// k rows): lane l supplies row l%32 and the 8 consecutive d values 16*s + 8*(l/32) .. +8 of k-step s.
+// A finished 32x32 tile goes through a wavefront-private LDS patch so that it leaves as 16-byte
+// stores (half a row per lane) instead of 2-byte ones.
+constexpr int kScoreCols = 256;
 template <typename T>
 __global__ __launch_bounds__(256) void score_mfma_kernel(const T* __restrict__ qc,
                                                          const T* __restrict__ kc,
-                                                         T* __restrict__ score, int nbq, int nbk,
-                                                         int D) {
+                                                         T* __restrict__ score, int nbq, int nbk) {
     typedef typename Vec8<T>::type V8;
+    constexpr int D = 128;
+    __shared__ __attribute__((aligned(16))) T patch[4][32][40];      // 80-byte rows: 16-byte aligned, bank-spread
     const int bh = blockIdx.z;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int m0 = blockIdx.y * 64 + (wave >> 1) * 32;
-    const int n0 = blockIdx.x * 64 + (wave & 1) * 32;
-    if (m0 >= nbq || n0 >= nbk) return;   // whole wavefront out of range
+    const int m0 = blockIdx.y * 128 + wave * 32;
+    const int n_begin = blockIdx.x * kScoreCols;
+    const int n_end = min(n_begin + kScoreCols, nbk);
+    if (m0 >= nbq) return;                    // whole wavefront out of range (no workgroup barrier below)
     const int lr = lane & 31, lh = lane >> 5;
     const int mrow = min(m0 + lr, nbq - 1);   // clamp: rows past the end are computed, not stored
-    const int nrow = min(n0 + lr, nbk - 1);
     const T* qa = qc + ((int64_t)bh * nbq + mrow) * D + lh * 8;
-    const T* kb = kc + ((int64_t)bh * nbk + nrow) * D + lh * 8;
-    f32x16 acc;
+    V8 a[8], b[8], bn[8];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    for (int s = 0; s < D / 16; ++s) {
-        const V8 a = *reinterpret_cast<const V8*>(qa + s * 16);
-        const V8 b = *reinterpret_cast<const V8*>(kb + s * 16);
-        acc = mfma32(a, b, acc);
-    }
-    // accumulator i of lane l: row 8*(i/4) + 4*(l/32) + i%4, column l%32
-    const int n = n0 + lr;
-    if (n < nbk) {
+    for (int s = 0; s < 8; ++s) a[s] = *reinterpret_cast<const V8*>(qa + s * 16);
+    auto load_b = [&](V8* dst, int n0) {
+        const T* kb = kc + ((int64_t)bh * nbk + min(n0 + lr, nbk - 1)) * D + lh * 8;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int m = m0 + 8 * (i / 4) + 4 * lh + (i % 4);
-            if (m < nbq) score[((int64_t)bh * nbq + m) * nbk + n] = (T)acc[i];
+        for (int s = 0; s < 8; ++s) dst[s] = *reinterpret_cast<const V8*>(kb + s * 16);
+    };
+    load_b(b, n_begin);
+    T (*mine)[40] = patch[wave];
+    const bool vec_ok = (nbk % 8) == 0;       // rows of the score matrix stay 16-byte aligned
+    for (int n0 = n_begin; n0 < n_end; n0 += 32) {
+        if (n0 + 32 < n_end) load_b(bn, n0 + 32);
+        f32x16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) acc = mfma32(a[s], b[s], acc);
+        // accumulator i of lane l: row 8*(i/4) + 4*(l/32) + i%4, column l%32
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mine[8 * (i / 4) + 4 * lh + (i % 4)][lr] = (T)acc[i];
+        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): this wavefront's LDS writes have landed
+        __builtin_amdgcn_wave_barrier();
+        const int r = lane >> 1, c0 = (lane & 1) * 16;
+        const int m = m0 + r;
+        if (m < nbq) {
+            T* dst = score + ((int64_t)bh * nbq + m) * nbk + n0 + c0;
+            if (vec_ok && n0 + c0 + 16 <= nbk) {
+                *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(&mine[r][c0]);
+                *reinterpret_cast<uint4*>(dst + 8) = *reinterpret_cast<const uint4*>(&mine[r][c0 + 8]);
+            } else {
+                for (int c = 0; c < 16 && n0 + c0 + c < nbk; ++c) dst[c] = mine[r][c0 + c];
+            }
         }
+        __builtin_amdgcn_s_waitcnt(0xc07f);   // the patch is read before the next tile overwrites it
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int s = 0; s < 8; ++s) b[s] = bn[s];
     }
 }
 
@@ -115,15 +141,26 @@ template <> struct KeyOf<uint32_t> {   // fp32 bit patterns
     __device__ static int index(uint64_t k) { return (int)(0xFFFFFFFFu - (uint32_t)k); }
 };
 
-constexpr int kMaxSel = 1024;   // keys kept in LDS per wavefront
+constexpr int kMaxSel = 1024;   // winners kept in LDS per wavefront
 
-template <typename S, int NPL>
+// Order-preserving image of a score alone (ties stay ties).
+__device__ inline uint32_t ord_of(uint16_t s) { return ord16(s); }
+__device__ inline uint32_t ord_of(uint32_t s) { return ord32(s); }
+
+// One wavefront per score row; lane l holds columns l, l + 64, ... in registers.
+//   1. bitwise binary search for the k-th largest score value t (counting = ballot + popcount);
+//   2. every score above t wins, and of the scores equal to t the ones with the lowest column
+//      index, as many as are still needed; walking the registers in column order hands out the
+//      positions of the ascending-block-order list at the same time (no sort);
+//   3. only when the score-order list is wanted: rank the winners by (score desc, index asc).
+template <typename S, int NPL, bool SCORE_ORDER>
 __global__ __launch_bounds__(256) void topk_kernel(const S* __restrict__ score,
                                                    int32_t* __restrict__ idx_out,
                                                    int32_t* __restrict__ idx_sorted_out,
                                                    int32_t* __restrict__ lens_out, int64_t rows,
                                                    int nbk, int k_sel) {
     typedef typename KeyOf<S>::type K;
+    constexpr int kValueBits = 8 * (int)sizeof(S);
     __shared__ K sel[4][kMaxSel];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + wave;
@@ -132,50 +169,60 @@ __global__ __launch_bounds__(256) void topk_kernel(const S* __restrict__ score,
     if (k_sel == 0) return;
 
     const S* srow = score + row * nbk;
-    K key[NPL];
+    uint32_t val[NPL];                      // ord(score); 0 for columns past the end of the row
 #pragma unroll
     for (int j = 0; j < NPL; ++j) {
         const int i = j * 64 + lane;
-        key[j] = i < nbk ? KeyOf<S>::make(srow[i], i) : (K)0;   // 0 is below every real key
+        const S raw = srow[min(i, nbk - 1)];               // unconditional load, masked afterwards
+        val[j] = i < nbk ? ord_of(raw) : 0u;
     }
-    // largest T with count(key >= T) >= k_sel; keys are unique, so the count ends at k_sel
-    K thr = 0;
-    for (int bit = KeyOf<S>::kBits - 1; bit >= 0; --bit) {
-        const K cand = thr | ((K)1 << bit);
+    // Largest t with count(ord >= t) >= k_sel, t = 0 if there is none above.  Every candidate is at
+    // least 1, so the zeros past the end of the row never count.  Leaving early with exactly k_sel
+    // columns at or above t is fine: the winners are then all columns at or above t.
+    uint32_t thr = 0;
+    for (int bit = kValueBits - 1; bit >= 0; --bit) {
+        const uint32_t cand = thr | (1u << bit);
         int cnt = 0;
 #pragma unroll
-        for (int j = 0; j < NPL; ++j) cnt += __popcll(__ballot(key[j] >= cand));
+        for (int j = 0; j < NPL; ++j) cnt += __popcll(__ballot(val[j] >= cand));
         if (cnt >= k_sel) {
             thr = cand;
             if (cnt == k_sel) break;
         }
     }
-    // compact the winners into LDS (any order), then rank them
+    // every column above thr wins; of the real columns equal to thr, the first need_eq in column order
+    int cnt_gt = 0;
+#pragma unroll
+    for (int j = 0; j < NPL; ++j) cnt_gt += __popcll(__ballot(val[j] > thr));
+    const int need_eq = k_sel - cnt_gt;
+
     K* mine = sel[wave];
-    int base = 0;
+    int pos = 0, eq_seen = 0;
     const uint64_t lt = ((uint64_t)1 << lane) - 1;
 #pragma unroll
     for (int j = 0; j < NPL; ++j) {
-        const bool win = key[j] >= thr;
+        const int i = j * 64 + lane;
+        const bool eq = val[j] == thr && i < nbk;          // thr may be 0, like the padding of val
+        const uint64_t meq = __ballot(eq);
+        const bool win = val[j] > thr || (eq && eq_seen + __popcll(meq & lt) < need_eq);
         const uint64_t m = __ballot(win);
-        if (win) mine[base + __popcll(m & lt)] = key[j];
-        base += __popcll(m);
+        if (win) {
+            const int p = pos + __popcll(m & lt);
+            if (idx_sorted_out) idx_sorted_out[row * k_sel + p] = i;          // column order = ascending block order
+            if (SCORE_ORDER) mine[p] = KeyOf<S>::make(srow[i], i);
+        }
+        pos += __popcll(m);
+        eq_seen += __popcll(meq);
     }
+    if (!SCORE_ORDER) return;
     __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): LDS writes of this wavefront landed
     __builtin_amdgcn_wave_barrier();
-    // idx_out: descending score, ties towards the lowest index (the order of the keys);
-    // idx_sorted_out: the same set in ascending block index
+    // descending score, ties towards the lowest index: the order of the combined keys
     for (int e = lane; e < k_sel; e += 64) {
         const K me = mine[e];
-        const int my_idx = KeyOf<S>::index(me);
-        int rank = 0, rank_idx = 0;
-        for (int o = 0; o < k_sel; ++o) {
-            const K other = mine[o];
-            rank += other > me;
-            rank_idx += KeyOf<S>::index(other) < my_idx;
-        }
-        if (idx_out) idx_out[row * k_sel + rank] = my_idx;
-        if (idx_sorted_out) idx_sorted_out[row * k_sel + rank_idx] = my_idx;
+        int rank = 0;
+        for (int o = 0; o < k_sel; ++o) rank += mine[o] > me;
+        idx_out[row * k_sel + rank] = KeyOf<S>::index(me);
     }
 }
 
@@ -183,9 +230,13 @@ template <typename S>
 hipError_t launch_topk_t(const S* score, int32_t* idx, int32_t* idx_sorted, int32_t* lens, int64_t rows,
                          int nbk, int k_sel, hipStream_t st) {
     dim3 grid((unsigned)((rows + 3) / 4)), block(256);
-#define BSA_TOPK(N)                                                                          \
-    hipLaunchKernelGGL((topk_kernel<S, N>), grid, block, 0, st, score, idx, idx_sorted, lens, rows, \
-                       nbk, k_sel)
+#define BSA_TOPK(N)                                                                                \
+    do {                                                                                           \
+        if (idx != nullptr)                                                                        \
+            hipLaunchKernelGGL((topk_kernel<S, N, true>), grid, block, 0, st, score, idx, idx_sorted, lens, rows, nbk, k_sel);  \
+        else                                                                                       \
+            hipLaunchKernelGGL((topk_kernel<S, N, false>), grid, block, 0, st, score, idx, idx_sorted, lens, rows, nbk, k_sel); \
+    } while (0)
     if (nbk <= 4 * 64) BSA_TOPK(4);
     else if (nbk <= 8 * 64) BSA_TOPK(8);
     else if (nbk <= 16 * 64) BSA_TOPK(16);
@@ -205,15 +256,13 @@ hipError_t launch_score(const void* q_cmp, const void* k_cmp, void* score, int B
         hipLaunchKernelGGL(score_f32_kernel, grid, dim3(256), 0, st, (const float*)q_cmp,
                            (const float*)k_cmp, (float*)score, nbq, nbk, D);
     } else {
-        dim3 grid((nbk + 63) / 64, (nbq + 63) / 64, BH);
+        dim3 grid((nbk + kScoreCols - 1) / kScoreCols, (nbq + 127) / 128, BH);
         if (dtype == BSA_BF16)
             hipLaunchKernelGGL((score_mfma_kernel<__bf16>), grid, dim3(256), 0, st,
-                               (const __bf16*)q_cmp, (const __bf16*)k_cmp, (__bf16*)score, nbq,
-                               nbk, D);
+                               (const __bf16*)q_cmp, (const __bf16*)k_cmp, (__bf16*)score, nbq, nbk);
         else
             hipLaunchKernelGGL((score_mfma_kernel<_Float16>), grid, dim3(256), 0, st,
-                               (const _Float16*)q_cmp, (const _Float16*)k_cmp, (_Float16*)score,
-                               nbq, nbk, D);
+                               (const _Float16*)q_cmp, (const _Float16*)k_cmp, (_Float16*)score, nbq, nbk);
     }
     return hipGetLastError();
 }
