@@ -253,7 +253,7 @@ def main():
     permute_bytes = HEADS * (S + Sp) * D * es
 
     result = {
-        "metric": "BSA fwd ms/layer + sparse TFLOPS (% bf16 MFMA peak) at 720p 86.4k tokens",
+        "metric": "BSA fwd ms/layer + sparse TFLOPS (% bf16 MFMA peak) at " + ("720p 86.4k tokens" if args.workload == "c3" else "480p 37.4k tokens"),
         "value": round(tflops_step, 2),
         "unit": "TFLOP/s (sparse-actual, whole operator)",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

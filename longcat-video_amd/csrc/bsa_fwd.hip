@@ -573,14 +573,20 @@ hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t
     }
     // One launch per round of as many work items as the device runs at once: the workgroups of a
     // launch start together and walk their (ascending) KV lists in step, so that a tile fetched
-    // by one of them is still in L2 when its neighbours ask for it.  Rounds do not straddle a
-    // (batch, head) boundary: all workgroups of a round share one head's K/V.
+    // by one of them is still in L2 when its neighbours ask for it.  Rounds normally end at a
+    // (batch, head) boundary, so that all workgroups of a round share one head's K/V; when that
+    // would leave the last round of every head mostly empty (few query tiles per head), rounds
+    // run across the boundaries instead.
     const int per_head = (int)(Sq / kTile);
     const int round = resident_workgroups();
-    for (int bh = 0; bh < B * Hn; ++bh) {
-        for (int first = 0; first < per_head; first += round) {
+    const int tail = per_head % round;
+    const bool across = tail != 0 && tail * 10 < round * 7;
+    const int n_outer = across ? 1 : B * Hn;
+    const int n_inner = across ? B * Hn * per_head : per_head;
+    for (int bh = 0; bh < n_outer; ++bh) {
+        for (int first = 0; first < n_inner; first += round) {
             const int begin = bh * per_head + first;
-            const int end = bh * per_head + (first + round < per_head ? first + round : per_head);
+            const int end = bh * per_head + (first + round < n_inner ? first + round : n_inner);
             const dim3 grid((unsigned)(end - begin));
             if (dtype == BSA_BF16)
                 hipLaunchKernelGGL((fwd_mfma_kernel<__bf16>), grid, block, 0, st, (const __bf16*)q,
