@@ -114,7 +114,7 @@ def cpu_baseline(torch, latent, sparsity, seed, rms, budget_s):
 
 
 def run_c4(torch, args):
-    """BASELINE config 4: long-video continuation, grid 48x30x52 with 12 conditioning frames.  Two operator
+    """benchmark configuration 4: long-video continuation, grid 48x30x52 with 12 conditioning frames.  Two operator
     calls per layer as in attention.py:124-135, writing into one output buffer."""
     from longcat_video_amd.block_sparse_attention import bsa_interface as I
     T, Hh, W, cond = 48, 30, 52, 12
@@ -146,7 +146,7 @@ def run_c4(torch, args):
 
 
 def run_c5(torch, args):
-    """BASELINE config 5: the attention sub-chain of one DiT block at 720p: RMSNorm -> QKV projection ->
+    """benchmark configuration 5: the attention sub-chain of one DiT block at 720p: RMSNorm -> QKV projection ->
     per-head RMSNorm + 3-D RoPE -> block-sparse attention -> output projection + residual (dim 4096)."""
     from longcat_video_amd.modules import attention as M
     latent = WORKLOADS["c3"][0]

@@ -277,7 +277,7 @@ class Attention(nn.Module):
 def attention_block_forward(x: torch.Tensor, pre_norm_weight: torch.Tensor, attn: Attention, shape,
                             num_cond_latents=None, eps: float = 1e-6) -> torch.Tensor:
     """RMSNorm -> QKV projection -> QK RMSNorm -> 3-D RoPE -> block-sparse attention -> out projection
-    -> residual: the attention sub-chain of one DiT block as BASELINE config 5 words it."""
+    -> residual: the attention sub-chain of one DiT block as benchmark configuration 5 words it."""
     y = rms_norm(x, pre_norm_weight, eps)
     return attn(y, shape=shape, num_cond_latents=num_cond_latents, residual=x)
 

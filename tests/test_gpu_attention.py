@@ -147,7 +147,7 @@ def test_large_logits_do_not_overflow():
 
 
 def test_480p_two_heads_sampled_rows():
-    """BASELINE config 2 geometry with 2 heads: 624 blocks, 39 selected per row,
+    """benchmark configuration 2 geometry with 2 heads: 624 blocks, 39 selected per row,
     checked on sampled query blocks against the gathered fp32 oracle."""
     nb, ks = 624, 39
     q, k, v = seeded_qkv(1, 1, 2, nb * 64, nb * 64, 128, torch.bfloat16)

@@ -1,5 +1,5 @@
 """R8/R9 on the GPU: the whole operator through flash_attn_bsa_3d, from the
-BASELINE configs at reduced head count up to the full 720p shape."""
+benchmark configurations at reduced head count up to the full 720p shape."""
 import math
 
 import numpy as np
@@ -149,7 +149,7 @@ def test_480p_two_heads():
 
 
 def test_long_video_continuation_two_heads():
-    """BASELINE config 4 geometry with 2 heads: grid 48x30x52, the first 12 latent frames are
+    """benchmark configuration 4 geometry with 2 heads: grid 48x30x52, the first 12 latent frames are
     conditioning tokens.  Two operator calls as in attention.py:124-135: conditioning queries
     against conditioning keys (312 blocks, 39 kept), noise queries against all keys
     (936 x 1248 blocks, 156 kept)."""
@@ -170,7 +170,7 @@ def test_long_video_continuation_two_heads():
 
 
 def test_720p_full_shape_sampled():
-    """BASELINE config 3 at full size (32 heads, 86 400 tokens, RMS-normalised q/k,
+    """benchmark configuration 3 at full size (32 heads, 86 400 tokens, RMS-normalised q/k,
     density 1/16): two heads are checked against the oracle on sampled query
     blocks; all heads for finiteness, determinism and row-stochastic bounds."""
     latent = (24, 45, 80)

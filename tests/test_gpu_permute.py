@@ -99,7 +99,7 @@ def test_pool_exact_on_representable_inputs():
 
 
 def test_full_size_720p_round_trip_and_checksum():
-    """BASELINE config 3 shape, all 32 heads: size-independent properties."""
+    """benchmark configuration 3 shape, all 32 heads: size-independent properties."""
     latent, chunk = (24, 45, 80), (4, 4, 4)
     g = torch.Generator(device="cuda").manual_seed(5)
     x = torch.randn(1, 32, 86400, 128, generator=g, device="cuda", dtype=torch.bfloat16)

@@ -98,7 +98,7 @@ def test_padded_keys_are_ignored():
 
 
 def test_config1_end_to_end_on_cpu():
-    """BASELINE config 1: B=1, 4 heads, D=128, grid 4x8x8, chunk 4x4x4, top-2 of 4, fp32."""
+    """benchmark configuration 1: B=1, 4 heads, D=128, grid 4x8x8, chunk 4x4x4, top-2 of 4, fp32."""
     q, k, v = seeded_qkv(0, 1, 4, 256, 256, 128, torch.float32)
     out, idx, lens, score = O.flash_attn_bsa_3d(q, k, v, (4, 8, 8), (4, 8, 8), sparsity=0.5,
                                                 chunk_3d_shape_q=(4, 4, 4), chunk_3d_shape_k=(4, 4, 4))
