@@ -115,6 +115,25 @@ int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32
                    int32_t* lens_out, void* score_out, int B, int Hn, int nbq, int nbk, int D,
                    int k_sel, int dtype, void* stream);
 
+/*
+ * Selection by cumulative attention mass.  Replaces get_select_indices_cdf_from_score (bsa:233-243) and, with
+ * k_min > 0, get_select_indices_cdf_topk_from_score (bsa:252-266).
+ *   weights = softmax(score * sm_scale) per row; the columns are ordered by descending score, ties towards
+ *   the lowest index; a row keeps the leading columns whose running sum of weights is <= cdf_threshold
+ *   (torch.searchsorted(cdf, threshold, right=True), bsa:241), at least k_min and at most idx_stride of them.
+ *   idx_out / idx_sorted_out  int32 [B, Hn, nbq, idx_stride], row m filled up to lens_out[m], -1 behind
+ *   (the reference returns all nbk sorted columns, of which the attention kernel reads the first lens).
+ * The weights are fp32 for every storage type and the running sum is kept in double precision: a row may
+ * differ from an fp32 running sum only where that sum comes within rounding of the threshold.
+ * Limits as for bsa_score_topk; idx_stride <= min(nbk, 1024).
+ */
+int bsa_score_cdf(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32_t* idx_sorted_out,
+                  int32_t* lens_out, void* score_out, int B, int Hn, int nbq, int nbk, int D,
+                  float cdf_threshold, float sm_scale, int k_min, int idx_stride, int dtype, void* stream);
+int bsa_cdf_from_score(const void* score, int32_t* idx_out, int32_t* idx_sorted_out, int32_t* lens_out,
+                       int B, int Hn, int nbq, int nbk, float cdf_threshold, float sm_scale, int k_min,
+                       int idx_stride, int dtype, void* stream);
+
 /* R4 alone, from a caller-supplied score tensor [B, Hn, nbq, nbk] in `dtype`. */
 int bsa_topk_from_score(const void* score, int32_t* idx_out, int32_t* idx_sorted_out, int32_t* lens_out,
                         int B, int Hn, int nbq, int nbk, int k_sel, int dtype, void* stream);
@@ -145,7 +164,9 @@ int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, con
  * _attention_bsa.forward, bsa:535-568 (cdf_threshold = None).
  *   q [B, Hn, Tq*Hq*Wq, D] with element strides q_strides = {B, Hn, S}; same
  *   for k, v; o likewise with o_strides.  k_sel from bsa_num_selected() on the
- *   padded KV block count.  workspace: bsa_workspace_bytes() bytes, 256-byte
+ *   padded KV block count.  With p->cdf_threshold > 0 the selection follows
+ *   bsa_score_cdf instead (bsa:268-277 dispatch), at most min(nbk, 1024) blocks per
+ *   row, and idx_out has that many columns.  workspace: bsa_workspace_bytes() bytes, 256-byte
  *   aligned.  idx_out/lens_out/score_out are optional copies for inspection
  *   (shapes as in bsa_score_topk).
  * For bf16 / fp16 no permuted copy of q, k, v or o is made: one pass over q and k
@@ -157,8 +178,9 @@ typedef struct bsa_3d_params {
     int B, Hn, D, dtype;
     int Tq, Hq, Wq, Tk, Hk, Wk;      /* latent grids */
     int tq, hq, wq, tk, hk, wk;      /* chunk shapes */
-    int k_sel;
+    int k_sel;                       /* top-k count; with cdf_threshold > 0: the minimum per row (0 = none) */
     float sm_scale;
+    float cdf_threshold;             /* > 0 selects by cumulative attention mass (bsa_score_cdf), else top-k */
 } bsa_3d_params;
 
 size_t bsa_workspace_bytes(const bsa_3d_params* p);

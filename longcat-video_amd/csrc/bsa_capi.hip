@@ -148,13 +148,51 @@ int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32
     if (!q_cmp || !k_cmp || !lens_out || (!idx_out && !idx_sorted_out)) return set_error(BSA_ERR_BAD_ARG, "score_topk: null pointer");
     if (!score_out) return set_error(BSA_ERR_BAD_ARG, "score_topk: a score buffer of B*heads*nbq*nbk elements is required");
     BSA_TRY(check_topk(B, Hn, nbq, nbk, k_sel, dtype));
-    if (D <= 0 || D % 16 != 0 || D > 256) return set_error(BSA_ERR_UNSUPPORTED, "score: head dim %d must be a multiple of 16, at most 256", D);
+    if (D != 128) return set_error(BSA_ERR_UNSUPPORTED, "score: head dim %d is not built (only 128)", D);
     if ((int64_t)B * Hn > 65535) return set_error(BSA_ERR_UNSUPPORTED, "B*heads exceeds 65535");
     if (!aligned16(q_cmp) || !aligned16(k_cmp)) return set_error(BSA_ERR_BAD_ARG, "score: pooled tensors must be 16-byte aligned");
     hipError_t e = launch_score(q_cmp, k_cmp, score_out, B * Hn, nbq, nbk, D, dtype, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "score launch");
     e = launch_topk(score_out, idx_out, idx_sorted_out, lens_out, (int64_t)B * Hn * nbq, nbk, k_sel, dtype, (hipStream_t)stream);
     return e == hipSuccess ? BSA_OK : hip_fail(e, "top-k launch");
+}
+
+static int check_cdf(float thr, float scale, int k_min, int idx_stride, int nbk) {
+    if (!(thr > 0.f) || !std::isfinite(thr)) return set_error(BSA_ERR_BAD_ARG, "cdf: threshold must be positive and finite");
+    if (!(scale > 0.f) || !std::isfinite(scale)) return set_error(BSA_ERR_BAD_ARG, "cdf: sm_scale must be positive and finite");
+    if (idx_stride <= 0 || idx_stride > nbk || idx_stride > 1024)
+        return set_error(BSA_ERR_SHAPE, "cdf: idx_stride=%d outside [1, min(%d, 1024)]", idx_stride, nbk);
+    if (k_min < 0 || k_min > idx_stride) return set_error(BSA_ERR_SHAPE, "cdf: k_min=%d outside [0, %d]", k_min, idx_stride);
+    return BSA_OK;
+}
+
+int bsa_cdf_from_score(const void* score, int32_t* idx_out, int32_t* idx_sorted_out, int32_t* lens_out, int B, int Hn,
+                       int nbq, int nbk, float cdf_threshold, float sm_scale, int k_min, int idx_stride, int dtype,
+                       void* stream) {
+    if (!score || !lens_out || (!idx_out && !idx_sorted_out)) return set_error(BSA_ERR_BAD_ARG, "cdf: null pointer");
+    BSA_TRY(check_topk(B, Hn, nbq, nbk, 0, dtype));
+    BSA_TRY(check_cdf(cdf_threshold, sm_scale, k_min, idx_stride, nbk));
+    const int64_t rows = (int64_t)B * Hn * nbq;
+    hipError_t e = launch_cdf_count(score, lens_out, rows, nbk, cdf_threshold, sm_scale, k_min, idx_stride, dtype, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "cdf count launch");
+    e = launch_topk(score, idx_out, idx_sorted_out, lens_out, rows, nbk, 0, dtype, (hipStream_t)stream, lens_out, idx_stride);
+    return e == hipSuccess ? BSA_OK : hip_fail(e, "top-k launch");
+}
+
+int bsa_score_cdf(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32_t* idx_sorted_out, int32_t* lens_out,
+                  void* score_out, int B, int Hn, int nbq, int nbk, int D, float cdf_threshold, float sm_scale, int k_min,
+                  int idx_stride, int dtype, void* stream) {
+    if (!q_cmp || !k_cmp || !lens_out || (!idx_out && !idx_sorted_out)) return set_error(BSA_ERR_BAD_ARG, "score_cdf: null pointer");
+    if (!score_out) return set_error(BSA_ERR_BAD_ARG, "score_cdf: a score buffer of B*heads*nbq*nbk elements is required");
+    BSA_TRY(check_topk(B, Hn, nbq, nbk, 0, dtype));
+    BSA_TRY(check_cdf(cdf_threshold, sm_scale, k_min, idx_stride, nbk));
+    if (D != 128) return set_error(BSA_ERR_UNSUPPORTED, "score: head dim %d is not built (only 128)", D);
+    if ((int64_t)B * Hn > 65535) return set_error(BSA_ERR_UNSUPPORTED, "B*heads exceeds 65535");
+    if (!aligned16(q_cmp) || !aligned16(k_cmp)) return set_error(BSA_ERR_BAD_ARG, "score: pooled tensors must be 16-byte aligned");
+    const hipError_t e = launch_score(q_cmp, k_cmp, score_out, B * Hn, nbq, nbk, D, dtype, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "score launch");
+    return bsa_cdf_from_score(score_out, idx_out, idx_sorted_out, lens_out, B, Hn, nbq, nbk, cdf_threshold, sm_scale, k_min,
+                              idx_stride, dtype, stream);
 }
 
 int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, const int32_t* lens,
@@ -186,6 +224,8 @@ struct Plan {
     Grid3 gq, gk;
     int64_t Sqp, Skp;
     int nbq, nbk, es;
+    int sel_width;        // columns of the index lists: k_sel, or the cap of the CDF rule
+    bool cdf;
     bool direct_qo, direct_kv;
     size_t off_qp, off_kp, off_vp, off_op, off_qc, off_kc, off_score, off_idx, off_idx_sorted, off_lens, off_valid, off_qrows, off_ktiles, total;
 };
@@ -204,6 +244,9 @@ int make_plan(const bsa_3d_params* p, Plan* pl) {
     pl->nbq = pl->gq.blocks();
     pl->nbk = pl->gk.blocks();
     BSA_TRY(check_topk(p->B, p->Hn, pl->nbq, pl->nbk, p->k_sel, p->dtype));
+    pl->cdf = p->cdf_threshold > 0.f;
+    pl->sel_width = pl->cdf ? (pl->nbk < 1024 ? pl->nbk : 1024) : p->k_sel;
+    if (pl->cdf && !std::isfinite(p->cdf_threshold)) return set_error(BSA_ERR_BAD_ARG, "cdf_threshold must be finite");
     if (!(p->sm_scale > 0.f) || !std::isfinite(p->sm_scale)) return set_error(BSA_ERR_BAD_ARG, "sm_scale must be positive and finite");
     pl->Sqp = (int64_t)pl->nbq * pl->gq.chunk();
     pl->Skp = (int64_t)pl->nbk * pl->gk.chunk();
@@ -224,8 +267,8 @@ int make_plan(const bsa_3d_params* p, Plan* pl) {
     pl->off_qc = take(bh * pl->nbq * p->D * pl->es);
     pl->off_kc = take(bh * pl->nbk * p->D * pl->es);
     pl->off_score = take(bh * pl->nbq * (size_t)pl->nbk * pl->es);
-    pl->off_idx = take(bh * pl->nbq * (size_t)(p->k_sel > 0 ? p->k_sel : 1) * sizeof(int32_t));
-    pl->off_idx_sorted = take(bh * pl->nbq * (size_t)(p->k_sel > 0 ? p->k_sel : 1) * sizeof(int32_t));
+    pl->off_idx = take(bh * pl->nbq * (size_t)(pl->sel_width > 0 ? pl->sel_width : 1) * sizeof(int32_t));
+    pl->off_idx_sorted = take(bh * pl->nbq * (size_t)(pl->sel_width > 0 ? pl->sel_width : 1) * sizeof(int32_t));
     pl->off_lens = take(bh * pl->nbq * sizeof(int32_t));
     pl->off_valid = take((size_t)(pl->Skp / 64) * sizeof(uint64_t));
     pl->off_qrows = take(pl->direct_qo ? (size_t)pl->Sqp * sizeof(int32_t) : 0);
@@ -393,18 +436,25 @@ int bsa_fwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3]
     BSA_HIP(launch_score(w.qc, w.kc, w.score, p->B * p->Hn, pl.nbq, pl.nbk, p->D, p->dtype, st), "score");
     // the attention kernel walks each list in ascending block order (L2 locality); the score
     // order is only produced when the caller asks for the selection
-    BSA_HIP(launch_topk(w.score, idx_out ? w.idx : nullptr, w.idx_sorted, w.lens, (int64_t)p->B * p->Hn * pl.nbq, pl.nbk, p->k_sel, p->dtype, st), "top-k");
+    const int64_t sel_rows = (int64_t)p->B * p->Hn * pl.nbq;
+    if (pl.cdf) {
+        BSA_HIP(launch_cdf_count(w.score, w.lens, sel_rows, pl.nbk, p->cdf_threshold, p->sm_scale, p->k_sel < pl.sel_width ? p->k_sel : pl.sel_width,
+                                 pl.sel_width, p->dtype, st), "cdf count");
+        BSA_HIP(launch_topk(w.score, idx_out ? w.idx : nullptr, w.idx_sorted, w.lens, sel_rows, pl.nbk, 0, p->dtype, st, w.lens, pl.sel_width), "top-k");
+    } else {
+        BSA_HIP(launch_topk(w.score, idx_out ? w.idx : nullptr, w.idx_sorted, w.lens, sel_rows, pl.nbk, p->k_sel, p->dtype, st), "top-k");
+    }
     if (pl.direct_qo) {
-        BSA_HIP(attention_thw(pl, p, w, q, q_strides, k, k_strides, v, v_strides, o, o_strides, w.idx_sorted, w.lens, p->k_sel,
+        BSA_HIP(attention_thw(pl, p, w, q, q_strides, k, k_strides, v, v_strides, o, o_strides, w.idx_sorted, w.lens, pl.sel_width,
                               nullptr, st), "attention");
     } else {
         BSA_HIP(launch_fwd(w.qp, w.kp, w.vp, w.idx_sorted, w.lens, padded_k ? w.valid : nullptr, w.op, nullptr, p->B, p->Hn, pl.Sqp, pl.Skp,
-                           pl.gq.chunk(), pl.gk.chunk(), p->k_sel, p->sm_scale, p->dtype, st), "attention");
+                           pl.gq.chunk(), pl.gk.chunk(), pl.sel_width, p->sm_scale, p->dtype, st), "attention");
         BSA_HIP(launch_unpermute(w.op, o, o_strides, p->B, p->Hn, pl.gq, p->D, p->dtype, st), "unpermute");
     }
     const size_t bh = (size_t)p->B * p->Hn;
-    if (idx_out && p->k_sel > 0)
-        BSA_HIP(hipMemcpyAsync(idx_out, w.idx, bh * pl.nbq * p->k_sel * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy idx");
+    if (idx_out && pl.sel_width > 0)
+        BSA_HIP(hipMemcpyAsync(idx_out, w.idx, bh * pl.nbq * pl.sel_width * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy idx");
     if (lens_out) BSA_HIP(hipMemcpyAsync(lens_out, w.lens, bh * pl.nbq * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy lens");
     if (score_out) BSA_HIP(hipMemcpyAsync(score_out, w.score, bh * pl.nbq * (size_t)pl.nbk * pl.es, hipMemcpyDeviceToDevice, st), "copy score");
 #undef BSA_HIP

@@ -110,8 +110,14 @@ hipError_t launch_mean_pool(const void* x, void* out, int B, int Hn, int64_t S, 
 hipError_t launch_score(const void* q_cmp, const void* k_cmp, void* score, int BH, int nbq, int nbk,
                         int D, int dtype, hipStream_t st);
 // idx: descending score order; idx_sorted: ascending block index; either may be null
+// k_rows: one count per row instead of k_sel (may alias lens); stride: row pitch of idx / idx_sorted
+// (default k_sel), entries past a row's count are set to -1
 hipError_t launch_topk(const void* score, int32_t* idx, int32_t* idx_sorted, int32_t* lens, int64_t rows,
-                       int nbk, int k_sel, int dtype, hipStream_t st);
+                       int nbk, int k_sel, int dtype, hipStream_t st, const int32_t* k_rows = nullptr,
+                       int stride = 0);
+// lens[row] = number of columns the CDF rule keeps, clamped to [k_min, cap]
+hipError_t launch_cdf_count(const void* score, int32_t* lens, int64_t rows, int nbk, float threshold,
+                            float scale, int k_min, int cap, int dtype, hipStream_t st);
 hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t* idx,
                       const int32_t* lens, const uint64_t* tile_valid, void* o, float* lse,
                       int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride,

@@ -158,14 +158,22 @@ __global__ __launch_bounds__(256) void topk_kernel(const S* __restrict__ score,
                                                    int32_t* __restrict__ idx_out,
                                                    int32_t* __restrict__ idx_sorted_out,
                                                    int32_t* __restrict__ lens_out, int64_t rows,
-                                                   int nbk, int k_sel) {
+                                                   int nbk, int k_all, const int32_t* __restrict__ k_rows,
+                                                   int stride) {
     typedef typename KeyOf<S>::type K;
     constexpr int kValueBits = 8 * (int)sizeof(S);
     __shared__ K sel[4][kMaxSel];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + wave;
     if (row >= rows) return;
+    // the number of columns to keep: the same for every row, or one count per row (k_rows may be lens_out)
+    const int k_sel = k_rows != nullptr ? k_rows[row] : k_all;
     if (lane == 0) lens_out[row] = k_sel;
+    // unused tail of the row's lists
+    for (int e = k_sel + lane; e < stride; e += 64) {
+        if (idx_out) idx_out[row * stride + e] = -1;
+        if (idx_sorted_out) idx_sorted_out[row * stride + e] = -1;
+    }
     if (k_sel == 0) return;
 
     const S* srow = score + row * nbk;
@@ -208,7 +216,7 @@ __global__ __launch_bounds__(256) void topk_kernel(const S* __restrict__ score,
         const uint64_t m = __ballot(win);
         if (win) {
             const int p = pos + __popcll(m & lt);
-            if (idx_sorted_out) idx_sorted_out[row * k_sel + p] = i;          // column order = ascending block order
+            if (idx_sorted_out) idx_sorted_out[row * stride + p] = i;         // column order = ascending block order
             if (SCORE_ORDER) mine[p] = KeyOf<S>::make(srow[i], i);
         }
         pos += __popcll(m);
@@ -222,20 +230,123 @@ __global__ __launch_bounds__(256) void topk_kernel(const S* __restrict__ score,
         const K me = mine[e];
         int rank = 0;
         for (int o = 0; o < k_sel; ++o) rank += mine[o] > me;
-        idx_out[row * k_sel + rank] = KeyOf<S>::index(me);
+        idx_out[row * stride + rank] = KeyOf<S>::index(me);
     }
+}
+
+// ---------------------------------------------------------------- CDF rule
+__device__ inline float score_value(uint16_t s, int dtype) {
+    if (dtype == BSA_F16) return (float)__builtin_bit_cast(_Float16, s);
+    return __uint_as_float((uint32_t)s << 16);
+}
+__device__ inline float score_value(uint32_t s, int) { return __uint_as_float(s); }
+__device__ inline double wave_sum(double x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+    return x;
+}
+
+// How many columns the CDF rule keeps per row: with the columns sorted by descending score (ties towards
+// the lowest index) and weights softmax(score * scale), the number of leading columns whose running sum
+// of weights stays at or below `threshold`; never fewer than k_min (the "cdf + top-k" rule) and never
+// more than `cap`.  One wavefront per row.  Sums run in double precision on the unnormalised weights
+// e_i = exp((s_i - max) * scale): sum_top(e) <= threshold * sum_all(e).  The columns at or above a score
+// value t form a prefix of the sorted order, so a bitwise binary search over t finds the value group in
+// which the running sum crosses the threshold; inside that group every column weighs the same.
+template <typename S, int NPL>
+__global__ __launch_bounds__(256) void cdf_count_kernel(const S* __restrict__ score, int32_t* __restrict__ lens_out,
+                                                        int64_t rows, int nbk, float threshold, float scale, int k_min,
+                                                        int cap, int dtype) {
+    constexpr int kValueBits = 8 * (int)sizeof(S);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    if (row >= rows) return;
+    const S* srow = score + row * nbk;
+    uint32_t val[NPL];
+    float e[NPL];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < NPL; ++j) {
+        const int i = j * 64 + lane;
+        const S raw = srow[min(i, nbk - 1)];
+        val[j] = i < nbk ? ord_of(raw) : 0u;
+        e[j] = i < nbk ? score_value(raw, dtype) : -INFINITY;
+        mx = fmaxf(mx, e[j]);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    double total = 0.0;
+#pragma unroll
+    for (int j = 0; j < NPL; ++j) {
+        e[j] = j * 64 + lane < nbk ? expf((e[j] - mx) * scale) : 0.f;
+        total += (double)e[j];
+    }
+    total = wave_sum(total);
+    const double budget = (double)threshold * total;
+    // largest t whose columns at or above t outweigh the budget (t = 0: all columns, if even that holds)
+    auto mass_ge = [&](uint32_t t) {
+        double m = 0.0;
+#pragma unroll
+        for (int j = 0; j < NPL; ++j) m += val[j] >= t ? (double)e[j] : 0.0;     // padding has e = 0
+        return wave_sum(m);
+    };
+    int n;
+    if (!(total > budget)) {
+        n = nbk;                                  // threshold >= 1: everything
+    } else {
+        uint32_t thr = 0;
+        for (int bit = kValueBits - 1; bit >= 0; --bit) {
+            const uint32_t cand = thr | (1u << bit);
+            if (mass_ge(cand) > budget) thr = cand;
+        }
+        // columns above thr fit; the group equal to thr crosses: take as many of it as still fit
+        double above = 0.0, one = 0.0;
+        int cnt_gt = 0, cnt_eq = 0;
+#pragma unroll
+        for (int j = 0; j < NPL; ++j) {
+            const bool real = j * 64 + lane < nbk;
+            above += val[j] > thr ? (double)e[j] : 0.0;
+            cnt_gt += __popcll(__ballot(val[j] > thr));
+            const bool eq = real && val[j] == thr;
+            cnt_eq += __popcll(__ballot(eq));
+            if (eq) one = (double)e[j];
+        }
+        above = wave_sum(above);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) one = fmax(one, __shfl_xor(one, o));
+        int fit = one > 0.0 ? (int)floor((budget - above) / one) : cnt_eq;
+        fit = max(0, min(fit, cnt_eq));
+        n = cnt_gt + fit;
+    }
+    n = min(max(n, k_min), min(cap, nbk));
+    if (lane == 0) lens_out[row] = n;
+}
+
+template <typename S>
+hipError_t launch_cdf_count_t(const S* score, int32_t* lens, int64_t rows, int nbk, float threshold, float scale,
+                              int k_min, int cap, int dtype, hipStream_t st) {
+    dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+#define BSA_CDF(N) hipLaunchKernelGGL((cdf_count_kernel<S, N>), grid, block, 0, st, score, lens, rows, nbk, threshold, scale, k_min, cap, dtype)
+    if (nbk <= 4 * 64) BSA_CDF(4);
+    else if (nbk <= 8 * 64) BSA_CDF(8);
+    else if (nbk <= 16 * 64) BSA_CDF(16);
+    else if (nbk <= 24 * 64) BSA_CDF(24);
+    else if (nbk <= 32 * 64) BSA_CDF(32);
+    else BSA_CDF(64);
+#undef BSA_CDF
+    return hipGetLastError();
 }
 
 template <typename S>
 hipError_t launch_topk_t(const S* score, int32_t* idx, int32_t* idx_sorted, int32_t* lens, int64_t rows,
-                         int nbk, int k_sel, hipStream_t st) {
+                         int nbk, int k_sel, const int32_t* k_rows, int stride, hipStream_t st) {
     dim3 grid((unsigned)((rows + 3) / 4)), block(256);
 #define BSA_TOPK(N)                                                                                \
     do {                                                                                           \
         if (idx != nullptr)                                                                        \
-            hipLaunchKernelGGL((topk_kernel<S, N, true>), grid, block, 0, st, score, idx, idx_sorted, lens, rows, nbk, k_sel);  \
+            hipLaunchKernelGGL((topk_kernel<S, N, true>), grid, block, 0, st, score, idx, idx_sorted, lens, rows, nbk, k_sel, k_rows, stride);  \
         else                                                                                       \
-            hipLaunchKernelGGL((topk_kernel<S, N, false>), grid, block, 0, st, score, idx, idx_sorted, lens, rows, nbk, k_sel); \
+            hipLaunchKernelGGL((topk_kernel<S, N, false>), grid, block, 0, st, score, idx, idx_sorted, lens, rows, nbk, k_sel, k_rows, stride); \
     } while (0)
     if (nbk <= 4 * 64) BSA_TOPK(4);
     else if (nbk <= 8 * 64) BSA_TOPK(8);
@@ -268,10 +379,18 @@ hipError_t launch_score(const void* q_cmp, const void* k_cmp, void* score, int B
 }
 
 hipError_t launch_topk(const void* score, int32_t* idx, int32_t* idx_sorted, int32_t* lens, int64_t rows,
-                       int nbk, int k_sel, int dtype, hipStream_t st) {
+                       int nbk, int k_sel, int dtype, hipStream_t st, const int32_t* k_rows, int stride) {
+    if (stride <= 0) stride = k_sel;
     if (dtype == BSA_F32)
-        return launch_topk_t<uint32_t>((const uint32_t*)score, idx, idx_sorted, lens, rows, nbk, k_sel, st);
-    return launch_topk_t<uint16_t>((const uint16_t*)score, idx, idx_sorted, lens, rows, nbk, k_sel, st);
+        return launch_topk_t<uint32_t>((const uint32_t*)score, idx, idx_sorted, lens, rows, nbk, k_sel, k_rows, stride, st);
+    return launch_topk_t<uint16_t>((const uint16_t*)score, idx, idx_sorted, lens, rows, nbk, k_sel, k_rows, stride, st);
+}
+
+hipError_t launch_cdf_count(const void* score, int32_t* lens, int64_t rows, int nbk, float threshold, float scale,
+                            int k_min, int cap, int dtype, hipStream_t st) {
+    if (dtype == BSA_F32)
+        return launch_cdf_count_t<uint32_t>((const uint32_t*)score, lens, rows, nbk, threshold, scale, k_min, cap, dtype, st);
+    return launch_cdf_count_t<uint16_t>((const uint16_t*)score, lens, rows, nbk, threshold, scale, k_min, cap, dtype, st);
 }
 
 }  // namespace bsa

@@ -23,7 +23,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libb
 class Bsa3dParams(C.Structure):
     _fields_ = [(n, C.c_int) for n in (
         "B", "Hn", "D", "dtype", "Tq", "Hq", "Wq", "Tk", "Hk", "Wk",
-        "tq", "hq", "wq", "tk", "hk", "wk", "k_sel")] + [("sm_scale", C.c_float)]
+        "tq", "hq", "wq", "tk", "hk", "wk", "k_sel")] + [("sm_scale", C.c_float), ("cdf_threshold", C.c_float)]
 
 
 _i, _i64, _p, _f = C.c_int, C.c_int64, C.c_void_p, C.c_float
@@ -40,6 +40,8 @@ SIGNATURES = {
     "bsa_mean_pool": (_i, [_p, _p, _i, _i, _i64, _i, _i, _i, _p]),
     "bsa_score_topk": (_i, [_p, _p, _p, _p, _p, _p] + [_i] * 7 + [_p]),
     "bsa_topk_from_score": (_i, [_p, _p, _p, _p] + [_i] * 6 + [_p]),
+    "bsa_score_cdf": (_i, [_p, _p, _p, _p, _p, _p] + [_i] * 5 + [_f, _f, _i, _i, _i, _p]),
+    "bsa_cdf_from_score": (_i, [_p, _p, _p, _p] + [_i] * 4 + [_f, _f, _i, _i, _i, _p]),
     "bsa_fwd": (_i, [_p] * 8 + [_i, _i, _i64, _i64, _i, _i, _i, _i, _f, _i, _p]),
     "bsa_workspace_bytes": (C.c_size_t, [C.POINTER(Bsa3dParams)]),
     "bsa_fwd_3d": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,

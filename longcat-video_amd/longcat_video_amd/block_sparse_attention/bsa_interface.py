@@ -181,13 +181,90 @@ def get_select_indices_topk(q: torch.Tensor, k: torch.Tensor, sparsity: float):
     return idx.long(), lens
 
 
+def _cdf_width(nbk: int) -> int:
+    return min(int(nbk), 1024)       # columns kept per row at most
+
+
+def _select_cdf(score, q_cmp, k_cmp, cdf_threshold, sm_scale, k_min, order="score"):
+    """CDF rule on a given score tensor, or on pooled q/k (score is then computed too)."""
+    lib = _capi.load()
+    if score is not None:
+        _need_gpu(score)
+        score = score.contiguous()
+        B, H, nbq, nbk = score.shape
+        dev, dt = score.device, score
+    else:
+        _need_gpu(q_cmp, k_cmp)
+        q_cmp, k_cmp = q_cmp.contiguous(), k_cmp.contiguous()
+        B, H, nbq, D = q_cmp.shape
+        nbk = k_cmp.shape[2]
+        dev, dt = q_cmp.device, q_cmp
+        score = torch.empty(B, H, nbq, nbk, dtype=q_cmp.dtype, device=dev)
+    width = _cdf_width(nbk)
+    idx = torch.empty(B, H, nbq, width, dtype=torch.int32, device=dev)
+    lens = torch.empty(B, H, nbq, dtype=torch.int32, device=dev)
+    a, b = (_ptr(idx), None) if order == "score" else (None, _ptr(idx))
+    with torch.cuda.device(dev):
+        if q_cmp is None:
+            _capi.check(lib.bsa_cdf_from_score(_ptr(score), a, b, _ptr(lens), B, H, nbq, nbk, float(cdf_threshold),
+                                               float(sm_scale), int(k_min), width, _code(dt), _stream(dt)), "cdf")
+        else:
+            _capi.check(lib.bsa_score_cdf(_ptr(q_cmp), _ptr(k_cmp), a, b, _ptr(lens), _ptr(score), B, H, nbq, nbk,
+                                          q_cmp.shape[3], float(cdf_threshold), float(sm_scale), int(k_min), width,
+                                          _code(dt), _stream(dt)), "score_cdf")
+    return idx, lens, score
+
+
+def get_select_indices_cdf_from_score(score: torch.Tensor, cdf_threshold: float, sm_scale: float):
+    """bsa_interface.py:233-243.  Indices int64 [B,H,nbq,min(nbk,1024)]: row m holds its selection in
+    descending score order up to lens[m] and -1 behind (the reference returns all nbk sorted columns, of
+    which only the first lens[m] are ever read); lens int32."""
+    idx, lens, _ = _select_cdf(score, None, None, cdf_threshold, sm_scale, 0)
+    return idx.long(), lens
+
+
+def get_select_indices_cdf(q: torch.Tensor, k: torch.Tensor, cdf_threshold: float):
+    """bsa_interface.py:226-231."""
+    idx, lens, _ = _select_cdf(None, q, k, cdf_threshold, 1 / q.shape[-1] ** 0.5, 0)
+    return idx.long(), lens
+
+
+def get_select_indices_cdf_topk_from_score(score: torch.Tensor, sparsity: float, cdf_threshold: float, sm_scale: float):
+    """bsa_interface.py:252-266: the CDF rule, but never fewer blocks than top-k would keep."""
+    idx, lens, _ = _select_cdf(score, None, None, cdf_threshold, sm_scale,
+                               min(num_selected(sparsity, score.shape[-1]), _cdf_width(score.shape[-1])))
+    return idx.long(), lens
+
+
+def get_select_indices_cdf_topk(q: torch.Tensor, k: torch.Tensor, sparsity: float, cdf_threshold: float):
+    """bsa_interface.py:245-250."""
+    idx, lens, _ = _select_cdf(None, q, k, cdf_threshold, 1 / q.shape[-1] ** 0.5,
+                               min(num_selected(sparsity, k.shape[2]), _cdf_width(k.shape[2])))
+    return idx.long(), lens
+
+
 def get_select_indices(q, k, sparsity, cdf_threshold):
     """bsa_interface.py:268-277."""
     if sparsity is not None and cdf_threshold is None:
         return get_select_indices_topk(q, k, sparsity)
-    if sparsity is None and cdf_threshold is None:
-        raise ValueError
-    raise NotImplementedError("CDF-threshold selection is not built; pass cdf_threshold=None")
+    if sparsity is None and cdf_threshold is not None:
+        return get_select_indices_cdf(q, k, cdf_threshold)
+    if sparsity is not None and cdf_threshold is not None:
+        return get_select_indices_cdf_topk(q, k, sparsity, cdf_threshold)
+    raise ValueError
+
+
+def get_select_indices_from_score(score, sparsity, cdf_threshold, sm_scale=None):
+    """bsa_interface.py:279-288.  The reference forgets to pass sm_scale to its CDF helpers there (a TypeError
+    at :283 and :285); here it is an argument, defaulting to 1/sqrt(128)."""
+    sm_scale = 1 / 128 ** 0.5 if sm_scale is None else sm_scale
+    if sparsity is not None and cdf_threshold is None:
+        return get_select_indices_topk_from_score(score, sparsity)
+    if sparsity is None and cdf_threshold is not None:
+        return get_select_indices_cdf_from_score(score, cdf_threshold, sm_scale)
+    if sparsity is not None and cdf_threshold is not None:
+        return get_select_indices_cdf_topk_from_score(score, sparsity, cdf_threshold, sm_scale)
+    raise ValueError
 
 
 # ---------------------------------------------------------------------------
@@ -231,8 +308,10 @@ def flash_attn_bsa(q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold,
     if sparsity is None and cdf_threshold is None:
         raise ValueError
     if cdf_threshold is not None:
-        raise NotImplementedError("CDF-threshold selection is not built; pass cdf_threshold=None")
-    idx, lens, _ = _score_topk(q_cmp, k_cmp, num_selected(sparsity, k_cmp.shape[2]), order="block")
+        k_min = 0 if sparsity is None else min(num_selected(sparsity, k_cmp.shape[2]), _cdf_width(k_cmp.shape[2]))
+        idx, lens, _ = _select_cdf(None, q_cmp, k_cmp, cdf_threshold, 1 / D ** 0.5, k_min, order="block")   # bsa:229, 248
+    else:
+        idx, lens, _ = _score_topk(q_cmp, k_cmp, num_selected(sparsity, k_cmp.shape[2]), order="block")
     o, _ = attn_fwd_bsa_varlen(q, k, v, sm_scale, idx, lens, chunk_size_q, chunk_size_k, sparsity, tile_valid)
     return o
 
@@ -240,8 +319,10 @@ def flash_attn_bsa(q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold,
 # ---------------------------------------------------------------------------
 # R9: the operator
 # ---------------------------------------------------------------------------
-def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k, want_selection=False, out=None):
-    """`out`: optional [B,H,Sq,D] view (any B/H/S strides, contiguous D) to write into."""
+def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k, want_selection=False, out=None,
+            cdf_threshold=None):
+    """`out`: optional [B,H,Sq,D] view (any B/H/S strides, contiguous D) to write into.  `sparsity` may be
+    None when `cdf_threshold` is given (bsa_interface.py:268-277)."""
     _need_gpu(q, k, v)
     B, H, Sq, D = q.shape
     Tq, Hq, Wq = (int(x) for x in latent_shape_q)
@@ -256,9 +337,13 @@ def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k,
         k, v = k.contiguous(), v.contiguous()
     nbk = lib.bsa_padded_tokens(Tk, Hk, Wk, tk, hk, wk) // (tk * hk * wk)
     nbq = lib.bsa_padded_tokens(Tq, Hq, Wq, tq, hq, wq) // (tq * hq * wq)
-    k_sel = num_selected(sparsity, nbk)
+    k_sel = 0 if sparsity is None else num_selected(sparsity, nbk)
+    width = k_sel
+    if cdf_threshold is not None:
+        width = _cdf_width(nbk)
+        k_sel = min(k_sel, width)
     prm = _capi.Bsa3dParams(B, H, D, _code(q), Tq, Hq, Wq, Tk, Hk, Wk, tq, hq, wq, tk, hk, wk, k_sel,
-                            1.0 / D ** 0.5)
+                            1.0 / D ** 0.5, 0.0 if cdf_threshold is None else float(cdf_threshold))
     need = lib.bsa_workspace_bytes(C.byref(prm))
     if need == 0:
         _capi.check(lib.bsa_fwd_3d(C.byref(prm), None, None, None, None, None, None, None, None, None, 0,
@@ -268,7 +353,7 @@ def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k,
     assert o.shape == (B, H, Sq, D) and o.dtype == q.dtype and o.stride(3) == 1
     idx = lens = score = None
     if want_selection:
-        idx = torch.empty(B, H, nbq, k_sel, dtype=torch.int32, device=q.device)
+        idx = torch.empty(B, H, nbq, width, dtype=torch.int32, device=q.device)
         lens = torch.empty(B, H, nbq, dtype=torch.int32, device=q.device)
         score = torch.empty(B, H, nbq, nbk, dtype=q.dtype, device=q.device)
     with torch.cuda.device(q.device):
@@ -339,13 +424,15 @@ def attn_fwd_bsa_thw(q, k, v, latent_shape_q, latent_shape_k, chunk_3d_shape_q, 
 
 @torch.library.custom_op("longcat_video_amd::flash_attn_bsa_3d", mutates_args=())
 def _bsa_3d_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, latent_shape_q: Sequence[int],
-               latent_shape_k: Sequence[int], sparsity: float, chunk_3d_shape_q: Sequence[int],
+               latent_shape_k: Sequence[int], sparsity: float, cdf_threshold: float, chunk_3d_shape_q: Sequence[int],
                chunk_3d_shape_k: Sequence[int]) -> torch.Tensor:
-    return _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_3d_shape_q, chunk_3d_shape_k)
+    # a negative sparsity / cdf_threshold stands for None (operator schemas have no optional floats here)
+    return _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, None if sparsity < 0 else sparsity, chunk_3d_shape_q,
+                   chunk_3d_shape_k, cdf_threshold=None if cdf_threshold < 0 else cdf_threshold)
 
 
 @_bsa_3d_op.register_fake
-def _(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_3d_shape_q, chunk_3d_shape_k):
+def _(q, k, v, latent_shape_q, latent_shape_k, sparsity, cdf_threshold, chunk_3d_shape_q, chunk_3d_shape_k):
     return q.new_empty(q.shape)
 
 
@@ -381,8 +468,7 @@ def flash_attn_bsa_3d(
     assert head_dim_q in {16, 32, 64, 128, 256}
     if sparsity is None and cdf_threshold is None:
         raise ValueError
-    if cdf_threshold is not None:
-        raise NotImplementedError("CDF-threshold selection is not built; pass cdf_threshold=None")
     _no_grad(q, k, v)
     return _bsa_3d_op(q, k, v, [int(x) for x in latent_shape_q], [int(x) for x in latent_shape_k],
-                      float(sparsity), [int(x) for x in chunk_3d_shape_q], [int(x) for x in chunk_3d_shape_k])
+                      -1.0 if sparsity is None else float(sparsity), -1.0 if cdf_threshold is None else float(cdf_threshold),
+                      [int(x) for x in chunk_3d_shape_q], [int(x) for x in chunk_3d_shape_k])

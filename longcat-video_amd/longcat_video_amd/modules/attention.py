@@ -196,12 +196,10 @@ class Attention(nn.Module):
         Tq, Tk = SQ // (Hh * W), SKV // (Hh * W)
         prm = dict(sparsity=0.875, cdf_threshold=None, chunk_3d_shape_q=[4, 4, 8], chunk_3d_shape_k=[4, 4, 8])
         prm.update(self.bsa_params)
-        if prm["cdf_threshold"] is not None:
-            raise NotImplementedError("CDF-threshold selection is not built; pass cdf_threshold=None")
-        if prm["sparsity"] is None:
+        if prm["sparsity"] is None and prm["cdf_threshold"] is None:
             raise ValueError
-        return _bsa_3d(q, k, v, (Tq, Hh, W), (Tk, Hh, W), float(prm["sparsity"]), prm["chunk_3d_shape_q"],
-                       prm["chunk_3d_shape_k"], out=out)
+        return _bsa_3d(q, k, v, (Tq, Hh, W), (Tk, Hh, W), prm["sparsity"], prm["chunk_3d_shape_q"],
+                       prm["chunk_3d_shape_k"], out=out, cdf_threshold=prm["cdf_threshold"])
 
     def _project_qkv(self, x):
         B, N, C = x.shape

@@ -33,12 +33,25 @@ fixtures for this path, so the pins are mathematical; see tests/test_oracle_*):
                                     LSE-merge identity; order invariance
   rms_norm / rope_3d_*              norm preservation, relative-position
                                     property, closed-form frequencies
+  select_cdf                        closed forms (equal scores, one dominant
+                                    column, log-weights), a Python loop, and
+                                    the reference's own library sequence
+                                    (softmax, sort, cumsum, searchsorted) on
+                                    tie-free fp32 scores
+  attention_module_forward_with_kv_cache / attention_module_kv
+                                    equality with the noise rows of the split
+                                    forward over all frames
+  layernorm_modulate_fp32 / gated_residual_fp32
+                                    torch F.layer_norm, closed forms
 
 What no CPU check can pin ("parity unpinned", because the reference executes
 them inside un-vendored third parties - Triton and ATen/Inductor of torch 2.6 -
 and holds no recorded outputs): torch.topk's order among exactly tied scores,
-Inductor's summation order inside the pooled mean (last-ulp bf16 flips), and the
-bit-level output of the Triton attention kernel.  For those the build rule is
+Inductor's summation order inside the pooled mean (last-ulp bf16 flips), the
+bit-level output of the Triton attention kernel, and for the CDF rule the order
+of torch.sort among equal weights, the fp32 rounding of torch.cumsum next to
+the threshold and the storage type of the weights (the reference's bf16 route
+does not run).  For those the build rule is
 stated in the function's docstring.
 """
 from __future__ import annotations
@@ -153,6 +166,28 @@ def select_topk(score: torch.Tensor, k_sel: int) -> Tuple[torch.Tensor, torch.Te
     idx = torch.from_numpy(np.ascontiguousarray(order[..., :k_sel]).astype(np.int64))
     lens = torch.full(score.shape[:3], k_sel, dtype=torch.int32)
     return idx, lens
+
+
+def select_cdf(score: torch.Tensor, cdf_threshold: float, sm_scale: float, k_min: int = 0, cap: int = None):
+    """bsa:233-243 (and bsa:252-266 with k_min = the top-k count): weights = softmax(score * sm_scale),
+    columns sorted by descending weight, cdf = cumsum, lens = searchsorted(cdf, threshold, right=True) = the
+    number of cdf entries <= threshold, raised to k_min.  Returns (indices int64 [B,H,nbq,nbk] in the full
+    sorted order, lens int32, cdf float64 in sorted order).
+    Build rules where the reference leaves freedom or cannot run: the sort key is (-score, index) (torch.sort
+    leaves ties unspecified; the softmax is monotone in the score); the weights are fp32 for every score
+    dtype (the reference's bf16 route stops at a dtype check inside torch.searchsorted, bsa:236-241); the
+    running sum is kept in float64, so a row can differ from an fp32 running sum only where that sum comes
+    within rounding of the threshold.  `cap` limits lens (the engine keeps at most 1024 blocks per row)."""
+    s = score.float()
+    w = torch.softmax(s * sm_scale, dim=-1)
+    order = np.argsort(-s.numpy(), axis=-1, kind="stable")
+    idx = torch.from_numpy(np.ascontiguousarray(order).astype(np.int64))
+    cdf = torch.cumsum(torch.gather(w, -1, idx).double(), dim=-1)
+    lens = (cdf <= float(np.float32(cdf_threshold))).sum(-1)
+    lens = torch.clamp(lens, min=int(k_min))
+    if cap is not None:
+        lens = torch.clamp(lens, max=int(cap))
+    return idx, lens.to(torch.int32), cdf
 
 
 def block_mask_from_indices(idx: torch.Tensor, lens: torch.Tensor, n_cols: int) -> torch.Tensor:

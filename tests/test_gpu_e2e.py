@@ -190,3 +190,34 @@ def test_720p_full_shape_sampled():
                          q_blocks=[0, 19, 700, 1439], heads=heads)
     o2 = I().flash_attn_bsa_3d(q, k, v, latent, latent, sparsity=0.9375, **CH)
     assert torch.equal(o, o2)
+
+
+@pytest.mark.parametrize("sparsity", [None, 0.75])
+def test_operator_with_cdf_selection(sparsity):
+    """flash_attn_bsa_3d with cdf_threshold (bsa_interface.py:268-277, 555): rows keep different numbers of
+    blocks; the output is judged against the oracle evaluated with the GPU's own selection."""
+    latent = (5, 8, 12)
+    S = int(np.prod(latent))
+    q, k, v = seeded_qkv(51, 1, 2, S, S, 128, torch.bfloat16)
+    q = q * 3                                               # sharper pooled scores: a wider spread of list lengths
+    o, idx, lens, score = I()._bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, sparsity, (4, 4, 4), (4, 4, 4), True,
+                                      cdf_threshold=0.6)
+    nb = int(np.prod(O.block_grid(latent, (4, 4, 4))))
+    assert idx.shape == (1, 2, nb, nb)
+    k_min = 0 if sparsity is None else O.num_selected(sparsity, nb)
+    want_idx, want_lens, cdf = O.select_cdf(score.cpu(), 0.6, 1 / math.sqrt(128), k_min=k_min)
+    near = (cdf - float(np.float32(0.6))).abs().min(-1).values < 1e-5
+    assert torch.equal(lens.cpu().long()[~near], want_lens.long()[~near])
+    assert int(lens.min()) >= k_min and int(lens.min()) < int(lens.max())
+    qp = O.rearrange_thw_to_3d_block(q, latent, (4, 4, 4))
+    kp = O.rearrange_thw_to_3d_block(k, latent, (4, 4, 4))
+    vp = O.rearrange_thw_to_3d_block(v, latent, (4, 4, 4))
+    kvalid = torch.from_numpy(O.slot_validity(latent, (4, 4, 4)))
+    want_o, _ = O.gathered_attention(qp, kp, vp, idx.cpu().long().clamp(min=0), lens.cpu(), 64, 64, 1 / math.sqrt(128),
+                                     key_valid=kvalid, q_blocks=range(nb))
+    got_p = O.rearrange_thw_to_3d_block(o.cpu(), latent, (4, 4, 4))
+    qvalid = torch.from_numpy(O.slot_validity(latent, (4, 4, 4)))
+    d = (got_p[:, :, qvalid].float() - want_o[:, :, qvalid]).abs()
+    assert d.max() <= MAX_ABS and d.mean() <= MEAN_ABS
+    pub = I().flash_attn_bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, sparsity=sparsity, cdf_threshold=0.6, **CH)
+    assert torch.equal(pub, o)

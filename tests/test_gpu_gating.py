@@ -125,3 +125,70 @@ def test_full_size_720p_selection():
         assert torch.equal(idx[:, h:h + 1].cpu().long(), want)
     idx2, _, _ = I()._score_topk(qc, kc, 90)
     assert torch.equal(idx, idx2)
+
+
+# ---------------------------------------------------------------------------
+# selection by cumulative attention mass (bsa_interface.py:226-266)
+# ---------------------------------------------------------------------------
+def check_cdf_selection(score, idx, lens, thr, scale, k_min=0):
+    """idx/lens from the GPU against the oracle on the same scores: the count may only differ where the
+    running sum comes within rounding of the threshold; given the count, the list is the oracle's order."""
+    nbk = score.shape[-1]
+    cap = min(nbk, 1024)
+    want_idx, want_lens, cdf = O.select_cdf(score, thr, scale, k_min=k_min, cap=cap)
+    lens = lens.cpu().long()
+    near = (cdf - float(np.float32(thr))).abs().min(-1).values < 1e-5
+    assert torch.equal(lens[~near], want_lens.long()[~near])
+    assert (lens - want_lens.long()).abs().max() <= 1
+    assert near.float().mean() < 0.05
+    idx = idx.cpu().long()
+    assert idx.shape[-1] == cap
+    pos = torch.arange(cap).expand_as(idx)
+    used = pos < lens.unsqueeze(-1)
+    assert torch.equal(idx[used], want_idx[..., :cap][used])
+    assert torch.all(idx[~used] == -1)
+    return lens
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_cdf_selection_from_score(dtype):
+    g = torch.Generator().manual_seed(21)
+    score = (torch.randn(1, 2, 33, 200, generator=g) * 4).to(dtype)
+    for thr, scale in [(0.5, 1.0), (0.9, 0.25), (0.999, 0.0883883)]:
+        idx, lens = I().get_select_indices_cdf_from_score(score.cuda(), thr, scale)
+        assert idx.dtype == torch.int64 and lens.dtype == torch.int32
+        got = check_cdf_selection(score, idx, lens, thr, scale)
+        assert got.min() < got.max()                       # rows keep different numbers of blocks
+    # with a top-k floor (bsa_interface.py:252-266)
+    idx, lens = I().get_select_indices_cdf_topk_from_score(score.cuda(), 0.9, 0.5, 1.0)
+    check_cdf_selection(score, idx, lens, 0.5, 1.0, k_min=O.num_selected(0.9, 200))
+    assert int(lens.min()) >= O.num_selected(0.9, 200) == 19      # int((1 - 0.9) * 200) truncates 19.999...
+
+
+def test_cdf_selection_edge_cases():
+    score = torch.zeros(1, 1, 4, 130)
+    score[0, 0, 1, 7] = 60.0                                # one column holds all the mass
+    score[0, 0, 2, :] = torch.arange(130).float() * 0.01
+    idx, lens = I().get_select_indices_cdf_from_score(score.cuda(), 0.5, 1.0)
+    assert lens.cpu().tolist() == [[[65, 0, int(O.select_cdf(score, 0.5, 1.0)[1][0, 0, 2]), 65]]]
+    assert torch.equal(idx[0, 0, 0, :65].cpu(), torch.arange(65))          # ties: lowest index first
+    assert int(idx[0, 0, 1, 0]) == -1
+    idx, lens = I().get_select_indices_cdf_from_score(score.cuda(), 2.0, 1.0)   # threshold above one: everything
+    assert torch.all(lens == 130)
+    big = torch.randn(1, 1, 3, 1440, generator=torch.Generator().manual_seed(22)).bfloat16()
+    idx, lens = I().get_select_indices_cdf_from_score(big.cuda(), 0.95, 1.0)
+    check_cdf_selection(big, idx, lens, 0.95, 1.0)
+    assert idx.shape[-1] == 1024 and int(lens.max()) <= 1024               # at most 1024 blocks per row
+
+
+def test_cdf_selection_from_pooled_vectors_and_dispatch():
+    g = torch.Generator().manual_seed(23)
+    q = torch.randn(1, 2, 24, 128, generator=g).bfloat16()
+    k = torch.randn(1, 2, 96, 128, generator=g).bfloat16()
+    score = I().cal_score(q.cuda(), k.cuda()).cpu()
+    idx, lens = I().get_select_indices(q.cuda(), k.cuda(), None, 0.7)
+    check_cdf_selection(score, idx, lens, 0.7, 1 / 128 ** 0.5)
+    idx2, lens2 = I().get_select_indices(q.cuda(), k.cuda(), 0.75, 0.7)
+    check_cdf_selection(score, idx2, lens2, 0.7, 1 / 128 ** 0.5, k_min=24)
+    idx3, lens3 = I().get_select_indices_from_score(score.cuda(), None, 0.7)
+    assert torch.equal(idx3, idx) and torch.equal(lens3, lens)

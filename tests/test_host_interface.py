@@ -49,10 +49,12 @@ def test_selection_mode_errors():
     q, k, v = qkv()
     with pytest.raises(ValueError):
         I.flash_attn_bsa_3d(q, k, v, (4, 8, 8), (4, 8, 8), sparsity=None, cdf_threshold=None)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError, match="GPU only"):          # the CDF rule is built: CPU tensors get as far as the engine
         I.flash_attn_bsa_3d(q, k, v, (4, 8, 8), (4, 8, 8), sparsity=None, cdf_threshold=0.9)
     with pytest.raises(ValueError):
         I.get_select_indices(q, k, None, None)
+    with pytest.raises(ValueError):
+        I.get_select_indices_from_score(q, None, None)
 
 
 def test_no_cpu_fallback_and_forward_only():

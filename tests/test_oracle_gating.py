@@ -100,3 +100,57 @@ def test_block_mask_brute_force():
             for j in range(int(lens[0, h, m])):
                 want[idx[0, h, m, j]] = True
             assert torch.equal(mask[0, h, m], want)
+
+
+# ---------------------------------------------------------------------------
+# selection by cumulative attention mass (bsa_interface.py:233-266)
+# ---------------------------------------------------------------------------
+def test_cdf_rule_closed_forms():
+    # equal scores: equal weights 1/n, cdf_j = j/n, ties in index order
+    score = torch.zeros(1, 1, 2, 8)
+    idx, lens, cdf = O.select_cdf(score, 0.5, 0.3)
+    assert torch.equal(idx[0, 0, 0], torch.arange(8)) and lens.tolist() == [[[4, 4]]]
+    assert torch.allclose(cdf[0, 0, 0], torch.arange(1, 9).double() / 8)
+    # one dominant column outweighs the threshold alone: nothing is kept, unless a minimum is asked for
+    score = torch.tensor([[[[0.0, 50.0, 1.0, 2.0]]]])
+    idx, lens, _ = O.select_cdf(score, 0.9, 1.0)
+    assert idx[0, 0, 0].tolist() == [1, 3, 2, 0] and int(lens) == 0
+    assert int(O.select_cdf(score, 0.9, 1.0, k_min=2)[1]) == 2
+    # a threshold above one keeps every column; cap limits it
+    assert int(O.select_cdf(score, 1.5, 1.0)[1]) == 4 and int(O.select_cdf(score, 1.5, 1.0, cap=3)[1]) == 3
+    # two columns of weight 1/4 each and one of 1/2: log-weights as scores with scale 1
+    score = torch.log(torch.tensor([[[[0.25, 0.5, 0.25]]]]))
+    assert int(O.select_cdf(score, 0.5, 1.0)[1]) == 1 and int(O.select_cdf(score, 0.76, 1.0)[1]) == 2
+    assert O.select_cdf(score, 0.76, 1.0)[0][0, 0, 0].tolist() == [1, 0, 2]
+
+
+def test_cdf_rule_against_a_python_loop_and_the_library_pipeline():
+    g = torch.Generator().manual_seed(7)
+    score = torch.randn(2, 3, 5, 37, generator=g) * 3
+    thr, scale = 0.8, 0.7
+    idx, lens, cdf = O.select_cdf(score, thr, scale)
+    for b, h, m in [(0, 0, 0), (1, 2, 4), (0, 1, 3)]:
+        row = score[b, h, m].tolist()
+        order = sorted(range(37), key=lambda j: (-row[j], j))
+        mx = max(row)
+        e = [float(np.float32(np.exp(np.float32((row[j] - mx) * scale)))) for j in order]
+        z = sum(e)
+        run, n = 0.0, 0
+        for x in e:
+            run += x / z
+            if run <= thr:
+                n += 1
+        assert idx[b, h, m].tolist() == order
+        assert abs(int(lens[b, h, m]) - n) <= (1 if min(abs(c - thr) for c in cdf[b, h, m].tolist()) < 1e-5 else 0)
+    # the reference's own sequence of library calls (bsa:234-241) on tie-free fp32 scores
+    weights = torch.softmax(score * scale, dim=-1)
+    ws = torch.sort(weights, dim=-1, descending=True)
+    ref_cdf = torch.cumsum(ws.values, dim=-1)
+    ref_n = torch.searchsorted(ref_cdf, torch.full(score.shape[:3] + (1,), thr), right=True).squeeze(-1)
+    clear = (cdf - thr).abs().min(-1).values > 1e-5
+    assert clear.float().mean() > 0.9
+    assert torch.equal(ref_n[clear], lens.long()[clear])
+    assert torch.equal(ws.indices, idx)
+    # cdf + top-k: never fewer than the top-k count
+    lens2 = O.select_cdf(score, thr, scale, k_min=9)[1]
+    assert torch.equal(lens2, torch.clamp(lens, min=9))
