@@ -268,7 +268,7 @@ int bsa_norm_rope(const void* src, const int64_t src_strides[3], void* dst, cons
 
 /* out[M,N] = x[M,K] . w[N,K]^T (+ bias[N]) (+ residual[M,N]), bf16 in/out, fp32 accumulate, on MFMA
  * through hipBLASLt.  Replaces the nn.Linear calls attention.py:111 and :142.  `workspace`: at least
- * 32 MiB of device memory (BSA_ERR_WORKSPACE otherwise); its contents do not matter.  Creates one
+ * 64 MiB of device memory (BSA_ERR_WORKSPACE otherwise); its contents do not matter.  Creates one
  * process-wide hipBLASLt handle on first use. */
 int bsa_linear_bf16(const void* x, const void* w, const void* bias, const void* residual, void* out,
                     int64_t M, int N, int K, void* workspace, size_t workspace_bytes, void* stream);

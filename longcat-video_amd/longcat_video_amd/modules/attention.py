@@ -60,6 +60,18 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return out
 
 
+_GEMM_WORKSPACES = {}
+
+
+def _gemm_workspace(device) -> torch.Tensor:
+    """64 MiB per device and stream, kept: calls on one stream run one after the other."""
+    key = (str(device), torch.cuda.current_stream(device).cuda_stream)
+    ws = _GEMM_WORKSPACES.get(key)
+    if ws is None:
+        ws = _GEMM_WORKSPACES[key] = torch.empty(64 << 20, dtype=torch.uint8, device=device)
+    return ws
+
+
 def linear_bf16(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
                 residual: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -82,7 +94,7 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
         r = residual.reshape(-1, N).contiguous()
         assert r.shape == out.shape and r.dtype == torch.bfloat16
     if workspace is None:
-        workspace = torch.empty(32 << 20, dtype=torch.uint8, device=x.device)
+        workspace = _gemm_workspace(x.device)
     with torch.cuda.device(x.device):
         _capi.check(_capi.load().bsa_linear_bf16(_ptr(x2), _ptr(w), _ptr(b), _ptr(r), _ptr(out), x2.shape[0], N, K,
                                                  _ptr(workspace), workspace.numel(), _stream(x)), "linear")
