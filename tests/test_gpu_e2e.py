@@ -221,3 +221,19 @@ def test_operator_with_cdf_selection(sparsity):
     assert d.max() <= MAX_ABS and d.mean() <= MEAN_ABS
     pub = I().flash_attn_bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, sparsity=sparsity, cdf_threshold=0.6, **CH)
     assert torch.equal(pub, o)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_two_batches_on_a_ragged_grid(dtype):
+    """Batch and head strides of the direct (T,H,W)-order path: B = 2, three heads, every axis ragged."""
+    latent = (5, 9, 13)
+    S = int(np.prod(latent))
+    q, k, v = seeded_qkv(52, 2, 3, S, S, 128, dtype)
+    o, idx, lens, score = I()._bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, 0.75, (4, 4, 4), (4, 4, 4), True)
+    nb = int(np.prod(O.block_grid(latent, (4, 4, 4))))
+    for b in range(2):
+        check_against_oracle(q[b:b + 1], k[b:b + 1], v[b:b + 1], latent, latent, 0.75, o[b:b + 1], idx[b:b + 1],
+                             lens[b:b + 1], score[b:b + 1], q_blocks=[0, nb // 3, nb - 1])
+    # each batch entry on its own gives the same bits
+    o0 = I()._bsa_3d(q[1:].cuda(), k[1:].cuda(), v[1:].cuda(), latent, latent, 0.75, (4, 4, 4), (4, 4, 4))
+    assert torch.equal(o0, o[1:])
