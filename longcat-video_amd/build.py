@@ -68,7 +68,7 @@ def build(keep_temps: bool = False, verbose: bool = True) -> str:
             print(out)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(4, len(sources))) as ex:
+    with ThreadPoolExecutor(max_workers=min(6, len(sources))) as ex:
         objs = list(ex.map(compile_one, sources))
     _run([cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs, "-lhipblaslt"])
     if verbose:

@@ -47,52 +47,13 @@
 // L2 hits (the 4 MB L2 of an XCD cannot hold the 47 MB of K/V of one 720p head,
 // and L2 misses are served at only ~8 TB/s for 16 KB tiles).  One launch of the
 // whole grid loses this: workgroups then start whenever a slot frees up.
-#include "bsa_common.h"
-
-#include <type_traits>
+#include "bsa_mfma.h"
 
 namespace bsa {
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
+using namespace mfma;
 
-__device__ inline f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
-__device__ inline f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-}
-template <typename T> struct Vec8;
-template <> struct Vec8<__bf16> { typedef bf16x8 type; };
-template <> struct Vec8<_Float16> { typedef f16x8 type; };
-
-constexpr int kD = 128;          // head dim
-constexpr int kTile = 64;        // query rows per work item, keys per tile
-constexpr int kTileBytes = kTile * kD * 2;
-constexpr float kLog2e = 1.44269504f;
-constexpr float kLn2 = 0.6931471824645996f;
-constexpr float kLazyTau = 8.0f; // log2 headroom before the running max is raised
-constexpr int kListCap = 1024;   // tiles whose addresses are staged in LDS at a time
-
-// 16 bytes per lane from global memory straight into LDS.  The LDS address is
-// m0 + 16*lane; the global address is sbase + voff.  Issued from inline assembly
-// so that the compiler does not order later LDS reads of other stages behind it;
-// completion is awaited explicitly (s_waitcnt vmcnt) before the stage is read.
-__device__ inline void load_to_lds_16(const void* sbase, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
-}
-__device__ inline uint32_t lds_address(const void* p) {
-    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
-}
-// 4 keys x 16 d patch -> this lane's d, 4 keys (see the header comment)
-__device__ inline s16x4 lds_read_tr16(const void* p) {
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
-}
 template <typename T>
 __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
