@@ -150,7 +150,10 @@ int bsa_topk_from_score(const void* score, int32_t* idx_out, int32_t* idx_sorted
  *   o = softmax(q k^T * sm_scale) v restricted to the listed blocks; logits are
  *   fp32, the scale is applied after the dot as sm_scale*log2(e), probabilities
  *   are rounded to `dtype` for the P V product while the row sum stays fp32.
- *   An empty list gives o = 0, lse = -inf.
+ *   An empty list gives o = 0, lse = -inf.  The kernels clamp every block index
+ *   to [0, Sk/bs_k) and every length to [0, idx_stride]: a malformed list gives
+ *   wrong numbers for its query block, never an access outside k and v (the
+ *   reference's kernel reads wherever such an index points).
  * Limits: D == 128; bs_q, bs_k multiples of 64; Sq % bs_q == 0, Sk % bs_k == 0.
  */
 int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, const int32_t* lens,
@@ -272,6 +275,24 @@ int bsa_norm_rope(const void* src, const int64_t src_strides[3], void* dst, cons
  * process-wide hipBLASLt handle on first use. */
 int bsa_linear_bf16(const void* x, const void* w, const void* bias, const void* residual, void* out,
                     int64_t M, int N, int K, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The same product with row strides (in elements): x rows ldx apart, w rows ldw apart, out (and residual)
+ * rows ldo apart.  Lets one output block of a LoRA up-projection that is split over the output features
+ * (lora_utils.py:12-21: chunk the rank axis, one Linear per chunk, concatenate) read its slice of the
+ * rank axis and write its slice of the output columns in place. */
+int bsa_linear_bf16_ld(const void* x, int64_t ldx, const void* w, int64_t ldw, const void* bias, const void* residual,
+                       void* out, int64_t ldo, int64_t M, int N, int K, void* workspace, size_t workspace_bytes,
+                       void* stream);
+
+/* LoRA side branches of a Linear (longcat_video_dit.py:234-249): out = org + total, where total sums
+ * up_i * multiplier_i * alpha_scale_i over the active branches, up_i = lora_up(lora_down(x)) already
+ * computed (bsa_linear_bf16 / _ld).  Every product and every sum is rounded to `dtype` as the eager
+ * expression does: s_i = T(T(up_i * multiplier_i) * alpha_scale_i); total = s_0, then T(total + s_i);
+ * out = T(org + total).  up, multiplier, alpha_scale are HOST arrays of n_loras entries (1..4); the
+ * up[i] are device pointers to n elements each; out may alias org.  The caller passes alpha_scale as the
+ * reference holds it (a buffer cast to the model dtype, longcat_video_dit.py:221). */
+int bsa_lora_add(const void* org, const void* const* up, const float* multiplier, const float* alpha_scale, int n_loras,
+                 void* out, int64_t n, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

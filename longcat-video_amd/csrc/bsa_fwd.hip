@@ -122,7 +122,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     const int64_t q_bh = (int64_t)(bh / Hn) * L.q_st[0] + (int64_t)(bh % Hn) * L.q_st[1];
     const int64_t o_bh = (int64_t)(bh / Hn) * L.o_st[0] + (int64_t)(bh % Hn) * L.o_st[1];
     const int32_t* list = idx + ((int64_t)bh * nbq + qblock) * idx_stride;
-    const int ntiles = lens[(int64_t)bh * nbq + qblock] * nsub;
+    const int ntiles = min(max(lens[(int64_t)bh * nbq + qblock], 0), idx_stride) * nsub;   // never past the list row
     const char* kbase = reinterpret_cast<const char*>(k + (int64_t)(bh / Hn) * L.k_st[0] + (int64_t)(bh % Hn) * L.k_st[1]);
     const char* vbase = reinterpret_cast<const char*>(v + (int64_t)(bh / Hn) * L.v_st[0] + (int64_t)(bh % Hn) * L.v_st[1]);
 
@@ -174,7 +174,9 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     __syncthreads();                          // previous chunk / previous item fully consumed
     for (int j = tid; j < nloc; j += 256) {
         const int it = chunk0 + j;
-        const int tile = list[it / nsub] * nsub + it % nsub;
+        // a block index outside [0, Sk / bs_k) is clamped: a malformed list gives wrong numbers, never a fault
+        const int blk = min(max(list[it / nsub], 0), (int)(Sk / bs_k) - 1);
+        const int tile = blk * nsub + it % nsub;
         const uint32_t entry = L.k_tiles != nullptr ? L.k_tiles[tile] : (uint32_t)tile * kTile;
         tile_row_sm[j] = (int)entry;
         tile_mask_sm[j] = tile_valid ? tile_valid[tile] : ~0ull;
@@ -430,7 +432,7 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(
     const int qblock = (int)(qrow0 / bs_q);
     const int nsub = bs_k / kTile;
     const int32_t* list = idx + ((int64_t)bh * nbq + qblock) * idx_stride;
-    const int ntiles = lens[(int64_t)bh * nbq + qblock] * nsub;
+    const int ntiles = min(max(lens[(int64_t)bh * nbq + qblock], 0), idx_stride) * nsub;   // never past the list row
     const float* kbase = k + (int64_t)bh * Sk * kD;
     const float* vbase = v + (int64_t)bh * Sk * kD;
 
@@ -443,7 +445,7 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(
     }
     float m_i = -INFINITY, l_i = 0.f;
     for (int it = 0; it < ntiles; ++it) {
-        const int64_t row0 = (int64_t)list[it / nsub] * bs_k + (int64_t)(it % nsub) * kTile;
+        const int64_t row0 = (int64_t)min(max(list[it / nsub], 0), (int)(Sk / bs_k) - 1) * bs_k + (int64_t)(it % nsub) * kTile;
         const uint64_t vmask = tile_valid ? tile_valid[row0 / kTile] : ~0ull;
         __syncthreads();
         for (int i = tid; i < kTile * kD / 4; i += 256) {

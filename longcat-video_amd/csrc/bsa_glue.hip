@@ -125,6 +125,40 @@ __global__ __launch_bounds__(256) void gated_residual_kernel(const T* __restrict
     *reinterpret_cast<uint4*>(out + row * dim + d) = *reinterpret_cast<const uint4*>(res);
 }
 
+// ------------------------------------------------- LoRA side branches
+// out = T(org + total) with total = s_0, then T(total + s_i), and s_i = T(T(up_i * multiplier_i) * alpha_i):
+// every product and sum of the eager expression is rounded to the tensor dtype, one by one.
+constexpr int kMaxLoras = 4;
+struct LoraTerms {
+    const void* up[kMaxLoras];
+    float multiplier[kMaxLoras];
+    float alpha[kMaxLoras];
+    int n;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void lora_add_kernel(const T* __restrict__ org, LoraTerms terms, T* __restrict__ out,
+                                                       int64_t n8) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n8) return;
+    const uint4 raw = reinterpret_cast<const uint4*>(org)[i];
+    const T* oe = reinterpret_cast<const T*>(&raw);
+    T total[8];
+    for (int j = 0; j < terms.n; ++j) {
+        const uint4 ur = reinterpret_cast<const uint4*>(terms.up[j])[i];
+        const T* ue = reinterpret_cast<const T*>(&ur);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const T scaled = (T)__fmul_rn((float)(T)__fmul_rn((float)ue[k], terms.multiplier[j]), terms.alpha[j]);
+            total[k] = j == 0 ? scaled : (T)__fadd_rn((float)total[k], (float)scaled);
+        }
+    }
+    T res[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) res[k] = (T)__fadd_rn((float)oe[k], (float)total[k]);
+    reinterpret_cast<uint4*>(out)[i] = *reinterpret_cast<const uint4*>(res);
+}
+
 // ------------------------------------------------- per-head RMSNorm + RoPE
 // One row = one (token, head) vector of D = 128 elements, handled by 16 lanes
 // (8 elements each, i.e. 4 interleaved rotation pairs per lane).
@@ -275,6 +309,35 @@ int bsa_gated_residual(const void* x, const void* y, const float* gate, void* ou
     return e == hipSuccess ? BSA_OK : set_error(BSA_ERR_HIP, "gated_residual launch: %s", hipGetErrorString(e));
 }
 
+int bsa_lora_add(const void* org, const void* const* up, const float* multiplier, const float* alpha_scale, int n_loras,
+                 void* out, int64_t n, int dtype, void* stream) {
+    if (!org || !up || !multiplier || !alpha_scale || !out) return set_error(BSA_ERR_BAD_ARG, "lora_add: null pointer");
+    if (n_loras < 1 || n_loras > kMaxLoras) return set_error(BSA_ERR_UNSUPPORTED, "lora_add: %d side branches (1..%d are built)", n_loras, kMaxLoras);
+    if (n <= 0 || n % 8) return set_error(BSA_ERR_BAD_ARG, "lora_add: the element count must be a positive multiple of 8");
+    LoraTerms terms{};
+    terms.n = n_loras;
+    uintptr_t bits = reinterpret_cast<uintptr_t>(org) | reinterpret_cast<uintptr_t>(out);
+    for (int j = 0; j < n_loras; ++j) {
+        if (!up[j]) return set_error(BSA_ERR_BAD_ARG, "lora_add: null pointer");
+        terms.up[j] = up[j];
+        terms.multiplier[j] = multiplier[j];
+        terms.alpha[j] = alpha_scale[j];
+        bits |= reinterpret_cast<uintptr_t>(up[j]);
+    }
+    if (bits & 15u) return set_error(BSA_ERR_BAD_ARG, "lora_add: pointers must be 16-byte aligned");
+    const int64_t n8 = n / 8;
+    if ((n8 + 255) / 256 > 0x7fffffffLL) return set_error(BSA_ERR_UNSUPPORTED, "lora_add: too many elements");
+    const dim3 grid((unsigned)((n8 + 255) / 256)), block(256);
+    if (dtype == BSA_BF16)
+        hipLaunchKernelGGL((lora_add_kernel<__bf16>), grid, block, 0, (hipStream_t)stream, (const __bf16*)org, terms, (__bf16*)out, n8);
+    else if (dtype == BSA_F16)
+        hipLaunchKernelGGL((lora_add_kernel<_Float16>), grid, block, 0, (hipStream_t)stream, (const _Float16*)org, terms, (_Float16*)out, n8);
+    else
+        return set_error(BSA_ERR_UNSUPPORTED, "lora_add: dtype %d is not built (bf16, fp16)", dtype);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? BSA_OK : set_error(BSA_ERR_HIP, "lora_add launch: %s", hipGetErrorString(e));
+}
+
 int bsa_norm_rope(const void* src, const int64_t src_strides[3], void* dst, const int64_t dst_strides[3],
                   const void* weight, const float* rope_table, int B, int Hn, int T, int H, int W, int t_offset,
                   int table_T, int D, float eps, int dtype, void* stream) {
@@ -319,8 +382,15 @@ int bsa_qk_norm_rope(void* q, const int64_t q_strides[3], void* k, const int64_t
 
 int bsa_linear_bf16(const void* x, const void* w, const void* bias, const void* residual, void* out, int64_t M, int N,
                     int K, void* workspace, size_t workspace_bytes, void* stream) {
+    return bsa_linear_bf16_ld(x, K, w, K, bias, residual, out, N, M, N, K, workspace, workspace_bytes, stream);
+}
+
+int bsa_linear_bf16_ld(const void* x, int64_t ldx, const void* w, int64_t ldw, const void* bias, const void* residual,
+                       void* out, int64_t ldo, int64_t M, int N, int K, void* workspace, size_t workspace_bytes,
+                       void* stream) {
     if (!x || !w || !out) return set_error(BSA_ERR_BAD_ARG, "linear: null pointer");
     if (M <= 0 || N <= 0 || K <= 0) return set_error(BSA_ERR_BAD_ARG, "linear: sizes must be positive");
+    if (ldx < K || ldw < K || ldo < N) return set_error(BSA_ERR_BAD_ARG, "linear: a row stride is shorter than its row");
     // hipBLASLt has been seen to write through the workspace pointer for large problems even when it was
     // told that there is none, so a workspace is mandatory.  Its best algorithms for the 720p projections
     // want just under 64 MiB (1.52 PFLOP/s instead of 1.24 with 32 MiB); more brings nothing.
@@ -353,9 +423,9 @@ int bsa_linear_bf16(const void* x, const void* w, const void* bias, const void* 
             BSA_LT(hipblasLtMatmulDescSetAttribute(desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)));
             BSA_LT(hipblasLtMatmulDescSetAttribute(desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bt, sizeof(bt)));
         }
-        BSA_LT(hipblasLtMatrixLayoutCreate(&la, HIP_R_16BF, K, N, K));
-        BSA_LT(hipblasLtMatrixLayoutCreate(&lb, HIP_R_16BF, K, M, K));
-        BSA_LT(hipblasLtMatrixLayoutCreate(&lc, HIP_R_16BF, N, M, N));
+        BSA_LT(hipblasLtMatrixLayoutCreate(&la, HIP_R_16BF, K, N, ldw));
+        BSA_LT(hipblasLtMatrixLayoutCreate(&lb, HIP_R_16BF, K, M, ldx));
+        BSA_LT(hipblasLtMatrixLayoutCreate(&lc, HIP_R_16BF, N, M, ldo));
         BSA_LT(hipblasLtMatmulPreferenceCreate(&pref));
         const uint64_t wsb = workspace_bytes;
         BSA_LT(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &wsb, sizeof(wsb)));

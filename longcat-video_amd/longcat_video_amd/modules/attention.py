@@ -194,6 +194,17 @@ class Attention(nn.Module):
         self.q_norm = RMSNorm_FP32(self.head_dim, eps=1e-6)
         self.k_norm = RMSNorm_FP32(self.head_dim, eps=1e-6)
         self.proj = nn.Linear(dim, dim)
+        # LoRA side branches (lists of modules.lora.LoRABranch), as enable_loras attaches them to
+        # `attn.qkv` and `attn.proj` (longcat_video_dit.py:211-232); empty = the plain Linear
+        self.qkv_loras = []
+        self.proj_loras = []
+
+    def _linear(self, x, layer, loras, residual=None):
+        if any(b.use_lora for b in loras):
+            from .lora import lora_linear
+            y = lora_linear(x, layer.weight, layer.bias, loras)
+            return y if residual is None else y + residual
+        return linear_bf16(x, layer.weight, layer.bias, residual=residual)
 
     def _process_attn(self, q, k, v, shape, out=None):
         """attention.py:50-105, block-sparse branch; writes into `out` ([B,H,SQ,D] view) if given."""
@@ -215,7 +226,7 @@ class Attention(nn.Module):
 
     def _project_qkv(self, x):
         B, N, C = x.shape
-        qkv = linear_bf16(x, self.qkv.weight, self.qkv.bias)                      # [B, N, 3C]
+        qkv = self._linear(x, self.qkv, self.qkv_loras)                           # [B, N, 3C]
         return qkv.view(B, N, 3, self.num_heads, self.head_dim).permute(2, 0, 3, 1, 4).unbind(0)   # strided [B,H,N,D] views
 
     @torch.no_grad()
@@ -243,7 +254,7 @@ class Attention(nn.Module):
             self._process_attn(q[:, :, n:], k, v, shape, out=ov[:, :, n:])                       # attention.py:132-133
         else:
             self._process_attn(q, k, v, shape, out=ov)
-        y = linear_bf16(o.view(B, N, C), self.proj.weight, self.proj.bias, residual=residual)
+        y = self._linear(o.view(B, N, C), self.proj, self.proj_loras, residual=residual)
         if return_kv:
             return y, (k_cache, v.clone())
         return y
@@ -280,7 +291,7 @@ class Attention(nn.Module):
                       t_offset=num_cond_latents, table_grid=grid_full)
         o = torch.empty(B, N, Hn, D, dtype=x.dtype, device=x.device)
         self._process_attn(q, k_full, v_full, shape, out=o.permute(0, 2, 1, 3))
-        return linear_bf16(o.view(B, N, C), self.proj.weight, self.proj.bias, residual=residual)
+        return self._linear(o.view(B, N, C), self.proj, self.proj_loras, residual=residual)
 
 
 @torch.no_grad()

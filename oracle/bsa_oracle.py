@@ -43,6 +43,11 @@ fixtures for this path, so the pins are mathematical; see tests/test_oracle_*):
                                     forward over all frames
   layernorm_modulate_fp32 / gated_residual_fp32
                                     torch F.layer_norm, closed forms
+  lora_linear                       zero up-weights (the initial state) give the
+                                    plain Linear bit for bit; integer-valued
+                                    inputs give the merged weight
+                                    W + m*a*U.D exactly; split up-projection ==
+                                    one block-diagonal matrix; torch F.linear
 
 What no CPU check can pin ("parity unpinned", because the reference executes
 them inside un-vendored third parties - Triton and ATen/Inductor of torch 2.6 -
@@ -429,14 +434,16 @@ def rope_3d_apply(x: torch.Tensor, angles: torch.Tensor) -> torch.Tensor:
 
 
 def attention_module_forward(x, w_qkv, b_qkv, w_proj, b_proj, q_norm_w, k_norm_w, shape,
-                             num_heads: int, bsa_params: dict, num_cond_latents: int = 0):
+                             num_heads: int, bsa_params: dict, num_cond_latents: int = 0,
+                             qkv_loras=(), proj_loras=()):
     """attn:107-147 (Attention.forward) with the BSA branch of attn:58-67.
     x [B,N,C]; weights in nn.Linear layout [out,in].  Linear layers accumulate in
-    fp32 and round once to x.dtype, as a bf16 GEMM does."""
+    fp32 and round once to x.dtype, as a bf16 GEMM does.  qkv_loras / proj_loras: side
+    branches on the two Linears in the form lora_linear takes."""
     B, N, C = x.shape
     D = C // num_heads
     dt = x.dtype
-    qkv = (x.float() @ w_qkv.float().t() + b_qkv.float()).to(dt)
+    qkv = lora_linear(x.reshape(B * N, C), w_qkv, b_qkv, qkv_loras).view(B, N, 3 * C)
     qkv = qkv.view(B, N, 3, num_heads, D).permute(2, 0, 3, 1, 4)
     q, k, v = qkv.unbind(0)
     q, k = rms_norm_fp32(q, q_norm_w), rms_norm_fp32(k, k_norm_w)
@@ -447,7 +454,7 @@ def attention_module_forward(x, w_qkv, b_qkv, w_proj, b_proj, q_norm_w, k_norm_w
     else:
         o, *_ = flash_attn_bsa_3d(q, k, v, shape, shape, **bsa_params)
     o = o.to(dt).transpose(1, 2).reshape(B, N, C)
-    return (o.float() @ w_proj.float().t() + b_proj.float()).to(dt)
+    return lora_linear(o.reshape(B * N, C), w_proj, b_proj, proj_loras).view(B, N, C)
 
 
 def attention_module_kv(x, w_qkv, b_qkv, q_norm_w, k_norm_w, num_heads: int):
@@ -504,3 +511,25 @@ def gated_residual_fp32(x: torch.Tensor, gate: torch.Tensor, y: torch.Tensor) ->
     T = gate.shape[1]
     out = x.float().view(B, T, N // T, C) + gate.float() * y.float().view(B, T, N // T, C)
     return out.view(B, N, C).to(x.dtype)
+
+
+def lora_linear(x, weight, bias, loras):
+    """The patched Linear forward of longcat_video_dit.py:234-249: org_output + sum over the active branches of
+    lora_up(lora_down(x)) * multiplier * alpha_scale, every tensor op rounding to x.dtype (GEMMs accumulate
+    in fp32 and round once; the two scalings and the sums round one by one; `0 + first` is exact).
+    loras: sequence of (lora_down [n*r, in], [lora_up_i [out/n, r]] * n, multiplier, alpha_scale); the up
+    projection of a fused layer is one Linear per chunk of the rank axis, results concatenated
+    (lora_utils.py:12-21).  alpha_scale is held in x.dtype (longcat_video_dit.py:221 casts the buffer)."""
+    dt = x.dtype
+    lin = lambda a, w: (a.float() @ w.float().t()).to(dt)
+    org = (x.float() @ weight.float().t() + (0 if bias is None else bias.float())).to(dt)
+    total = None
+    for down, ups, multiplier, alpha_scale in loras:
+        lx = lin(x, down)
+        chunks = torch.chunk(lx, len(ups), dim=-1)
+        lx = torch.cat([lin(c, u) for c, u in zip(chunks, ups)], dim=-1)
+        a = torch.tensor(alpha_scale, dtype=dt).float()
+        term = ((lx.float() * float(torch.tensor(multiplier, dtype=torch.float32))).to(dt).float() * a).to(dt)
+        total = term if total is None else (total.float() + term.float()).to(dt)
+    return org if total is None else (org.float() + total.float()).to(dt)
+

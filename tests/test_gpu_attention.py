@@ -88,6 +88,26 @@ def test_variable_lengths_and_empty_rows():
     assert torch.allclose(lse[~empty], want_lse[~empty], atol=2e-3)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_malformed_lists_are_clamped(dtype):
+    """Block indices outside [0, nbk) and lengths outside [0, list width] are clamped by the kernels, so a bad list
+    costs wrong numbers for that query block and never an access outside k and v."""
+    q, k, v = seeded_qkv(27, 1, 2, 192, 320, 128, dtype)
+    idx, _ = random_lists(27, 1, 2, 3, 5, 3)
+    bad = idx.clone()                      # rows chosen so that the clamped lists hold no block twice
+    bad[0, 0, 0] = torch.tensor([-1, 2, 3])
+    bad[0, 0, 1] = torch.tensor([1, 2, 5])
+    bad[0, 1, 2] = torch.tensor([0, 2 ** 30, 1])
+    lens = torch.tensor([[[3, 3, 99], [-4, 3, 3]]], dtype=torch.int32)
+    o, lse = run(q, k, v, bad, lens)
+    mask = O.block_mask_from_indices(bad.clamp(0, 4), lens.clamp(0, 3), 5)
+    want, want_lse = O.masked_dense_attention(q, k, v, mask, 64, 64, 1 / math.sqrt(128))
+    close(o, want, dtype)
+    assert torch.all(o[0, 1, :64] == 0)
+    ok = ~torch.isinf(want_lse)
+    assert torch.allclose(lse[ok], want_lse[ok], atol=2e-3)
+
+
 @pytest.mark.parametrize("pattern", ["tail", "first16", "second_half", "sparse"])
 def test_padded_keys_are_masked(pattern):
     q, k, v = seeded_qkv(24, 1, 1, 128, 256, 128, torch.bfloat16)

@@ -239,6 +239,81 @@ def test_dit_self_attention_branch():
     assert d.max() <= 6e-2 and d.mean() <= 4e-3, (d.max(), d.mean())
 
 
+def L():
+    from longcat_video_amd.modules import lora
+    return lora
+
+
+def _branch(g, K, N, r, n_sep, multiplier, alpha, scale=0.05, integers=False):
+    if integers:
+        rnd = lambda *s: torch.randint(-2, 3, s, generator=g).bfloat16()
+    else:
+        rnd = lambda *s: (torch.randn(*s, generator=g) * scale).bfloat16()
+    down = rnd(n_sep * r, K)
+    ups = [rnd(N // n_sep, r) for _ in range(n_sep)]
+    return L().LoRABranch(down, ups, multiplier, alpha), (down, ups, multiplier, alpha / r)
+
+
+def test_lora_linear_integer_inputs_are_exact():
+    """Small integers make every GEMM, scaling and sum exact, so the three GEMMs (one of them with row
+    strides, in three column slices), and the combining pass must reproduce the oracle bit for bit."""
+    g = torch.Generator().manual_seed(30)
+    K, N, r = 256, 384, 128
+    x = torch.randint(-2, 3, (200, K), generator=g).bfloat16()
+    w = torch.randint(-2, 3, (N, K), generator=g).bfloat16()
+    b = torch.randint(-2, 3, (N,), generator=g).bfloat16()
+    br1, t1 = _branch(g, K, N, r, 3, 2.0, 64, integers=True)        # alpha_scale 0.5
+    br2, t2 = _branch(g, K, N, r, 1, 0.5, 32, integers=True)        # alpha_scale 0.25
+    for brs, terms in (([br1], [t1]), ([br1, br2], [t1, t2])):
+        want = O.lora_linear(x, w, b, terms)
+        for br in brs:
+            br.to("cuda")
+        got = L().lora_linear(x.cuda(), w.cuda(), b.cuda(), brs).cpu()
+        assert torch.equal(got, want)
+    br1.use_lora = br2.use_lora = False                            # set_use_lora(False): plain Linear
+    assert torch.equal(L().lora_linear(x.cuda(), w.cuda(), b.cuda(), [br1, br2]).cpu(), O.lora_linear(x, w, b, []))
+
+
+def test_lora_linear_random_inputs():
+    g = torch.Generator().manual_seed(31)
+    K, N, r = 512, 1536, 128
+    x = torch.randn(300, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16()
+    b = torch.randn(N, generator=g).bfloat16()
+    br, term = _branch(g, K, N, r, 3, 0.8, 64)
+    want = O.lora_linear(x, w, b, [term]).float()
+    plain = O.lora_linear(x, w, b, []).float()
+    got = L().lora_linear(x.cuda(), w.cuda(), b.cuda(), [br.to("cuda")]).cpu().float()
+    # GEMM summation order differs from the oracle's: an ulp of each rounded term
+    assert torch.all((got - want).abs() <= 3 * BF16_ULP * (want.abs() + plain.abs() + 0.05))
+    assert (want - plain).abs().mean() > 10 * (got - want).abs().mean()      # the side branch is not lost in the tolerance
+
+
+def test_module_forward_with_lora_branches():
+    """longcat_video_dit.py:211-249: LoRA branches on attn.qkv (up-projection split in three) and attn.proj."""
+    shape = (4, 8, 8)
+    m = make_module(sparsity=0.5)
+    g = torch.Generator().manual_seed(32)
+    x = torch.randn(1, 256, 512, generator=g).bfloat16()
+    bq, tq = _branch(g, 512, 1536, 128, 3, 1.0, 64, scale=0.02)
+    bp, tp = _branch(g, 512, 512, 128, 1, 1.0, 64, scale=0.02)
+    sd = {k: v.detach().cpu() for k, v in m.state_dict().items()}
+    prm = dict(sparsity=0.5, chunk_3d_shape_q=(4, 4, 4), chunk_3d_shape_k=(4, 4, 4))
+    args = (x, sd["qkv.weight"], sd["qkv.bias"], sd["proj.weight"], sd["proj.bias"], sd["q_norm.weight"],
+            sd["k_norm.weight"], shape, m.num_heads, prm, 0)
+    want = O.attention_module_forward(*args, qkv_loras=[tq], proj_loras=[tp])
+    plain = O.attention_module_forward(*args)
+    m = m.cuda()
+    m.qkv_loras, m.proj_loras = [bq.to("cuda")], [bp.to("cuda")]
+    got = m(x.cuda(), shape=shape).cpu()
+    d = (got.float() - want.float()).abs()
+    assert d.max() <= 2e-2 and d.mean() <= 2e-3, (d.max(), d.mean())
+    assert (want.float() - plain.float()).abs().mean() > 5 * d.mean()        # the branches change the result visibly
+    r = torch.randn(1, 256, 512, generator=g).bfloat16()
+    got_r = m(x.cuda(), shape=shape, residual=r.cuda()).cpu()
+    assert torch.equal(got_r, got + r)
+
+
 def test_unbuilt_branches_raise():
     m = make_module().cuda()
     x = torch.zeros(1, 256, 512, dtype=torch.bfloat16, device="cuda")

@@ -119,3 +119,69 @@ def test_gated_residual_closed_forms():
     gate = torch.randn(B, T, 1, C, generator=g)
     want = (x.float() + gate.expand(B, T, per, C).reshape(B, T * per, C) * y.float()).bfloat16()
     assert torch.equal(O.gated_residual_fp32(x, gate, y), want)
+
+
+# ---------------------------------------------------------------- LoRA side branches
+def _lora_case(seed, M=12, K=16, N=24, r=4, n_sep=1, integers=False, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    if integers:
+        rnd = lambda *s: torch.randint(-2, 3, s, generator=g).to(dtype)
+    else:
+        rnd = lambda *s: torch.randn(*s, generator=g).to(dtype)
+    x, w, b = rnd(M, K), rnd(N, K), rnd(N)
+    down = rnd(n_sep * r, K)
+    ups = [rnd(N // n_sep, r) for _ in range(n_sep)]
+    return x, w, b, down, ups
+
+
+def test_lora_with_zero_up_weights_is_the_plain_linear():
+    # the state right after LoRAModule.__init__ (lora_utils.py:60-65: lora_up zero-initialised)
+    x, w, b, down, ups = _lora_case(0, n_sep=3)
+    plain = torch.nn.functional.linear(x.float(), w.float(), b.float()).bfloat16()
+    got = O.lora_linear(x, w, b, [(down, [torch.zeros_like(u) for u in ups], 1.0, 0.5)])
+    assert torch.equal(got, plain)
+    assert torch.equal(O.lora_linear(x, w, b, []), plain)
+
+
+def test_lora_on_integers_equals_the_merged_weight():
+    # small integers: every product, sum and rounding is exact, so the side branch must equal the
+    # textbook merged form x (W + m a U D)^T + b
+    x, w, b, down, ups = _lora_case(1, integers=True)
+    m, a = 2.0, 0.5
+    merged = w.double() + m * a * (ups[0].double() @ down.double())
+    want = x.double() @ merged.t() + b.double()
+    got = O.lora_linear(x, w, b, [(down, ups, m, a)])
+    assert torch.equal(got.double(), want)
+
+
+def test_lora_split_up_projection_is_block_diagonal():
+    x, w, b, down, ups = _lora_case(2, n_sep=3, integers=True)
+    r = 4
+    full = torch.zeros(24, 12, dtype=torch.bfloat16)
+    for i, u in enumerate(ups):
+        full[8 * i:8 * i + 8, r * i:r * i + r] = u
+    a = O.lora_linear(x, w, b, [(down, ups, 1.0, 1.0)])
+    c = O.lora_linear(x, w, b, [(down, [full], 1.0, 1.0)])
+    assert torch.equal(a, c)
+    # and a transposed or shifted block assignment would not
+    wrong = torch.zeros_like(full)
+    for i, u in enumerate(ups):
+        wrong[8 * i:8 * i + 8, r * ((i + 1) % 3):r * ((i + 1) % 3) + r] = u
+    assert not torch.equal(a, O.lora_linear(x, w, b, [(down, [wrong], 1.0, 1.0)]))
+
+
+def test_lora_rounding_chain_and_two_branches():
+    # against the eager expression of longcat_video_dit.py:239-247 written with torch's own bf16 ops
+    # (scalar products and sums of bf16 tensors round once per op); the GEMMs are taken in fp32 and rounded
+    x, w, b, down, ups = _lora_case(3, n_sep=1)
+    _, _, _, down2, ups2 = _lora_case(4, n_sep=3)
+    lin = lambda t, wt: (t.float() @ wt.float().t()).bfloat16()
+    org = (x.float() @ w.float().t() + b.float()).bfloat16()
+    total = 0
+    for d, u, m, a in ((down, ups, 0.7, 0.5), (down2, ups2, 1.3, 0.25)):
+        lx = lin(x, d)
+        lx = torch.cat([lin(c, ui) for c, ui in zip(torch.chunk(lx, len(u), dim=-1), u)], dim=-1)
+        total = total + lx * m * torch.tensor(a, dtype=torch.bfloat16)
+    want = org + total
+    got = O.lora_linear(x, w, b, [(down, ups, 0.7, 0.5), (down2, ups2, 1.3, 0.25)])
+    assert want.dtype == torch.bfloat16 and torch.equal(got, want)
