@@ -251,6 +251,8 @@ int make_plan(const bsa_3d_params* p, Plan* pl) {
     pl->Sqp = (int64_t)pl->nbq * pl->gq.chunk();
     pl->Skp = (int64_t)pl->nbk * pl->gk.chunk();
     pl->es = dtype_size(p->dtype);
+    if ((pl->Sqp / 64) * (int64_t)p->B * p->Hn > 0x7fffffffLL || (p->dtype != BSA_F32 && pl->Skp >= (1 << 24)) || pl->Skp > 0x7fffffffLL)
+        return set_error(BSA_ERR_UNSUPPORTED, "problem too large (32-bit work item indices, 24-bit key rows for the 16-bit types)");
     const size_t bh = (size_t)p->B * p->Hn;
     size_t off = 0;
     auto take = [&](size_t bytes) { const size_t o = off; off += up256(bytes); return o; };
