@@ -55,6 +55,24 @@ def make_inputs(torch, latent, seed, rms):
     return out
 
 
+def make_coherent_inputs(torch, latent, seed):
+    """q = k = smooth functions of the grid position plus noise (per-head random low frequencies), v random:
+    pooled scores then fall off with distance, so neighbouring query blocks select largely the same KV blocks,
+    as attention over real video does.  Not the headline workload; shows the kernel when tiles are shared."""
+    T, H, W = latent
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    ax = lambda n, shape: torch.arange(n, device="cuda").view(shape).expand(T, H, W).reshape(-1, 1).float() / 4
+    pos = torch.cat([ax(T, (T, 1, 1)), ax(H, (1, H, 1)), ax(W, (1, 1, W))], 1)          # in chunks
+    q = torch.empty(1, HEADS, T * H * W, D, dtype=torch.bfloat16, device="cuda")
+    for h in range(HEADS):
+        freq = torch.randn(3, D, generator=g, device="cuda") * 0.3
+        phase = torch.rand(1, D, generator=g, device="cuda") * 2 * math.pi
+        x = torch.cos(pos @ freq + phase) * math.sqrt(2) + torch.randn(pos.shape[0], D, generator=g, device="cuda")
+        q[0, h] = (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
+    v = torch.randn(1, HEADS, T * H * W, D, generator=g, device="cuda").bfloat16()
+    return q, q.clone(), v
+
+
 def time_events(torch, fn, steps, warmup):
     for _ in range(warmup):
         fn()
@@ -192,6 +210,8 @@ def main():
                          "for the cond/noise split and for the attention module")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the CPU baseline's attention sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--data", default="random", choices=["random", "coherent"],
+                    help="random (the benchmark's definition) or spatially coherent q/k (c2, c3 only; no CPU baseline)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (the operator shards over heads; "
@@ -208,7 +228,8 @@ def main():
     if args.workload == "c5":
         return run_c5(torch, args)
     latent, sparsity, seed, rms, desc = WORKLOADS[args.workload]
-    q, k, v = make_inputs(torch, latent, seed, rms)
+    coherent = args.data == "coherent"
+    q, k, v = make_coherent_inputs(torch, latent, seed) if coherent else make_inputs(torch, latent, seed, rms)
     prm = dict(sparsity=sparsity, chunk_3d_shape_q=list(CHUNK), chunk_3d_shape_k=list(CHUNK))
 
     # ---- whole operator: warm-up, then exactly K timed steps between synchronisations ----
@@ -259,7 +280,10 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic N(0,1) q/k/v%s, seeded on the GPU" % (" with per-head RMS-normalised q/k" if rms else ""),
+        "dtype": "bf16",
+        "data": ("synthetic, spatially coherent q = k (smooth in the grid position + noise, RMS-normalised), random v, seeded on the GPU"
+                 if coherent else
+                 "synthetic N(0,1) q/k/v%s, seeded on the GPU" % (" with per-head RMS-normalised q/k" if rms else "")),
         "config": {"workload": "%s: %s" % (args.workload, desc), "chunk": list(CHUNK), "kv_blocks": nbk, "k_sel": k_sel,
                    "block_pairs": pairs, "padded_tokens": Sp},
         "ms_per_layer": round(ms_step, 4),
@@ -271,10 +295,10 @@ def main():
         "permute_gbs": round(permute_bytes / (ms_permute * 1e-3) / 1e9, 1),
         "roofline": {"kernel": "fwd_mfma_kernel<bf16> (all launches of one layer)", "bound": "mfma", "achieved": round(tflops_attn, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops_attn / PEAK_BF16_TFLOPS, 4),
-                     "traffic": ATTENTION_TRAFFIC_BYTES.get(args.workload), "ms": round(ms_attn, 4)},
+                     "traffic": None if coherent else ATTENTION_TRAFFIC_BYTES.get(args.workload), "ms": round(ms_attn, 4)},
     }
     del o
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not coherent:
         result["cpu_baseline"] = cpu_baseline(torch, latent, sparsity, seed, rms, args.cpu_seconds)
         result["cpu_baseline"]["value"] = round(result["cpu_baseline"]["value"], 5)
         result["cpu_baseline"]["ms_per_layer"] = round(result["cpu_baseline"]["ms_per_layer"], 1)

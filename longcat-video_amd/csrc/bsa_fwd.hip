@@ -47,6 +47,9 @@
 // L2 hits (the 4 MB L2 of an XCD cannot hold the 47 MB of K/V of one 720p head,
 // and L2 misses are served at only ~8 TB/s for 16 KB tiles).  One launch of the
 // whole grid loses this: workgroups then start whenever a slot frees up.
+// Within a round every XCD takes a contiguous run of the query blocks (workgroup b
+// runs on XCD b % 8): spatial neighbours select largely the same KV blocks on real
+// inputs, and only the workgroups of one XCD share an L2.
 #include "bsa_mfma.h"
 
 namespace bsa {
@@ -114,7 +117,15 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
         vaddr[t] = vkey0 * kD + ((chunk ^ vsw) << 3) + (s16 & 1) * 4;
     }
 
-    for (int item = item_begin + blockIdx.x; item < item_end; item += gridDim.x) {
+    // Workgroup b of a launch runs on XCD b % 8 (round-robin dispatch).  Each XCD gets a contiguous run of
+    // the launch's work items: neighbouring query blocks tend to select the same KV blocks, and only
+    // workgroups of one XCD share an L2.
+    int local = blockIdx.x;
+    {
+        const int n = item_end - item_begin, x = local & 7;
+        local = x * (n >> 3) + min(x, n & 7) + (local >> 3);
+    }
+    for (int item = item_begin + local; item < item_end; item += gridDim.x) {
     const int bh = item / nqt;
     const int qtile = item % nqt;
     const int64_t qrow0 = (int64_t)qtile * kTile;
