@@ -315,7 +315,11 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
         l_i += psum;
         mask_tile(s_next, mask_next);
         row_pref = tile_row_sm[it + 3 < nloc ? it + 3 : 0];  // consumed at the top of the next step
-        // O += P(it) V(it); the row maximum of S(it+1) fills the VALU slots between the MFMAs
+        // O += P(it) V(it); the row maximum of S(it+1) fills the VALU slots between the MFMAs.
+        // This stretch runs at a raised wave priority: of the two wavefronts that share a SIMD (one of
+        // each resident workgroup) the one in its MFMA-only phase goes first, reaches the top of its next
+        // step - where the tile loads are issued - sooner, and the two fall into alternating phases.
+        __builtin_amdgcn_s_setprio(1);
         float mx = fmaxf(s_next[0], s_next[1]);
 #pragma unroll
         for (int u = 0; u < 8; ++u) {        // u = 2*t + c
@@ -324,6 +328,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
             if (u < 7) mx = fmaxf(fmaxf(mx, s_next[2 * u + 2]), s_next[2 * u + 3]);
             __builtin_amdgcn_sched_barrier(0);
         }
+        __builtin_amdgcn_s_setprio(0);
         raise_max(finish_max(mx));
     };
     // last_step: the final tile of the list, nothing left to prefetch or to overlap with.
