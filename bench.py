@@ -36,8 +36,8 @@ WORKLOADS = {
 }
 # Bytes that leave L2 per layer in the attention kernel (all of its launches), from rocprofv3 --pmc
 # FETCH_SIZE (x2) and WRITE_SIZE (x1) as recorded in profiles/bsa_operator_c3_720p.md: 96 launches
-# x (731.8 MB + 7.4 MB).  Re-measure after kernel changes.
-ATTENTION_TRAFFIC_BYTES = {"c3": 96 * (731.8e6 + 7.4e6)}
+# x (607.1 MB + 7.4 MB).  Re-measure after kernel changes.
+ATTENTION_TRAFFIC_BYTES = {"c3": 96 * (607.1e6 + 7.4e6)}
 CHUNK = (4, 4, 4)
 HEADS, D = 32, 128
 
