@@ -107,14 +107,16 @@ template <typename T>
 __global__ __launch_bounds__(256) void gated_residual_kernel(const T* __restrict__ x, const T* __restrict__ y,
                                                              const float* __restrict__ gate, T* __restrict__ out,
                                                              int64_t rows, int rows_per_group, int dim) {
-    const int per_row = dim / 8;
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= rows * per_row) return;
-    const int64_t row = i / per_row;
-    const int d = (int)(i % per_row) * 8;
+    // the launch is limited to 2^31 threads: 32-bit divisions (64-bit ones cost more than the 48 bytes moved)
+    const uint32_t per_row = (uint32_t)dim / 8;
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= (uint64_t)rows * per_row) return;
+    const uint32_t row_u = i / per_row;
+    const int64_t row = row_u;
+    const int d = (int)(i - row_u * per_row) * 8;
     const uint4 xr = *reinterpret_cast<const uint4*>(x + row * dim + d);
     const uint4 yr = *reinterpret_cast<const uint4*>(y + row * dim + d);
-    const float* g = gate + (row / rows_per_group) * dim + d;
+    const float* g = gate + (int64_t)(row_u / (uint32_t)rows_per_group) * dim + d;
     const float4 g0 = *reinterpret_cast<const float4*>(g), g1 = *reinterpret_cast<const float4*>(g + 4);
     const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
     const T* xe = reinterpret_cast<const T*>(&xr);
@@ -181,27 +183,62 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(const T* __restrict__ sr
     constexpr int D = 128;
     constexpr int nt = (D - 4 * (D / 6)) / 2, nh = (D / 6), nw = (D / 6);   // pairs per axis: 22, 21, 21
     const int sub = threadIdx.x & 15;
-    const int64_t S = (int64_t)Tn * Hg * Wg;
-    const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-    if (row >= (int64_t)B * Hn * S) return;
-    int64_t s;
-    int hd, b;
-    if (head_fastest) { hd = (int)(row % Hn); s = (row / Hn) % S; b = (int)(row / (S * Hn)); }
-    else { s = row % S; hd = (int)((row / S) % Hn); b = (int)(row / (S * Hn)); }
-    const T* p = src + b * sB + hd * sH + s * sS;
-    T* o = dst + b * dB + hd * dH + s * dS;
-
-    const uint4 raw = *reinterpret_cast<const uint4*>(p + sub * 8);
+    // row counts fit 31 bits (checked by the caller): 32-bit divisions, the 64-bit ones cost more than the move
+    const uint32_t S = (uint32_t)Tn * Hg * Wg;
+    const uint32_t rows = (uint32_t)B * Hn * S;
+    // Four rows in flight per 16-lane group.  When the heads of a token lie next to each other in the
+    // source (and their count is a multiple of four) the four rows are four heads of one token: they
+    // share the token's position and rotation angles, which are then worked out once.
+    constexpr int R = 4;
+    const bool share = head_fastest && (Hn % R) == 0;
+    const uint32_t group = blockIdx.x * 16u + (threadIdx.x >> 4);
+    uint32_t s_of[R];
+    T* o_of[R];
+    uint4 raw_of[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const uint32_t row = share ? group * R + j : blockIdx.x * (16u * R) + (threadIdx.x >> 4) + 16u * j;
+        if (row >= rows) { o_of[j] = nullptr; s_of[j] = 0; continue; }
+        uint32_t s, hd, b;
+        if (head_fastest) { const uint32_t t = row / Hn; hd = row - t * Hn; b = t / S; s = t - b * S; }
+        else { const uint32_t t = row / S; s = row - t * S; b = t / Hn; hd = t - b * Hn; }
+        s_of[j] = s;
+        o_of[j] = dst + b * dB + hd * dH + s * dS;
+        raw_of[j] = *reinterpret_cast<const uint4*>(src + b * sB + hd * sH + s * sS + sub * 8);
+    }
+    uint4 wraw = make_uint4(0, 0, 0, 0);
+    if (w != nullptr) wraw = *reinterpret_cast<const uint4*>(w + sub * 8);
+    // cos / sin of this lane's four rotation pairs at token s
+    auto angles = [&](uint32_t s, float (&c)[4], float (&sn)[4]) {
+        const uint32_t u = s / (uint32_t)Wg, v = u / (uint32_t)Hg;
+        const int wi = (int)(s - u * Wg), hi = (int)(u - v * Hg), ti = t0 + (int)v;
+        const float* cos_t = tab;                        const float* sin_t = cos_t + (int64_t)Ttab * nt;
+        const float* cos_h = sin_t + (int64_t)Ttab * nt; const float* sin_h = cos_h + (int64_t)Hg * nh;
+        const float* cos_w = sin_h + (int64_t)Hg * nh;   const float* sin_w = cos_w + (int64_t)Wg * nw;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int pair = sub * 4 + jj;         // 0..63
+            if (pair < nt) { c[jj] = cos_t[ti * nt + pair]; sn[jj] = sin_t[ti * nt + pair]; }
+            else if (pair < nt + nh) { c[jj] = cos_h[hi * nh + pair - nt]; sn[jj] = sin_h[hi * nh + pair - nt]; }
+            else { c[jj] = cos_w[wi * nw + pair - nt - nh]; sn[jj] = sin_w[wi * nw + pair - nt - nh]; }
+        }
+    };
+    float c[4] = {1.f, 1.f, 1.f, 1.f}, sn[4] = {0.f, 0.f, 0.f, 0.f};
+    if (tab != nullptr && share) angles(s_of[0], c, sn);      // row 0 of a group exists whenever any does
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+    if (o_of[j] == nullptr) continue;
+    T* o = o_of[j];
+    const uint4 raw = raw_of[j];
     if (w == nullptr && tab == nullptr) {                 // plain move
         *reinterpret_cast<uint4*>(o + sub * 8) = raw;
-        return;
+        continue;
     }
     const T* e = reinterpret_cast<const T*>(&raw);
     float f[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) f[i] = (float)e[i];
     if (w != nullptr) {
-        const uint4 wraw = *reinterpret_cast<const uint4*>(w + sub * 8);
         const T* we = reinterpret_cast<const T*>(&wraw);
         float ss = 0.f;
 #pragma unroll
@@ -214,27 +251,20 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(const T* __restrict__ sr
     }
     T res[8];
     if (tab != nullptr) {
-        const int wi = (int)(s % Wg), hi = (int)((s / Wg) % Hg), ti = t0 + (int)(s / ((int64_t)Wg * Hg));
-        const float* cos_t = tab;                        const float* sin_t = cos_t + (int64_t)Ttab * nt;
-        const float* cos_h = sin_t + (int64_t)Ttab * nt; const float* sin_h = cos_h + (int64_t)Hg * nh;
-        const float* cos_w = sin_h + (int64_t)Hg * nh;   const float* sin_w = cos_w + (int64_t)Wg * nw;
+        if (!share) angles(s_of[j], c, sn);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int pair = sub * 4 + j;          // 0..63
-            float c, sn;
-            if (pair < nt) { c = cos_t[ti * nt + pair]; sn = sin_t[ti * nt + pair]; }
-            else if (pair < nt + nh) { c = cos_h[hi * nh + pair - nt]; sn = sin_h[hi * nh + pair - nt]; }
-            else { c = cos_w[wi * nw + pair - nt - nh]; sn = sin_w[wi * nw + pair - nt - nh]; }
-            const float x0 = f[2 * j], x1 = f[2 * j + 1];
+        for (int jj = 0; jj < 4; ++jj) {
+            const float x0 = f[2 * jj], x1 = f[2 * jj + 1];
             // two products, then one add, each rounded: the order of operations of the eager expression
-            res[2 * j] = (T)__fadd_rn(__fmul_rn(x0, c), __fmul_rn(-x1, sn));
-            res[2 * j + 1] = (T)__fadd_rn(__fmul_rn(x1, c), __fmul_rn(x0, sn));
+            res[2 * jj] = (T)__fadd_rn(__fmul_rn(x0, c[jj]), __fmul_rn(-x1, sn[jj]));
+            res[2 * jj + 1] = (T)__fadd_rn(__fmul_rn(x1, c[jj]), __fmul_rn(x0, sn[jj]));
         }
     } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i) res[i] = (T)f[i];
     }
     *reinterpret_cast<uint4*>(o + sub * 8) = *reinterpret_cast<const uint4*>(res);
+    }
 }
 
 // ------------------------------------------------------------- linear (GEMM)
@@ -297,7 +327,7 @@ int bsa_gated_residual(const void* x, const void* y, const float* gate, void* ou
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(out)) & 15u)
         return set_error(BSA_ERR_BAD_ARG, "gated_residual: pointers must be 16-byte aligned");
     const int64_t n = rows * (dim / 8);
-    if ((n + 255) / 256 > 0x7fffffffLL) return set_error(BSA_ERR_UNSUPPORTED, "gated_residual: too many elements");
+    if (n > 0x7fffffffLL) return set_error(BSA_ERR_UNSUPPORTED, "gated_residual: too many elements (32-bit thread indices)");
     const dim3 grid((unsigned)((n + 255) / 256)), block(256);
     if (dtype == BSA_BF16)
         hipLaunchKernelGGL((gated_residual_kernel<__bf16>), grid, block, 0, (hipStream_t)stream, (const __bf16*)x, (const __bf16*)y, gate, (__bf16*)out, rows, rows_per_group, dim);
@@ -353,8 +383,8 @@ int bsa_norm_rope(const void* src, const int64_t src_strides[3], void* dst, cons
         return set_error(BSA_ERR_BAD_ARG, "norm_rope: pointers must be 16-byte aligned");
     if (!(eps >= 0.f)) return set_error(BSA_ERR_BAD_ARG, "norm_rope: eps must be non-negative");
     const int64_t rows = (int64_t)B * Hn * T * H * W;
-    if ((rows + 15) / 16 > 0x7fffffffLL) return set_error(BSA_ERR_UNSUPPORTED, "norm_rope: too many rows");
-    const dim3 grid((unsigned)((rows + 15) / 16)), block(256);
+    if (rows > 0x7fffffffLL) return set_error(BSA_ERR_UNSUPPORTED, "norm_rope: too many rows (32-bit row indices)");
+    const dim3 grid((unsigned)((rows + 63) / 64)), block(256);       // 16 lane groups x 4 rows each
     const int head_fastest = src_strides[1] < src_strides[2] ? 1 : 0;
     if (dtype == BSA_BF16)
         hipLaunchKernelGGL((norm_rope_kernel<__bf16>), grid, block, 0, (hipStream_t)stream, (const __bf16*)src, src_strides[0],
