@@ -284,6 +284,17 @@ int bsa_linear_bf16_ld(const void* x, int64_t ldx, const void* w, int64_t ldw, c
                        void* out, int64_t ldo, int64_t M, int N, int K, void* workspace, size_t workspace_bytes,
                        void* stream);
 
+/* One-time tuning of a linear shape (no counterpart in the reference, whose nn.Linear leaves the choice to the
+ * BLAS library): runs every algorithm hipBLASLt proposes for this call (up to 32, each four times on the given
+ * buffers; `out` is overwritten), and remembers the fastest for later bsa_linear_bf16 / _ld calls with the same
+ * M, N, K, row strides, bias / residual presence in this process.  Unlike every other entry point it WAITS for
+ * the stream, so call it at set-up, outside graph capture.  Returns the number of algorithms timed (> 0) or a
+ * negative status; default_ms / best_ms (optional) receive the time of the algorithm an untuned call uses and
+ * of the one chosen.  Algorithms differ in summation order, so results can differ in the last bit. */
+int bsa_linear_bf16_tune(const void* x, int64_t ldx, const void* w, int64_t ldw, const void* bias, const void* residual,
+                         void* out, int64_t ldo, int64_t M, int N, int K, void* workspace, size_t workspace_bytes,
+                         void* stream, float* default_ms, float* best_ms);
+
 /* LoRA side branches of a Linear (longcat_video_dit.py:234-249): out = org + total, where total sums
  * up_i * multiplier_i * alpha_scale_i over the active branches, up_i = lora_up(lora_down(x)) already
  * computed (bsa_linear_bf16 / _ld).  Every product and every sum is rounded to `dtype` as the eager

@@ -5,7 +5,9 @@
 
 #include <hipblaslt/hipblaslt.h>
 
+#include <map>
 #include <mutex>
+#include <tuple>
 
 namespace bsa {
 namespace {
@@ -268,9 +270,22 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(const T* __restrict__ sr
 }
 
 // ------------------------------------------------------------- linear (GEMM)
+// Shape of a linear call -> the algorithm bsa_linear_bf16_tune measured to be the fastest for it.
+struct LinearKey {
+    int64_t M, ldx, ldw, ldo;
+    int N, K, bias, residual;
+    bool operator<(const LinearKey& o) const {
+        return std::tie(M, ldx, ldw, ldo, N, K, bias, residual) < std::tie(o.M, o.ldx, o.ldw, o.ldo, o.N, o.K, o.bias, o.residual);
+    }
+};
+struct TunedAlgo {
+    hipblasLtMatmulAlgo_t algo;
+    size_t workspace;
+};
 struct LtState {
     std::mutex mu;
     hipblasLtHandle_t handle = nullptr;
+    std::map<LinearKey, TunedAlgo> tuned;
 };
 LtState& lt_state() { static LtState s; return s; }
 
@@ -415,9 +430,25 @@ int bsa_linear_bf16(const void* x, const void* w, const void* bias, const void* 
     return bsa_linear_bf16_ld(x, K, w, K, bias, residual, out, N, M, N, K, workspace, workspace_bytes, stream);
 }
 
+static int linear_impl(const void* x, int64_t ldx, const void* w, int64_t ldw, const void* bias, const void* residual,
+                       void* out, int64_t ldo, int64_t M, int N, int K, void* workspace, size_t workspace_bytes,
+                       void* stream, bool tune, float* default_ms, float* best_ms);
+
 int bsa_linear_bf16_ld(const void* x, int64_t ldx, const void* w, int64_t ldw, const void* bias, const void* residual,
                        void* out, int64_t ldo, int64_t M, int N, int K, void* workspace, size_t workspace_bytes,
                        void* stream) {
+    return linear_impl(x, ldx, w, ldw, bias, residual, out, ldo, M, N, K, workspace, workspace_bytes, stream, false, nullptr, nullptr);
+}
+
+int bsa_linear_bf16_tune(const void* x, int64_t ldx, const void* w, int64_t ldw, const void* bias, const void* residual,
+                         void* out, int64_t ldo, int64_t M, int N, int K, void* workspace, size_t workspace_bytes,
+                         void* stream, float* default_ms, float* best_ms) {
+    return linear_impl(x, ldx, w, ldw, bias, residual, out, ldo, M, N, K, workspace, workspace_bytes, stream, true, default_ms, best_ms);
+}
+
+static int linear_impl(const void* x, int64_t ldx, const void* w, int64_t ldw, const void* bias, const void* residual,
+                       void* out, int64_t ldo, int64_t M, int N, int K, void* workspace, size_t workspace_bytes,
+                       void* stream, bool tune, float* default_ms, float* best_ms) {
     if (!x || !w || !out) return set_error(BSA_ERR_BAD_ARG, "linear: null pointer");
     if (M <= 0 || N <= 0 || K <= 0) return set_error(BSA_ERR_BAD_ARG, "linear: sizes must be positive");
     if (ldx < K || ldw < K || ldo < N) return set_error(BSA_ERR_BAD_ARG, "linear: a row stride is shorter than its row");
@@ -459,13 +490,56 @@ int bsa_linear_bf16_ld(const void* x, int64_t ldx, const void* w, int64_t ldw, c
         BSA_LT(hipblasLtMatmulPreferenceCreate(&pref));
         const uint64_t wsb = workspace_bytes;
         BSA_LT(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &wsb, sizeof(wsb)));
-        hipblasLtMatmulHeuristicResult_t heur[8];
+        const LinearKey key{M, ldx, ldw, ldo, N, K, bias ? 1 : 0, residual ? 1 : 0};
+        const auto hit = st.tuned.find(key);
+        if (!tune && hit != st.tuned.end() && hit->second.workspace <= workspace_bytes) {
+            BSA_LT(hipblasLtMatmul(st.handle, desc, &alpha, w, la, x, lb, &beta, residual ? residual : out, lc, out, lc,
+                                   &hit->second.algo, workspace, workspace_bytes, (hipStream_t)stream));
+            goto done;
+        }
+        constexpr int kMaxAlgos = 32;
+        hipblasLtMatmulHeuristicResult_t heur[kMaxAlgos];
         int found = 0, pick = -1;
-        BSA_LT(hipblasLtMatmulAlgoGetHeuristic(st.handle, desc, la, lb, lc, lc, pref, 8, heur, &found));
+        BSA_LT(hipblasLtMatmulAlgoGetHeuristic(st.handle, desc, la, lb, lc, lc, pref, tune ? kMaxAlgos : 8, heur, &found));
         // never hand the library less workspace than the algorithm says it uses
         for (int i = 0; i < found && pick < 0; ++i)
             if (heur[i].state == HIPBLAS_STATUS_SUCCESS && heur[i].workspaceSize <= workspace_bytes) pick = i;
         if (pick < 0) { rc = set_error(BSA_ERR_UNSUPPORTED, "linear: no GEMM algorithm for M=%lld N=%d K=%d within %zu bytes of workspace", (long long)M, N, K, workspace_bytes); goto done; }
+        if (tune) {
+            // every candidate once to warm up, then three timed runs; the stream is waited for
+            hipEvent_t e0 = nullptr, e1 = nullptr;
+            if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+                if (e0) (void)hipEventDestroy(e0);
+                rc = set_error(BSA_ERR_HIP, "linear tune: hipEventCreate failed");
+                goto done;
+            }
+            float best = 0.f;
+            int best_i = -1, tried = 0;
+            for (int i = 0; i < found; ++i) {
+                if (heur[i].state != HIPBLAS_STATUS_SUCCESS || heur[i].workspaceSize > workspace_bytes) continue;
+                bool ok = true;
+                for (int r = 0; r < 4 && ok; ++r) {
+                    if (r == 1) ok = hipEventRecord(e0, (hipStream_t)stream) == hipSuccess;
+                    ok = ok && hipblasLtMatmul(st.handle, desc, &alpha, w, la, x, lb, &beta, residual ? residual : out, lc, out, lc,
+                                               &heur[i].algo, workspace, workspace_bytes, (hipStream_t)stream) == HIPBLAS_STATUS_SUCCESS;
+                }
+                float ms = 0.f;
+                ok = ok && hipEventRecord(e1, (hipStream_t)stream) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+                     hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+                if (!ok) continue;
+                ms /= 3.f;
+                if (i == pick && default_ms) *default_ms = ms;
+                if (best_i < 0 || ms < best) { best = ms; best_i = i; }
+                ++tried;
+            }
+            (void)hipEventDestroy(e0);
+            (void)hipEventDestroy(e1);
+            if (best_i < 0) { rc = set_error(BSA_ERR_HIP, "linear tune: no candidate ran"); goto done; }
+            st.tuned[key] = TunedAlgo{heur[best_i].algo, heur[best_i].workspaceSize};
+            if (best_ms) *best_ms = best;
+            rc = tried;
+            goto done;
+        }
         BSA_LT(hipblasLtMatmul(st.handle, desc, &alpha, w, la, x, lb, &beta, residual ? residual : out, lc, out, lc,
                                &heur[pick].algo, workspace, workspace_bytes, (hipStream_t)stream));
     }

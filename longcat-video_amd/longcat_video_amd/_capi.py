@@ -56,6 +56,7 @@ SIGNATURES = {
     "bsa_qk_norm_rope": (_i, [_p, _strides, _p, _strides, _p, _p, _p] + [_i] * 6 + [_f, _i, _p]),
     "bsa_linear_bf16": (_i, [_p, _p, _p, _p, _p, _i64, _i, _i, _p, C.c_size_t, _p]),
     "bsa_linear_bf16_ld": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i, _i, _p, C.c_size_t, _p]),
+    "bsa_linear_bf16_tune": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i, _i, _p, C.c_size_t, _p, _p, _p]),
     "bsa_lora_add": (_i, [_p, _p, _p, _p, _i, _p, _i64, _i, _p]),
 }
 

@@ -101,6 +101,30 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
     return out.view(*x.shape[:-1], N)
 
 
+def tune_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], residual: bool = False,
+                workspace: Optional[torch.Tensor] = None):
+    """One-time choice of the GEMM algorithm for ``linear_bf16`` calls of this shape (rows of x, weight shape, bias and
+    residual presence): times what hipBLASLt proposes and keeps the fastest for the rest of the process.  Waits for
+    the stream; call at set-up.  Returns (algorithms timed, ms of the default choice, ms of the chosen one)."""
+    if not x.is_cuda:
+        raise RuntimeError("the engine runs on the GPU only")
+    K, N = x.shape[-1], weight.shape[0]
+    x2 = x.reshape(-1, K).contiguous()
+    w = weight.to(torch.bfloat16).contiguous()
+    b = None if bias is None else bias.to(torch.bfloat16).contiguous()
+    out = torch.empty(x2.shape[0], N, dtype=torch.bfloat16, device=x.device)
+    r = torch.zeros_like(out) if residual else None
+    if workspace is None:
+        workspace = _gemm_workspace(x.device)
+    d, best = C.c_float(0), C.c_float(0)
+    with torch.cuda.device(x.device):
+        n = _capi.load().bsa_linear_bf16_tune(_ptr(x2), K, _ptr(w), K, _ptr(b), _ptr(r), _ptr(out), N, x2.shape[0], N, K,
+                                              _ptr(workspace), workspace.numel(), _stream(x), C.byref(d), C.byref(best))
+    if n <= 0:
+        _capi.check(n if n < 0 else _capi.BSA_ERR_HIP, "linear tune")
+    return n, d.value, best.value
+
+
 _ROPE_TABLES = {}
 
 
@@ -205,6 +229,13 @@ class Attention(nn.Module):
             y = lora_linear(x, layer.weight, layer.bias, loras)
             return y if residual is None else y + residual
         return linear_bf16(x, layer.weight, layer.bias, residual=residual)
+
+    @torch.no_grad()
+    def tune(self, x: torch.Tensor, residual: bool = False):
+        """Picks the GEMM algorithms of the two projections for inputs shaped like x ([B, N, C]); see tune_linear."""
+        a = tune_linear(x, self.qkv.weight, self.qkv.bias)
+        b = tune_linear(x, self.proj.weight, self.proj.bias, residual=residual)
+        return a, b
 
     def _process_attn(self, q, k, v, shape, out=None):
         """attention.py:50-105, block-sparse branch; writes into `out` ([B,H,SQ,D] view) if given."""

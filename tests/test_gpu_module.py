@@ -322,3 +322,20 @@ def test_unbuilt_branches_raise():
     m.enable_bsa = False
     with pytest.raises(NotImplementedError):
         m(x, shape=(4, 8, 8))
+
+
+def test_linear_tuning_keeps_results_and_is_remembered():
+    """bsa_linear_bf16_tune times hipBLASLt's candidates for a shape and later calls of that shape use the winner;
+    the product stays the same GEMM (fp32 accumulation, one rounding; summation order may differ by an ulp)."""
+    g = torch.Generator().manual_seed(33)
+    x = torch.randn(1, 640, 512, generator=g).bfloat16().cuda()
+    w = (torch.randn(768, 512, generator=g) * 0.05).bfloat16().cuda()
+    b = torch.randn(768, generator=g).bfloat16().cuda()
+    before = M().linear_bf16(x, w, b).cpu()
+    n, default_ms, best_ms = M().tune_linear(x, w, b)
+    assert n >= 1 and 0 < best_ms <= default_ms * 1.001
+    after = M().linear_bf16(x, w, b).cpu()
+    want = x.cpu().float() @ w.cpu().float().t() + b.cpu().float()
+    for got in (before, after):
+        assert torch.all((got.float() - want).abs() <= want.abs() * BF16_ULP + 2e-3)
+    assert torch.equal(after, M().linear_bf16(x, w, b).cpu())          # the remembered choice is deterministic
