@@ -266,3 +266,38 @@ def test_operator_replays_from_a_hip_graph():
         torch.cuda.synchronize()
         assert torch.equal(got, want), "replay %d differs from the eager result" % step
         assert got.abs().sum() > 0
+
+
+def _random_case(rnd):
+    chunks = [(4, 4, 4), (4, 4, 8), (2, 8, 4), (1, 4, 16), (4, 2, 8), (2, 4, 8), (8, 2, 4), (1, 8, 8), (4, 8, 2), (2, 2, 16)]
+    chunk = rnd.choice(chunks)
+    nb = [rnd.randint(1, 3), rnd.randint(1, 5), rnd.randint(1, 5)]
+    lq = tuple(max(1, c * b - rnd.randint(0, c - 1)) for c, b in zip(chunk, nb))        # ragged in any axis
+    rect = rnd.random() < 0.25
+    lk = (lq[0] + rnd.randint(1, chunk[0] * 2), lq[1], lq[2]) if rect else lq            # more key frames than query frames
+    return dict(chunk=chunk, lq=lq, lk=lk, H=rnd.choice([1, 2, 3]), B=rnd.choice([1, 1, 2]),
+                dtype=rnd.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32]),
+                sparsity=rnd.choice([0.0, 0.25, 0.5, 0.75, 0.9]), strided=(not rect) and rnd.random() < 0.3)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_against_the_oracle(seed):
+    """Seeded random draws over chunk shapes, ragged and rectangular grids, batch and head counts, storage types,
+    sparsities and strided views of one projection output; every query block of every case is checked."""
+    import random
+    c = _random_case(random.Random(7000 + seed))
+    Sq, Sk = int(np.prod(c["lq"])), int(np.prod(c["lk"]))
+    g = torch.Generator().manual_seed(7000 + seed)
+    if c["strided"]:
+        qkv = torch.randn(c["B"], Sq, 3, c["H"], 128, generator=g).to(c["dtype"])
+        q, k, v = qkv.permute(2, 0, 3, 1, 4).unbind(0)
+        gq, gk, gv = qkv.cuda().permute(2, 0, 3, 1, 4).unbind(0)
+    else:
+        q, k, v = (torch.randn(c["B"], c["H"], s, 128, generator=g).to(c["dtype"]) for s in (Sq, Sk, Sk))
+        gq, gk, gv = q.cuda(), k.cuda(), v.cuda()
+    o, idx, lens, score = I()._bsa_3d(gq, gk, gv, c["lq"], c["lk"], c["sparsity"], c["chunk"], c["chunk"], True)
+    nbq = int(np.prod(O.block_grid(c["lq"], c["chunk"])))
+    for b in range(c["B"]):
+        check_against_oracle(q[b:b + 1], k[b:b + 1], v[b:b + 1], c["lq"], c["lk"], c["sparsity"], o[b:b + 1], idx[b:b + 1],
+                             lens[b:b + 1], score[b:b + 1], q_blocks=range(nbq), chunk=c["chunk"])
+    assert torch.isfinite(o.float()).all(), c
