@@ -212,3 +212,41 @@ def test_thw_attention_equals_permute_attend_unpermute(latent, chunk):
     got, lse = bi.attn_fwd_bsa_thw(q, k, v, latent, latent, chunk, chunk, idx, lens, sm_scale=0.11, return_lse=True)
     assert torch.equal(got, want)
     assert torch.equal(lse.cpu(), want_lse)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_lists_lengths_and_masks(seed):
+    """Seeded random draws: 64- and 128-token blocks, list widths, lengths from 0 to the width, lists in random
+    order, validity masks that blank random keys, whole tiles, whole 32-key halves or a tail, every storage type."""
+    import random
+    rnd = random.Random(6000 + seed)
+    B, H = rnd.choice([1, 1, 2]), rnd.choice([1, 2, 3])
+    bs_q, bs_k = rnd.choice([64, 64, 128]), rnd.choice([64, 64, 128])
+    nbq, nbk = rnd.randint(1, 6), rnd.randint(1, 12)
+    width = rnd.randint(1, nbk)
+    dtype = rnd.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+    Sq, Sk = nbq * bs_q, nbk * bs_k
+    g = torch.Generator().manual_seed(6000 + seed)
+    q, k, v = (torch.randn(B, H, s, 128, generator=g).to(dtype) for s in (Sq, Sk, Sk))
+    idx = torch.stack([torch.randperm(nbk, generator=g)[:width] for _ in range(B * H * nbq)]).view(B, H, nbq, width)
+    lens = torch.randint(0, width + 1, (B, H, nbq), generator=g, dtype=torch.int32)
+    valid, bits = None, None
+    mode = rnd.choice(["none", "rand", "tiles", "halves", "tail"])
+    if mode != "none":
+        valid = torch.ones(Sk, dtype=torch.bool)
+        if mode == "rand":
+            valid = torch.rand(Sk, generator=g) < 0.6
+        elif mode == "tiles":
+            valid.view(-1, 64)[torch.rand(Sk // 64, generator=g) < 0.4] = False
+        elif mode == "halves":
+            valid.view(-1, 32)[torch.rand(Sk // 32, generator=g) < 0.5] = False
+        else:
+            valid[rnd.randint(0, Sk - 1):] = False
+        bits = np.packbits(valid.numpy().reshape(-1, 64), axis=1, bitorder="little").view(np.uint64).reshape(-1)
+    o, lse = run(q, k, v, idx, lens, bs_q, bs_k, valid_bits=bits)
+    want, want_lse = O.masked_dense_attention(q, k, v, O.block_mask_from_indices(idx, lens, nbk), bs_q, bs_k,
+                                              1 / math.sqrt(128), key_valid=valid)
+    close(o, want, dtype)
+    fin = torch.isfinite(want_lse)
+    assert torch.allclose(lse[fin], want_lse[fin], atol=2e-3)
+    assert torch.all(torch.isinf(lse[~fin]) & (lse[~fin] < 0)) and torch.all(o[~fin] == 0)
