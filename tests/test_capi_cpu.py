@@ -134,3 +134,17 @@ def test_status_to_exception_mapping():
     with pytest.raises(NotImplementedError):
         _capi.check(rc)
     _capi.check(0)
+
+
+def test_header_and_library_from_a_plain_c_program(tmp_path):
+    """include/bsa_mi355x.h is C, and the library needs no Python or torch around it."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    exe = str(tmp_path / "capi_from_c")
+    src = os.path.join(ROOT, "tests", "capi_from_c.c")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), src, "-o", exe, "-ldl"], check=True)
+    _capi.load()                       # raises with the build hint if the library is missing
+    out = subprocess.run([exe, _capi.LIB_PATH], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0 and out.stdout.startswith("ok"), (out.returncode, out.stdout, out.stderr)
