@@ -552,14 +552,15 @@ hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t
     }
     // One launch per round of as many work items as the device runs at once: the workgroups of a
     // launch start together and walk their (ascending) KV lists in step, so that a tile fetched
-    // by one of them is still in L2 when its neighbours ask for it.  Rounds normally end at a
-    // (batch, head) boundary, so that all workgroups of a round share one head's K/V; when that
-    // would leave the last round of every head mostly empty (few query tiles per head), rounds
-    // run across the boundaries instead.
+    // by one of them is still in L2 when its neighbours ask for it.  When the query tiles of a head
+    // fill whole rounds, every round works on one head's K/V; otherwise the rounds run on across
+    // the (batch, head) boundaries rather than leave the last round of every head partly empty:
+    // an XCD takes a contiguous run of a round's items, so even in a round that holds two heads
+    // almost every XCD still works on one.
     const int per_head = (int)(Sq / kTile);
     const int round = resident_workgroups();
     const int tail = per_head % round;
-    const bool across = tail != 0 && tail * 10 < round * 7;
+    const bool across = tail != 0;
     const int n_outer = across ? 1 : B * Hn;
     const int n_inner = across ? B * Hn * per_head : per_head;
     for (int bh = 0; bh < n_outer; ++bh) {
