@@ -15,7 +15,9 @@ Differences from the reference, all supersets:
   * block indices are int32 inside the engine; the helpers that the reference
     returns int64 from (torch.topk) convert on the way out;
   * forward only: inputs that require grad are rejected while grad mode is on;
-  * ``cdf_threshold`` other than None raises NotImplementedError.
+  * the CDF selection rule (bsa_interface.py:226-266) keeps its weights in fp32 and its running sum in double
+    for every storage type, and ``get_select_indices_from_score`` takes the ``sm_scale`` the reference forgets
+    to pass on (bsa_interface.py:283, 285).
 """
 from __future__ import annotations
 
