@@ -3,13 +3,16 @@
 // score[bh, m, n] = sum_d q_cmp[bh, m, d] * k_cmp[bh, n, d]   (fp32 accumulate,
 // one rounding to the storage type, no softmax scale).
 //
-// Top-k: each wavefront owns one score row.  Every score is widened to a
-// unique, totally ordered integer key (order-preserving image of the score in
-// the high bits, inverted column index in the low bits) so that "larger key"
-// means "larger score, or equal score and lower index".  The k-th largest key
+// Top-k: each wavefront owns one score row and holds it in registers as
+// order-preserving integer images of the scores.  The k-th largest score VALUE
 // is found by a bitwise binary search whose counting step is a wavefront
-// ballot + popcount; the winners are compacted into LDS and ranked so that the
-// output is in descending score order with ties towards the lowest index.
+// ballot + popcount; every column above it wins, and of the columns equal to it
+// the lowest-indexed ones that are still needed ("larger score, or equal score
+// and lower index").  Walking the registers in column order emits the list in
+// ascending block order directly; the descending-score list (a total order
+// through keys that append the inverted column index to the score image) is
+// ranked in LDS only when it is asked for.  The CDF rule counts with the same
+// value search over masked sums of softmax weights.
 #include "bsa_common.h"
 
 namespace bsa {
