@@ -13,25 +13,14 @@
 // through keys that append the inverted column index to the score image) is
 // ranked in LDS only when it is asked for.  The CDF rule counts with the same
 // value search over masked sums of softmax weights.
-#include "bsa_common.h"
+#include "bsa_mfma.h"
 
 namespace bsa {
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-
-__device__ inline f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
-__device__ inline f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-}
-
-template <typename T> struct Vec8;
-template <> struct Vec8<__bf16> { typedef bf16x8 type; };
-template <> struct Vec8<_Float16> { typedef f16x8 type; };
+using mfma::f32x16;
+using mfma::mfma32;
+using mfma::Vec8;
 
 // ---------------------------------------------------------------- score GEMM
 // Workgroup = 4 wavefronts = 128 score rows x up to kScoreCols columns; each wavefront keeps its 32
