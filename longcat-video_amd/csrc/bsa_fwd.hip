@@ -133,7 +133,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     const int64_t q_bh = (int64_t)(bh / Hn) * L.q_st[0] + (int64_t)(bh % Hn) * L.q_st[1];
     const int64_t o_bh = (int64_t)(bh / Hn) * L.o_st[0] + (int64_t)(bh % Hn) * L.o_st[1];
     const int32_t* list = idx + ((int64_t)bh * nbq + qblock) * idx_stride;
-    const int ntiles = min(max(lens[(int64_t)bh * nbq + qblock], 0), idx_stride) * nsub;   // never past the list row
+    const int len_raw = lens[(int64_t)bh * nbq + qblock];
     const char* kbase = reinterpret_cast<const char*>(k + (int64_t)(bh / Hn) * L.k_st[0] + (int64_t)(bh % Hn) * L.k_st[1]);
     const char* vbase = reinterpret_cast<const char*>(v + (int64_t)(bh / Hn) * L.v_st[0] + (int64_t)(bh % Hn) * L.v_st[1]);
 
@@ -180,8 +180,13 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
         for (int i = 0; i < 16; ++i) oacc[t][i] = 0.f;
     float m_i = -INFINITY, l_i = 0.f;
 
+    // A list row of at most 256 tiles is staged whole before the length of the list has arrived (one
+    // dependent load less before the first tile can be fetched): what lies behind the length is
+    // clamped like any entry and never walked.  Longer rows wait for the length and go in chunks.
+    const bool early = idx_stride * nsub <= 256;
+    int ntiles = early ? idx_stride * nsub : min(max(len_raw, 0), idx_stride) * nsub;   // never past the list row
     for (int chunk0 = 0; chunk0 < ntiles; chunk0 += kListCap) {
-    const int nloc = min(ntiles - chunk0, kListCap);
+    int nloc = min(ntiles - chunk0, kListCap);
     __syncthreads();                          // previous chunk / previous item fully consumed
     for (int j = tid; j < nloc; j += 256) {
         const int it = chunk0 + j;
@@ -191,6 +196,10 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
         const uint32_t entry = L.k_tiles != nullptr ? L.k_tiles[tile] : (uint32_t)tile * kTile;
         tile_row_sm[j] = (int)entry;
         tile_mask_sm[j] = tile_valid ? tile_valid[tile] : ~0ull;
+    }
+    if (early) {
+        ntiles = nloc = min(max(len_raw, 0), idx_stride) * nsub;
+        if (ntiles == 0) break;
     }
     // consume the Q loads here: otherwise their vmcnt waits land inside the tile loop,
     // where they would also wait for the LDS loads of the next tile
