@@ -264,7 +264,7 @@ def main():
     nbk = k_cmp.shape[2]
     ms_permute = time_events(torch, lambda: I._permute(k, latent, CHUNK, want_pooled=True), ksteps, kwarm)
     ms_unpermute = time_events(torch, lambda: I.rearrange_3d_block_to_THW(qp, *[-(-n // c) for n, c in zip(latent, CHUNK)], *CHUNK, D, latent_shape=latent), ksteps, kwarm)
-    ms_select = time_events(torch, lambda: I._score_topk(q_cmp, k_cmp, k_sel), ksteps, kwarm)
+    ms_select = time_events(torch, lambda: I._score_topk(q_cmp, k_cmp, k_sel, order="block"), ksteps, kwarm)   # as the operator runs it
 
     S = q.shape[2]
     Sp = qp.shape[2]
