@@ -7,7 +7,7 @@ same constructor arguments, same parameter names (``qkv``, ``q_norm.weight``,
 C-ABI of the engine:
 
     qkv = Linear(x)                      bsa_linear_bf16   (attention.py:111)
-    q, k = RMSNorm(q), RMSNorm(k); RoPE  bsa_qk_norm_rope  (attention.py:116, :121)
+    q, k = RMSNorm(q), RMSNorm(k); RoPE  bsa_norm_rope     (attention.py:116, :121)
     block-sparse attention               bsa_fwd_3d        (attention.py:58-67, :124-137)
     x = Linear(o)                        bsa_linear_bf16   (attention.py:139-142)
 
