@@ -382,7 +382,8 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
     // ---- epilogue: merge the two key halves, normalise, store coalesced ----
     const int kc = tid & 15, kr = tid >> 4;
     float* xch = reinterpret_cast<float*>(&smem[0][0][0]);                  // [qh][66][64] fp32
-    T* ost = reinterpret_cast<T*>(reinterpret_cast<char*>(xch) + 2 * 66 * 64 * 4);   // [64][128]
+    constexpr int kOutPitch = kD + 8;
+    T* ost = reinterpret_cast<T*>(reinterpret_cast<char*>(xch) + 2 * 66 * 64 * 4);   // [64][kOutPitch]
     if (kh == 1) {
         float* dst = xch + qh * 66 * 64 + lane;
 #pragma unroll
@@ -405,7 +406,9 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
         const float a1 = __builtin_amdgcn_exp2f(m1 - m_safe);
         const float l = a0 * l0 + a1 * l1;
         const float inv = l > 0.f ? 1.0f / l : 0.f;
-        T* orow = ost + (32 * qh + lr) * kD;
+        // rows of the staging tile are 272 B apart: at 256 B the 32 rows that one store instruction touches
+        // would all lie in the same banks
+        T* orow = ost + (32 * qh + lr) * kOutPitch;
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -433,7 +436,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(
             if (L.q_rows != nullptr) row = L.q_rows[row];
             if (row >= 0)
                 *reinterpret_cast<uint4*>(o + o_bh + row * L.o_st[2] + kc * 8) =
-                    *reinterpret_cast<const uint4*>(ost + r * kD + kc * 8);
+                    *reinterpret_cast<const uint4*>(ost + r * kOutPitch + kc * 8);
         }
     }
     }   // work items
