@@ -171,7 +171,9 @@ int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, con
  *   bsa_score_cdf instead (bsa:268-277 dispatch), at most min(nbk, 1024) blocks per
  *   row, and idx_out has that many columns.  workspace: bsa_workspace_bytes() bytes, 256-byte
  *   aligned.  idx_out/lens_out/score_out are optional copies for inspection
- *   (shapes as in bsa_score_topk).
+ *   (shapes as in bsa_score_topk).  With cdf_threshold the lists differ in length: the work is then also
+ *   enqueued as one launch whose workgroups draw the query tiles longest list first, and a kernel decides
+ *   from the lengths, on the device, whether that or the usual rounds of equal tiles run (bf16 / fp16).
  * For bf16 / fp16 no permuted copy of q, k, v or o is made: one pass over q and k
  * produces the pooled means (and the tables of bsa_thw_prepare), and the attention
  * kernel reads and writes THW order directly; k and v must then share one token

@@ -227,7 +227,7 @@ struct Plan {
     int sel_width;        // columns of the index lists: k_sel, or the cap of the CDF rule
     bool cdf;
     bool direct_qo, direct_kv;
-    size_t off_qp, off_kp, off_vp, off_op, off_qc, off_kc, off_score, off_idx, off_idx_sorted, off_lens, off_valid, off_qrows, off_ktiles, total;
+    size_t off_qp, off_kp, off_vp, off_op, off_qc, off_kc, off_score, off_idx, off_idx_sorted, off_lens, off_valid, off_qrows, off_ktiles, off_order, off_queue, total;
 };
 inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
@@ -275,6 +275,9 @@ int make_plan(const bsa_3d_params* p, Plan* pl) {
     pl->off_valid = take((size_t)(pl->Skp / 64) * sizeof(uint64_t));
     pl->off_qrows = take(pl->direct_qo ? (size_t)pl->Sqp * sizeof(int32_t) : 0);
     pl->off_ktiles = take(pl->direct_kv ? (size_t)(pl->Skp / 64) * sizeof(uint32_t) : 0);
+    // lists of unequal length (the CDF rule): work items by descending length, and the counter they are drawn with
+    pl->off_order = take(pl->cdf && pl->direct_qo ? bh * (size_t)(pl->Sqp / 64) * sizeof(int32_t) : 0);
+    pl->off_queue = take(pl->cdf && pl->direct_qo ? 2 * sizeof(uint32_t) : 0);    // the counter and the choice of schedule
     pl->total = off;
     return BSA_OK;
 }
@@ -289,8 +292,8 @@ size_t bsa_workspace_bytes(const bsa_3d_params* p) {
 namespace {
 struct Ws {
     void *qp, *kp, *vp, *op, *qc, *kc, *score;
-    int32_t *idx, *idx_sorted, *lens, *qrows;
-    uint32_t* ktiles;
+    int32_t *idx, *idx_sorted, *lens, *qrows, *order;
+    uint32_t *ktiles, *queue;
     uint64_t* valid;
 };
 int carve(const Plan& pl, void* workspace, size_t workspace_bytes, const char* who, Ws* w) {
@@ -307,6 +310,8 @@ int carve(const Plan& pl, void* workspace, size_t workspace_bytes, const char* w
     w->valid = reinterpret_cast<uint64_t*>(ws + pl.off_valid);
     w->qrows = pl.direct_qo ? reinterpret_cast<int32_t*>(ws + pl.off_qrows) : nullptr;
     w->ktiles = pl.direct_kv ? reinterpret_cast<uint32_t*>(ws + pl.off_ktiles) : nullptr;
+    w->order = pl.cdf && pl.direct_qo ? reinterpret_cast<int32_t*>(ws + pl.off_order) : nullptr;
+    w->queue = pl.cdf && pl.direct_qo ? reinterpret_cast<uint32_t*>(ws + pl.off_queue) : nullptr;
     return BSA_OK;
 }
 bool kv_padded(const bsa_3d_params* p) { return (p->Tk % p->tk) || (p->Hk % p->hk) || (p->Wk % p->wk); }
@@ -345,7 +350,7 @@ hipError_t prepare_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, cons
 hipError_t attention_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, const void* q, const int64_t q_strides[3],
                          const void* k, const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
                          const int64_t o_strides[3], const int32_t* idx, const int32_t* lens, int idx_stride, float* lse,
-                         hipStream_t st) {
+                         hipStream_t st, bool by_length = false) {
     FwdLayout L;
     L.q_rows = w.qrows;
     L.k_tiles = w.ktiles;
@@ -363,7 +368,8 @@ hipError_t attention_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, co
     }
     return launch_fwd(q, pl.direct_kv ? k : w.kp, pl.direct_kv ? v : w.vp, idx, lens, kv_padded(p) ? w.valid : nullptr, o, lse,
                       p->B, p->Hn, pl.Sqp, pl.Skp, pl.gq.chunk(), pl.gk.chunk(), idx_stride, p->sm_scale, p->dtype, st, &L,
-                      (int64_t)p->Tq * p->Hq * p->Wq, (int64_t)edge_count(pl.gk) * pl.gk.chunk() * p->D * pl.es);
+                      (int64_t)p->Tq * p->Hq * p->Wq, (int64_t)edge_count(pl.gk) * pl.gk.chunk() * p->D * pl.es,
+                      by_length ? w.order : nullptr, by_length ? w.queue : nullptr);
 }
 
 int check_tensor(const void* x, const int64_t strides[3], const bsa_3d_params* p, const char* name) {
@@ -447,8 +453,11 @@ int bsa_fwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3]
         BSA_HIP(launch_topk(w.score, idx_out ? w.idx : nullptr, w.idx_sorted, w.lens, sel_rows, pl.nbk, p->k_sel, p->dtype, st), "top-k");
     }
     if (pl.direct_qo) {
+        // lists of unequal length: one launch whose workgroups draw the items, longest lists first
+        if (pl.cdf)
+            BSA_HIP(launch_order_by_length(w.lens, w.order, p->B * p->Hn, pl.nbq, pl.gq.chunk() / 64, pl.sel_width, st), "order by length");
         BSA_HIP(attention_thw(pl, p, w, q, q_strides, k, k_strides, v, v_strides, o, o_strides, w.idx_sorted, w.lens, pl.sel_width,
-                              nullptr, st), "attention");
+                              nullptr, st, pl.cdf), "attention");
     } else {
         BSA_HIP(launch_fwd(w.qp, w.kp, w.vp, w.idx_sorted, w.lens, padded_k ? w.valid : nullptr, w.op, nullptr, p->B, p->Hn, pl.Sqp, pl.Skp,
                            pl.gq.chunk(), pl.gk.chunk(), pl.sel_width, p->sm_scale, p->dtype, st), "attention");

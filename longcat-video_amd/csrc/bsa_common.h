@@ -122,6 +122,13 @@ hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t
                       const int32_t* lens, const uint64_t* tile_valid, void* o, float* lse,
                       int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride,
                       float sm_scale, int dtype, hipStream_t st, const FwdLayout* layout = nullptr,
-                      int64_t layout_lse_rows = 0, int64_t layout_edge_bytes = 0);
+                      int64_t layout_lse_rows = 0, int64_t layout_edge_bytes = 0, const int32_t* order = nullptr,
+                      uint32_t* queue = nullptr);
+// order: for every (batch, head) its 64-row query tiles by descending list length (lens is per query
+// block of tiles_per_block tiles, clamped to [0, max_len]); with `order` and a two-word `queue`
+// launch_fwd enqueues the 16-bit kernel both as rounds and as one launch whose workgroups draw items
+// from a counter, and a kernel that compares the list lengths decides on the device which of them runs
+hipError_t launch_order_by_length(const int32_t* lens, int32_t* order, int BH, int nbq, int tiles_per_block, int max_len,
+                                  hipStream_t st);
 
 }  // namespace bsa

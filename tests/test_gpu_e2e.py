@@ -301,3 +301,51 @@ def test_random_shapes_against_the_oracle(seed):
         check_against_oracle(q[b:b + 1], k[b:b + 1], v[b:b + 1], c["lq"], c["lk"], c["sparsity"], o[b:b + 1], idx[b:b + 1],
                              lens[b:b + 1], score[b:b + 1], q_blocks=range(nbq), chunk=c["chunk"])
     assert torch.isfinite(o.float()).all(), c
+
+
+@pytest.mark.parametrize("spread", ["wide", "narrow"])
+def test_cdf_lists_of_unequal_length_schedule(spread):
+    """With the CDF rule the operator enqueues two schedules of the attention kernel (rounds of equal work items,
+    and one launch whose workgroups draw the items longest list first) and picks one on the device from the list
+    lengths.  Whatever it picks, the output must equal, bit for bit, what the kernel gives in plain rounds on the
+    same lists (ThwAttention), here with more work items (640) than one round holds: 'wide' has lists from a few
+    blocks to most of them, 'narrow' lists of nearly equal length."""
+    latent, heads = (8, 32, 32), 5
+    S = int(np.prod(latent))
+    g = torch.Generator().manual_seed(52)
+    q = torch.randn(1, heads, S, 128, generator=g)
+    k = torch.randn(1, heads, S, 128, generator=g)
+    v = torch.randn(1, heads, S, 128, generator=g).bfloat16()
+    if spread == "wide":
+        # chunks whose queries all point the same way (peaked pooled scores, short lists) next to chunks of
+        # independent queries (flat scores, long lists)
+        pos = torch.arange(S)
+        chunk_id = ((pos // (32 * 32)) // 4) * 64 + (((pos // 32) % 32) // 4) * 8 + (pos % 32) // 4
+        peaked = (chunk_id % 10 != 0)      # nine short lists for every long one: the draw-from-a-counter schedule wins
+        common = torch.randn(1, heads, S // 64, 128, generator=g).repeat_interleave(64, dim=2)   # one direction per 64 tokens
+        chunk_dir = torch.zeros_like(q)
+        order = torch.argsort(chunk_id, stable=True)                 # tokens grouped by chunk: 64 each
+        chunk_dir[:, :, order] = common
+        q[:, :, peaked] = 3 * chunk_dir[:, :, peaked] + 0.1 * q[:, :, peaked]
+        k[:, :, peaked] = 3 * chunk_dir[:, :, peaked] + 0.1 * k[:, :, peaked]
+    q, k = q.bfloat16(), k.bfloat16()
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    o, idx, lens, score = I()._bsa_3d(qg, kg, vg, latent, latent, None, (4, 4, 4), (4, 4, 4), True, cdf_threshold=0.5)
+    lens_c = lens.cpu()
+    if spread == "wide":
+        assert int(lens_c.max()) > 4 * max(int(lens_c.min()), 1)
+    else:
+        assert int(lens_c.max()) <= 2 * max(int(lens_c.min()), 1)
+    big = idx.shape[-1] + 1
+    asc = torch.where(idx < 0, torch.full_like(idx, big), idx).sort(dim=-1).values
+    asc = torch.where(asc == big, torch.zeros_like(asc), asc)
+    rounds = I().ThwAttention(kg, vg, latent, latent, (4, 4, 4), (4, 4, 4))(qg, asc, lens)
+    assert torch.equal(o, rounds)
+    # and both agree with the oracle on a few query blocks of every head
+    qp, kp, vp = (O.rearrange_thw_to_3d_block(t, latent, (4, 4, 4)) for t in (q, k, v))
+    blocks = [0, 37, 127]
+    want_o, _ = O.gathered_attention(qp, kp, vp, asc.cpu().long(), lens_c, 64, 64, 1 / math.sqrt(128), q_blocks=blocks)
+    got_p = O.rearrange_thw_to_3d_block(o.cpu(), latent, (4, 4, 4))
+    for m in blocks:
+        d = (got_p[:, :, 64 * m:64 * m + 64].float() - want_o[:, :, 64 * m:64 * m + 64]).abs()
+        assert d.max() <= MAX_ABS and d.mean() <= MEAN_ABS
