@@ -239,14 +239,15 @@ def test_two_batches_on_a_ragged_grid(dtype):
     assert torch.equal(o0, o[1:])
 
 
-def test_operator_replays_from_a_hip_graph():
+@pytest.mark.parametrize("cdf", [None, 0.6])
+def test_operator_replays_from_a_hip_graph(cdf):
     """The operator makes no allocation, host wait or memset of its own, so a captured stream replays it.  The
     graph is replayed three times with eager work and synchronisations in between and new input values each
     time; every replay must equal the eager result on the same values bit for bit."""
     latent = (5, 9, 13)                                   # ragged in every axis: edge copies, masks, tables
     q, k, v = (t.cuda() for t in seeded_qkv(40, 1, 2, 5 * 9 * 13, 5 * 9 * 13, 128, torch.bfloat16))
     sq, sk, sv = q.clone(), k.clone(), v.clone()          # static inputs of the graph
-    run = lambda: I().flash_attn_bsa_3d(sq, sk, sv, latent, latent, sparsity=0.5, **CH)
+    run = lambda: I().flash_attn_bsa_3d(sq, sk, sv, latent, latent, sparsity=0.5, cdf_threshold=cdf, **CH)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
