@@ -38,8 +38,8 @@
 // rescale of the output accumulator drops out of almost every iteration.  The
 // result is the same softmax up to fp32 rounding.
 //
-// Scheduling.  The work items of one (batch, head) are launched in rounds of as
-// many workgroups as the device runs at once (2 per CU).  The workgroups of a
+// Scheduling.  The work items are launched in rounds of as many workgroups as
+// the device runs at once (2 per CU), head after head.  The workgroups of a
 // round start together and, because every item of a top-k selection has the
 // same number of tiles, stay roughly in step.  With KV lists in ascending block
 // order the workgroups of an XCD then sweep the K/V of a head in the same
@@ -49,7 +49,11 @@
 // whole grid loses this: workgroups then start whenever a slot frees up.
 // Within a round every XCD takes a contiguous run of the query blocks (workgroup b
 // runs on XCD b % 8): spatial neighbours select largely the same KV blocks on real
-// inputs, and only the workgroups of one XCD share an L2.
+// inputs, and only the workgroups of one XCD share an L2.  The second, MFMA-only
+// half of a step runs at raised wave priority, which puts the two wavefronts that
+// share a SIMD (one of each resident workgroup) into alternating phases.
+// Lists of unequal length (the CDF rule) have a second schedule: one launch
+// whose workgroups draw the items, longest list first, from a counter.
 #include "bsa_mfma.h"
 
 namespace bsa {
