@@ -570,9 +570,10 @@ __global__ __launch_bounds__(256) void order_by_length_kernel(const int32_t* __r
 
 // Rounds or queue?  A round lasts as long as its longest list, the queue keeps every workgroup busy but
 // gives up the lock-step walk (measured on equal lists: 1.55 x the time).  *choice = 1 (queue) when
-// 1.55 * (sum of lengths / round) + longest < sum over rounds of the longest list of each round.
+// 1.55 * (sum of lengths / resident workgroups) + longest < sum over rounds of the longest list of each round.
 __global__ __launch_bounds__(256) void choose_schedule_kernel(const int32_t* __restrict__ lens, int nbq, int tiles_per_block,
-                                                              int total, int round, int max_len, uint32_t* __restrict__ choice) {
+                                                              int total, int round, int resident, int max_len,
+                                                              uint32_t* __restrict__ choice) {
     constexpr int kMaxRounds = 8192;
     __shared__ int round_max[kMaxRounds];
     __shared__ unsigned long long sum_sm;
@@ -597,8 +598,10 @@ __global__ __launch_bounds__(256) void choose_schedule_kernel(const int32_t* __r
     __syncthreads();
     if (threadIdx.x == 0) {
         unsigned long long rounds_cost = 0ull;
-        for (int r = 0; r < n_rounds; ++r) rounds_cost += (unsigned long long)round_max[r];
-        const double queue_cost = 1.55 * (double)sum_sm / (double)round + (double)longest_sm;
+        for (int r = 0; r < n_rounds; ++r) rounds_cost += (unsigned long long)round_max[r] * (unsigned long long)(round / resident);
+        // rounds of `round` items run as round / resident waves of workgroups, each as long as its longest list:
+        // an upper bound for the rounds, which only makes the comparison cautious
+        const double queue_cost = 1.55 * (double)sum_sm / (double)resident + (double)longest_sm;
         *choice = queue_cost < (double)rounds_cost ? 1u : 0u;
     }
 }
@@ -662,17 +665,20 @@ hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t
     // an XCD takes a contiguous run of a round's items, so even in a round that holds two heads
     // almost every XCD still works on one.
     const int per_head = (int)(Sq / kTile);
-    const int round = resident_workgroups();
+    // short lists (at most 64 tiles): three items per resident workgroup and launch, so that the gap between
+    // launches and the wait for a round's slowest workgroup weigh less (480p: -4 %; nothing at 90 tiles)
+    const int resident = resident_workgroups();
+    const int round = resident * (idx_stride * (bs_k / kTile) <= 64 ? 3 : 1);
     const uint32_t* gate = nullptr;
     if (queue != nullptr) {
         // Lists of possibly unequal length.  queue[0] is the counter the items are drawn with, queue[1] the
         // choice between the two schedules, made on the device from the lengths; both are enqueued.
         const int total = B * Hn * per_head;
         hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, st, queue, 1);
-        hipLaunchKernelGGL(choose_schedule_kernel, dim3(1), dim3(256), 0, st, lens, (int)(Sq / bs_q), bs_q / kTile, total, round,
+        hipLaunchKernelGGL(choose_schedule_kernel, dim3(1), dim3(256), 0, st, lens, (int)(Sq / bs_q), bs_q / kTile, total, round, resident,
                            idx_stride, queue + 1);
         gate = queue + 1;
-        const dim3 grid((unsigned)(total < round ? total : round));
+        const dim3 grid((unsigned)(total < resident ? total : resident));
         if (dtype == BSA_BF16)
             hipLaunchKernelGGL((fwd_mfma_kernel<__bf16>), grid, block, 0, st, (const __bf16*)q,
                                (const __bf16*)k, (const __bf16*)v, idx, lens, tile_valid, (__bf16*)o,
