@@ -211,7 +211,9 @@ int bsa_fwd_3d(const bsa_3d_params* p,
  *   64-slot tiles made of whole (h, w) planes).  Call again whenever k or v change.
  * bsa_fwd_thw: the attention kernel alone.  idx / lens / idx_stride / lse as in bsa_fwd, block
  *   indices counted in the padded chunk grids; lse is [B, Hn, Tq*Hq*Wq] in THW order.
- *   p->k_sel is not used.  k and v must share one token stride.
+ *   p->k_sel is not used.  k and v must share one token stride.  p->cdf_threshold > 0 (any positive
+ *   value, in both calls) declares that the lists may differ in length: the kernel is then enqueued in
+ *   both schedules described at bsa_fwd_3d and the choice is made on the device.
  */
 int bsa_thw_prepare(const bsa_3d_params* p, const void* k, const int64_t k_strides[3],
                     const void* v, const int64_t v_strides[3],

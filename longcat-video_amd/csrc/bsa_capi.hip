@@ -410,8 +410,13 @@ int bsa_fwd_thw(const bsa_3d_params* p, const void* q, const int64_t q_strides[3
     BSA_TRY(check_tensor(o, o_strides, p, "o"));
     BSA_TRY(check_kv_views(pl, k_strides, v_strides, "fwd_thw"));
     if (!lens || idx_stride < 0 || (!idx && idx_stride > 0)) return set_error(BSA_ERR_BAD_ARG, "fwd_thw: selection is missing");
-    const hipError_t e = attention_thw(pl, p, w, q, q_strides, k, k_strides, v, v_strides, o, o_strides, idx, lens, idx_stride,
-                                       lse, (hipStream_t)stream);
+    hipError_t e = hipSuccess;
+    // p->cdf_threshold > 0 declares lists of unequal length: work items by length, both schedules enqueued
+    if (pl.cdf && idx_stride > 0)
+        e = launch_order_by_length(lens, w.order, p->B * p->Hn, pl.nbq, pl.gq.chunk() / 64, idx_stride, (hipStream_t)stream);
+    if (e == hipSuccess)
+        e = attention_thw(pl, p, w, q, q_strides, k, k_strides, v, v_strides, o, o_strides, idx, lens, idx_stride, lse,
+                          (hipStream_t)stream, pl.cdf && idx_stride > 0);
     return e == hipSuccess ? BSA_OK : hip_fail(e, "fwd_thw");
 }
 

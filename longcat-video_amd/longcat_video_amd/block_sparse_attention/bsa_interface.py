@@ -371,7 +371,8 @@ class ThwAttention:
     steps: the constructor prepares what depends on k and v (bsa_thw_prepare), every call runs the
     attention kernel alone (bsa_fwd_thw).  bf16 / fp16."""
 
-    def __init__(self, k, v, latent_shape_q, latent_shape_k, chunk_3d_shape_q, chunk_3d_shape_k, sm_scale=None):
+    def __init__(self, k, v, latent_shape_q, latent_shape_k, chunk_3d_shape_q, chunk_3d_shape_k, sm_scale=None,
+                 unequal_lengths=False):
         _need_gpu(k, v)
         B, H, Sk, D = k.shape
         self.gq = tuple(int(x) for x in latent_shape_q) + tuple(int(x) for x in chunk_3d_shape_q)
@@ -386,7 +387,9 @@ class ThwAttention:
         self.k, self.v = k, v
         self.nbq = lib.bsa_padded_tokens(Tq, Hq, Wq, tq, hq, wq) // (tq * hq * wq)
         scale = 1.0 / D ** 0.5 if sm_scale is None else float(sm_scale)
-        self.prm = _capi.Bsa3dParams(B, H, D, _code(k), Tq, Hq, Wq, Tk, Hk, Wk, tq, hq, wq, tk, hk, wk, 0, scale)
+        # unequal_lengths: the lists of later calls may differ in length (enqueue both schedules, choose on the device)
+        self.prm = _capi.Bsa3dParams(B, H, D, _code(k), Tq, Hq, Wq, Tk, Hk, Wk, tq, hq, wq, tk, hk, wk, 0, scale,
+                                     1.0 if unequal_lengths else 0.0)
         self.need = lib.bsa_workspace_bytes(C.byref(self.prm))
         self.ws = torch.empty(max(self.need, 1), dtype=torch.uint8, device=k.device)
         self.ks, self.vs = _capi.strides3(k.stride()[:3]), _capi.strides3(v.stride()[:3])

@@ -342,6 +342,9 @@ def test_cdf_lists_of_unequal_length_schedule(spread):
     asc = torch.where(asc == big, torch.zeros_like(asc), asc)
     rounds = I().ThwAttention(kg, vg, latent, latent, (4, 4, 4), (4, 4, 4))(qg, asc, lens)
     assert torch.equal(o, rounds)
+    # the same choice of schedule for a caller's own lists
+    either = I().ThwAttention(kg, vg, latent, latent, (4, 4, 4), (4, 4, 4), unequal_lengths=True)(qg, asc, lens)
+    assert torch.equal(either, rounds)
     # and both agree with the oracle on a few query blocks of every head
     qp, kp, vp = (O.rearrange_thw_to_3d_block(t, latent, (4, 4, 4)) for t in (q, k, v))
     blocks = [0, 37, 127]
