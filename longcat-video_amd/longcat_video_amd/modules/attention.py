@@ -64,12 +64,11 @@ _GEMM_WORKSPACES = {}
 
 
 def _gemm_workspace(device) -> torch.Tensor:
-    """128 MiB per device and stream, kept: calls on one stream run one after the other.  (The engine asks for
-    64 MiB at least; with 128 the 720p projections run 1.3 % faster, more brings nothing.)"""
+    """64 MiB per device and stream, kept: calls on one stream run one after the other."""
     key = (str(device), torch.cuda.current_stream(device).cuda_stream)
     ws = _GEMM_WORKSPACES.get(key)
     if ws is None:
-        ws = _GEMM_WORKSPACES[key] = torch.empty(128 << 20, dtype=torch.uint8, device=device)
+        ws = _GEMM_WORKSPACES[key] = torch.empty(64 << 20, dtype=torch.uint8, device=device)
     return ws
 
 
