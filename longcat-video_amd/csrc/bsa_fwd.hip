@@ -26,11 +26,13 @@
 // 16-byte chunk (l%16) ^ f(row) of its row.  Two stages of (K 16 KB + V 16 KB)
 // per workgroup, two workgroups per CU, one barrier per tile.
 //
-// Software pipeline.  MFMA and plain VALU instructions of one SIMD do not
-// overlap on this hardware (measured), but transcendental instructions do, and
-// a wavefront that waits on an MFMA result leaves the SIMD to its neighbour.
-// In iteration i the 8 MFMAs of S(i+1) are therefore interleaved with the
-// exp2 of tile i, and the 8 MFMAs of O += P(i) V(i) with the row sum.
+// Software pipeline.  An MFMA keeps the matrix pipe busy for 32 clocks, during
+// which the SIMD goes on issuing VALU instructions, of the same wavefront or of
+// its neighbour (measured: an MFMA followed by 7 independent VALU instructions
+// takes about 40 clocks, not 60); a wavefront that waits on an MFMA result leaves
+// the SIMD to its neighbour.  In iteration i the 8 MFMAs of S(i+1) are therefore
+// interleaved with the exp2 of tile i, and the 8 MFMAs of O += P(i) V(i) with
+// the row maximum of S(i+1).
 //
 // Softmax.  The running maximum is only raised when a row's new maximum
 // exceeds it by more than 2^8 (lazy rescale): probabilities are then at most
