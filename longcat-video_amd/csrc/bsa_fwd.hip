@@ -667,10 +667,12 @@ hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t
     // an XCD takes a contiguous run of a round's items, so even in a round that holds two heads
     // almost every XCD still works on one.
     const int per_head = (int)(Sq / kTile);
-    // short lists (at most 64 tiles): three items per resident workgroup and launch, so that the gap between
-    // launches and the wait for a round's slowest workgroup weigh less (480p: -4 %; nothing at 90 tiles)
+    // short lists: three (at most 64 tiles) or two (at most 128) items per resident workgroup and launch, so
+    // that the gap between launches and the wait for a round's slowest workgroup weigh less (39 tiles: -4 %,
+    // 90 tiles: -1.5 %, nothing at 156 tiles)
     const int resident = resident_workgroups();
-    const int round = resident * (idx_stride * (bs_k / kTile) <= 64 ? 3 : 1);
+    const int list_tiles = idx_stride * (bs_k / kTile);
+    const int round = resident * (list_tiles <= 64 ? 3 : list_tiles <= 128 ? 2 : 1);
     const uint32_t* gate = nullptr;
     if (queue != nullptr) {
         // Lists of possibly unequal length.  queue[0] is the counter the items are drawn with, queue[1] the
