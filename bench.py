@@ -35,9 +35,9 @@ WORKLOADS = {
     "c3": ((24, 45, 80), 0.9375, 2, True, "720p layer: 32 heads x 128, grid 24x45x80 (86400 tokens), density 1/16"),
 }
 # Bytes that leave L2 per layer in the attention kernel (all of its launches), from rocprofv3 --pmc
-# FETCH_SIZE (x2) and WRITE_SIZE (x1) as recorded in profiles/bsa_operator_c3_720p.md: 90 launches
-# x (620.7 MB + 7.9 MB).  Re-measure after kernel changes.
-ATTENTION_TRAFFIC_BYTES = {"c3": 90 * (620.7e6 + 7.9e6)}
+# FETCH_SIZE (x2) and WRITE_SIZE (x1) as recorded in profiles/bsa_operator_c3_720p.md: 45 launches
+# x (1286.6 MB + 15.7 MB).  Re-measure after kernel changes.
+ATTENTION_TRAFFIC_BYTES = {"c3": 45 * (1286.6e6 + 15.7e6)}
 CHUNK = (4, 4, 4)
 HEADS, D = 32, 128
 
