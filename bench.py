@@ -178,7 +178,8 @@ def run_c5(torch, args):
     attn.q_norm.weight.data.fill_(1.0)
     attn.k_norm.weight.data.fill_(1.0)
     w_pre = torch.ones(C, dtype=torch.bfloat16, device="cuda")
-    tuned = attn.tune(x, residual=True)              # one-time set-up: GEMM algorithm choice per projection shape
+    # one-time set-up: GEMM algorithm choice per projection shape (skipped under a profiler to keep its tables short)
+    tuned = ((0, 0.0, 0.0), (0, 0.0, 0.0)) if args.no_gemm_tuning else attn.tune(x, residual=True)
     for _ in range(args.warmup):
         M.attention_block_forward(x, w_pre, attn, latent)
     torch.cuda.synchronize()
@@ -213,6 +214,7 @@ def main():
                          "for the cond/noise split and for the attention module")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the CPU baseline's attention sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gemm-tuning", action="store_true", help="c5: leave the GEMM algorithm choice to hipBLASLt's first proposal")
     ap.add_argument("--data", default="random", choices=["random", "coherent"],
                     help="random (the benchmark's definition) or spatially coherent q/k (c2, c3 only; no CPU baseline)")
     args = ap.parse_args()
