@@ -36,6 +36,10 @@ constexpr int kListCap = 1024;   // tiles whose addresses are staged in LDS at a
 // m0 + 16*lane; the global address is sbase + voff.  Issued from inline assembly
 // so that the compiler does not order later LDS reads of other stages behind it;
 // completion is awaited explicitly (s_waitcnt vmcnt) before the stage is read.
+// m0 is not on the clobber list: it is a reserved register for this target (the compiler rejects it there
+// as undefined behaviour) and every compiler-generated use of m0 on gfx9 (movrel, readlane selectors, LDS DMA
+// builtins) writes m0 itself immediately before the instruction that reads it, so nothing is assumed to
+// survive this statement.  The kernels that use this helper index no register array dynamically.
 __device__ inline void load_to_lds_16(const void* sbase, uint32_t voff, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
