@@ -199,6 +199,30 @@ int bsa_fwd_3d(const bsa_3d_params* p,
                int32_t* idx_out, int32_t* lens_out, void* score_out, void* stream);
 
 /*
+ * bsa_fwd_3d without a workspace argument and without any allocation.  It has no counterpart in the
+ * reference; it is for callers that cannot allocate device memory around the call: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  What bsa_fwd_3d carves from its workspace
+ * lives in a buffer of BSA_STATIC_SCRATCH_BYTES that is part of the library's code object, so every GPU the
+ * library is used on holds that much memory from the first call on it until the process ends.
+ *   - Arguments and results are those of bsa_fwd_3d (same kernels, same bits).
+ *   - A problem whose bsa_workspace_bytes() exceeds BSA_STATIC_SCRATCH_BYTES is rejected with
+ *     BSA_ERR_WORKSPACE before anything is launched (64 MiB covers, in bf16 with 4x4x4 chunks, the 720p
+ *     grid at up to 6 heads or the 480p grid at up to 17 heads: one GPU's share of a head-sharded layer).
+ *   - The call itself makes no hipMalloc / hipFree and calls no allocating library routine.  The first call
+ *     on a device looks up the buffer's address (hipGetSymbolAddress); make that call outside graph capture.
+ *   - All calls on one GPU share the one buffer, which keeps the previous call's contents; nothing in it
+ *     needs to start at zero.  Calls that overlap in time on one GPU (different streams, different threads)
+ *     race on it and give wrong results: serialise them, or use bsa_fwd_3d with one workspace per stream.
+ */
+#define BSA_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
+int bsa_fwd_3d_static(const bsa_3d_params* p,
+                      const void* q, const int64_t q_strides[3],
+                      const void* k, const int64_t k_strides[3],
+                      const void* v, const int64_t v_strides[3],
+                      void* o, const int64_t o_strides[3],
+                      int32_t* idx_out, int32_t* lens_out, void* score_out, void* stream);
+
+/*
  * R1 + R5 + R6 + R7 with a caller-supplied selection, bf16 / fp16: attention over THW-order
  * tensors without permuted copies.  Replaces the sequence rearrange_THW_to_3d_block x3 (bsa:650-652),
  * attn_fwd_bsa_varlen_triton (bsa:290-341), rearrange_3d_block_to_THW (bsa:659) for callers that

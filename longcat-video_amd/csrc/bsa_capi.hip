@@ -2,6 +2,7 @@
 // sequencing.  Nothing here allocates device memory or waits for the GPU.
 #include "bsa_common.h"
 
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -420,13 +421,14 @@ int bsa_fwd_thw(const bsa_3d_params* p, const void* q, const int64_t q_strides[3
     return e == hipSuccess ? BSA_OK : hip_fail(e, "fwd_thw");
 }
 
-int bsa_fwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3], const void* k,
-               const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
-               const int64_t o_strides[3], void* workspace, size_t workspace_bytes, int32_t* idx_out,
-               int32_t* lens_out, void* score_out, void* stream) {
-    Plan pl;
+}  // extern "C"
+
+namespace {
+int fwd_3d_impl(const Plan& pl, const bsa_3d_params* p, const void* q, const int64_t q_strides[3], const void* k,
+                const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
+                const int64_t o_strides[3], void* workspace, size_t workspace_bytes, int32_t* idx_out,
+                int32_t* lens_out, void* score_out, void* stream) {
     Ws w;
-    BSA_TRY(make_plan(p, &pl));
     if (!q || !k || !v || !o || !workspace) return set_error(BSA_ERR_BAD_ARG, "fwd_3d: null pointer");
     BSA_TRY(carve(pl, workspace, workspace_bytes, "fwd_3d", &w));
     BSA_TRY(check_tensor(q, q_strides, p, "q"));
@@ -475,6 +477,60 @@ int bsa_fwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3]
     if (score_out) BSA_HIP(hipMemcpyAsync(score_out, w.score, bh * pl.nbq * (size_t)pl.nbk * pl.es, hipMemcpyDeviceToDevice, st), "copy score");
 #undef BSA_HIP
     return BSA_OK;
+}
+
+// The scratch memory of bsa_fwd_3d_static: what bsa_fwd_3d carves from its caller's workspace, held in the
+// code object instead.  Every GPU the library runs on holds its own copy at its own address until the
+// process ends.  In host code the name `scratch` is only a handle for hipGetSymbolAddress, never a device
+// address: the address is looked up once per device, with that device current, and kept.
+constexpr size_t kStaticScratchBytes = BSA_STATIC_SCRATCH_BYTES;
+__device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+int static_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "fwd_3d_static: hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return set_error(BSA_ERR_UNSUPPORTED, "fwd_3d_static: device %d beyond the %d supported", dev, kMaxDevices);
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) return hip_fail(e, "fwd_3d_static: hipGetSymbolAddress(scratch)");
+        // two threads racing here look up the same address for the same device
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return BSA_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int bsa_fwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3], const void* k,
+               const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
+               const int64_t o_strides[3], void* workspace, size_t workspace_bytes, int32_t* idx_out,
+               int32_t* lens_out, void* score_out, void* stream) {
+    Plan pl;
+    BSA_TRY(make_plan(p, &pl));
+    return fwd_3d_impl(pl, p, q, q_strides, k, k_strides, v, v_strides, o, o_strides, workspace, workspace_bytes, idx_out,
+                       lens_out, score_out, stream);
+}
+
+int bsa_fwd_3d_static(const bsa_3d_params* p, const void* q, const int64_t q_strides[3], const void* k,
+                      const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
+                      const int64_t o_strides[3], int32_t* idx_out, int32_t* lens_out, void* score_out, void* stream) {
+    Plan pl;
+    BSA_TRY(make_plan(p, &pl));
+    if (pl.total > kStaticScratchBytes)
+        return set_error(BSA_ERR_WORKSPACE, "fwd_3d_static: this problem needs %zu bytes of scratch memory, the built-in buffer holds %zu; "
+                         "use bsa_fwd_3d with a workspace of bsa_workspace_bytes()", pl.total, kStaticScratchBytes);
+    void* ws = nullptr;
+    BSA_TRY(static_scratch(&ws));
+    // Nothing in the buffer has to start at zero: every piece is written by the kernel sequence before it is
+    // read (the work counter of the queue schedule is cleared by a fill kernel inside launch_fwd).
+    return fwd_3d_impl(pl, p, q, q_strides, k, k_strides, v, v_strides, o, o_strides, ws, kStaticScratchBytes, idx_out,
+                       lens_out, score_out, stream);
 }
 
 }  // extern "C"

@@ -16,6 +16,7 @@ BSA_ERR_WORKSPACE = -4
 BSA_ERR_HIP = -5
 
 BSA_BF16, BSA_F16, BSA_F32 = 0, 1, 2
+BSA_STATIC_SCRATCH_BYTES = 64 << 20
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libbsa_mi355x.so")
 
@@ -46,6 +47,8 @@ SIGNATURES = {
     "bsa_workspace_bytes": (C.c_size_t, [C.POINTER(Bsa3dParams)]),
     "bsa_fwd_3d": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
                         _p, C.c_size_t, _p, _p, _p, _p]),
+    "bsa_fwd_3d_static": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
+                               _p, _p, _p, _p]),
     "bsa_thw_prepare": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, C.c_size_t, _p]),
     "bsa_fwd_thw": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
                          _p, _p, _i, _p, _p, C.c_size_t, _p]),

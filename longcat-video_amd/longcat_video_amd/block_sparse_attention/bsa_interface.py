@@ -322,9 +322,11 @@ def flash_attn_bsa(q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold,
 # R9: the operator
 # ---------------------------------------------------------------------------
 def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k, want_selection=False, out=None,
-            cdf_threshold=None):
+            cdf_threshold=None, static_scratch=False):
     """`out`: optional [B,H,Sq,D] view (any B/H/S strides, contiguous D) to write into.  `sparsity` may be
-    None when `cdf_threshold` is given (bsa_interface.py:268-277)."""
+    None when `cdf_threshold` is given (bsa_interface.py:268-277).  `static_scratch`: run through
+    bsa_fwd_3d_static, which keeps its scratch memory in a buffer built into the library instead of a
+    workspace tensor (problems beyond that buffer raise; calls on one GPU must not overlap)."""
     _need_gpu(q, k, v)
     B, H, Sq, D = q.shape
     Tq, Hq, Wq = (int(x) for x in latent_shape_q)
@@ -350,7 +352,7 @@ def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k,
     if need == 0:
         _capi.check(lib.bsa_fwd_3d(C.byref(prm), None, None, None, None, None, None, None, None, None, 0,
                                    None, None, None, None), "flash_attn_bsa_3d")
-    ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+    ws = None if static_scratch else torch.empty(need, dtype=torch.uint8, device=q.device)
     o = torch.empty(B, H, Sq, D, dtype=q.dtype, device=q.device) if out is None else out
     assert o.shape == (B, H, Sq, D) and o.dtype == q.dtype and o.stride(3) == 1
     idx = lens = score = None
@@ -359,10 +361,16 @@ def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k,
         lens = torch.empty(B, H, nbq, dtype=torch.int32, device=q.device)
         score = torch.empty(B, H, nbq, nbk, dtype=q.dtype, device=q.device)
     with torch.cuda.device(q.device):
-        _capi.check(lib.bsa_fwd_3d(
-            C.byref(prm), _ptr(q), _capi.strides3(q.stride()[:3]), _ptr(k), _capi.strides3(k.stride()[:3]),
-            _ptr(v), _capi.strides3(v.stride()[:3]), _ptr(o), _capi.strides3(o.stride()[:3]),
-            _ptr(ws), need, _ptr(idx), _ptr(lens), _ptr(score), _stream(q)), "flash_attn_bsa_3d")
+        if static_scratch:
+            _capi.check(lib.bsa_fwd_3d_static(
+                C.byref(prm), _ptr(q), _capi.strides3(q.stride()[:3]), _ptr(k), _capi.strides3(k.stride()[:3]),
+                _ptr(v), _capi.strides3(v.stride()[:3]), _ptr(o), _capi.strides3(o.stride()[:3]),
+                _ptr(idx), _ptr(lens), _ptr(score), _stream(q)), "flash_attn_bsa_3d (static scratch)")
+        else:
+            _capi.check(lib.bsa_fwd_3d(
+                C.byref(prm), _ptr(q), _capi.strides3(q.stride()[:3]), _ptr(k), _capi.strides3(k.stride()[:3]),
+                _ptr(v), _capi.strides3(v.stride()[:3]), _ptr(o), _capi.strides3(o.stride()[:3]),
+                _ptr(ws), need, _ptr(idx), _ptr(lens), _ptr(score), _stream(q)), "flash_attn_bsa_3d")
     return (o, idx, lens, score) if want_selection else o
 
 

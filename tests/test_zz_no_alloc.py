@@ -1,0 +1,71 @@
+"""The entry point that allocates nothing: bsa_fwd_3d_static keeps what bsa_fwd_3d carves from its workspace in
+a buffer built into the library.  It has no counterpart in the reference; it must give the bits of bsa_fwd_3d
+(same kernels), also on a second call with a smaller input that finds the first call's leftovers in the buffer,
+and must reject what does not fit."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import seeded_qkv
+
+pytestmark = pytest.mark.gpu
+
+
+def I():
+    from longcat_video_amd.block_sparse_attention import bsa_interface
+    return bsa_interface
+
+
+def both(seed, heads, latent, sparsity, chunk, dtype=torch.bfloat16, cdf=None):
+    S = int(np.prod(latent))
+    q, k, v = (t.cuda() for t in seeded_qkv(seed, 1, heads, S, S, 128, dtype))
+    got = I()._bsa_3d(q, k, v, latent, latent, sparsity, chunk, chunk, True, cdf_threshold=cdf, static_scratch=True)
+    torch.cuda.synchronize()
+    want = I()._bsa_3d(q, k, v, latent, latent, sparsity, chunk, chunk, True, cdf_threshold=cdf)
+    torch.cuda.synchronize()
+    return got, want
+
+
+def same(got, want):
+    o, idx, lens, score = got
+    o2, idx2, lens2, score2 = want
+    assert torch.equal(score, score2)
+    assert torch.equal(idx, idx2) and torch.equal(lens, lens2)          # integer results: bit-exact
+    assert torch.equal(o, o2)                                           # the same kernels on the same inputs
+    assert torch.isfinite(o.float()).all()
+
+
+def test_two_calls_in_a_row_the_second_smaller():
+    same(*both(90, 4, (9, 18, 26), 0.75, (4, 4, 4)))      # padded in t, h and w: edge copies, validity words, tables
+    same(*both(91, 2, (4, 8, 8), 0.5, (4, 4, 4)))         # smaller: every piece of the buffer sits at a lower offset
+    same(*both(92, 3, (5, 6, 12), 0.5, (4, 4, 8)))        # 128-token chunks
+    same(*both(93, 2, (4, 8, 8), 0.5, (4, 4, 4), dtype=torch.float32))   # fp32 route: blocked copies in the buffer
+    same(*both(94, 2, (5, 8, 12), 0.75, (4, 4, 4), cdf=0.6))             # lists of unequal length: order + queue words
+
+
+def test_matches_the_oracle_directly():
+    """Not only equal to the other entry point: the static route is held to the oracle on its own."""
+    from test_gpu_e2e import check_against_oracle
+    latent = (5, 9, 13)
+    S = int(np.prod(latent))
+    q, k, v = seeded_qkv(95, 1, 2, S, S, 128, torch.bfloat16)
+    o, idx, lens, score = I()._bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, 0.75, (4, 4, 4), (4, 4, 4), True,
+                                      static_scratch=True)
+    check_against_oracle(q, k, v, latent, latent, 0.75, o, idx, lens, score, q_blocks=range(24))
+
+
+def test_a_problem_beyond_the_buffer_is_rejected_before_any_launch():
+    from longcat_video_amd import _capi
+    lib = _capi.load()
+    latent = (24, 30, 52)                                 # 480p at 32 heads needs 118 MB of scratch memory
+    prm = _capi.Bsa3dParams(1, 32, 128, _capi.BSA_BF16, *latent, *latent, 4, 4, 4, 4, 4, 4, 39, 128 ** -0.5, 0.0)
+    assert lib.bsa_workspace_bytes(C.byref(prm)) > _capi.BSA_STATIC_SCRATCH_BYTES
+    one = torch.zeros(16, dtype=torch.bfloat16, device="cuda")           # never read: the size check comes first
+    st = _capi.strides3((0, 0, 128))
+    rc = lib.bsa_fwd_3d_static(C.byref(prm), one.data_ptr(), st, one.data_ptr(), st, one.data_ptr(), st, one.data_ptr(), st,
+                               None, None, None, None)
+    assert rc == _capi.BSA_ERR_WORKSPACE
+    assert "scratch" in _capi.last_error()
+    torch.cuda.synchronize()
