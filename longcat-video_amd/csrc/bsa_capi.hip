@@ -228,11 +228,14 @@ struct Plan {
     int sel_width;        // columns of the index lists: k_sel, or the cap of the CDF rule
     bool cdf;
     bool direct_qo, direct_kv;
+    bool frag;            // k and v are rewritten in fragment order for fwd_frag_kernel (bsa_fwd_frag.hip)
     size_t off_qp, off_kp, off_vp, off_op, off_qc, off_kc, off_score, off_idx, off_idx_sorted, off_lens, off_valid, off_qrows, off_ktiles, off_order, off_queue, total;
 };
 inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-int make_plan(const bsa_3d_params* p, Plan* pl) {
+// compact: keep the workspace small (k and v are gathered where they lie by fwd_mfma_kernel, only the chunks at the
+// padded edge are copied) instead of rewriting k and v in fragment order for the faster fwd_frag_kernel.
+int make_plan(const bsa_3d_params* p, Plan* pl, bool compact = false) {
     if (!p) return set_error(BSA_ERR_BAD_ARG, "params are null");
     BSA_TRY(check_row(p->D, p->dtype));
     BSA_TRY(check_grid(p->B, p->Hn, p->Tq, p->Hq, p->Wq, p->tq, p->hq, p->wq));
@@ -261,8 +264,10 @@ int make_plan(const bsa_3d_params* p, Plan* pl) {
     // order when the kv grid allows it; blocked copies are only made for the fp32 kernel and for
     // kv grids that do not qualify.
     pl->direct_qo = p->dtype != BSA_F32;
-    pl->direct_kv = pl->direct_qo && kv_direct_ok(pl->gk, (int64_t)p->D * pl->es);
+    pl->frag = pl->direct_qo && !compact;
+    pl->direct_kv = pl->direct_qo && !pl->frag && kv_direct_ok(pl->gk, (int64_t)p->D * pl->es);
     pl->off_qp = take(pl->direct_qo ? 0 : bh * pl->Sqp * p->D * pl->es);
+    // fragment order is a permutation of the padded blocked order: the same size
     const size_t kv_rows = pl->direct_kv ? (size_t)edge_count(pl->gk) * pl->gk.chunk() : (size_t)pl->Skp;
     pl->off_kp = take(bh * kv_rows * p->D * pl->es);
     pl->off_vp = take(bh * kv_rows * p->D * pl->es);
@@ -339,6 +344,19 @@ hipError_t prepare_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, cons
     else    // tables only: one (batch, head) slice of workgroups, no row is read
         e = launch_permute(q, q_strides, nullptr, nullptr, nullptr, 1, 1, pl.gq, p->D, p->dtype, st, false, w.qrows, nullptr);
     if (e != hipSuccess) return e;
+    if (pl.frag) {
+        // pooled means and validity words of k (one read of k), then k and v in fragment order
+        if (pool || padded_k) {
+            if (pool)
+                e = launch_permute(k, k_strides, nullptr, w.kc, padded_k ? w.valid : nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st);
+            else
+                e = launch_permute(k, k_strides, nullptr, nullptr, w.valid, 1, 1, pl.gk, p->D, p->dtype, st);
+            if (e != hipSuccess) return e;
+        }
+        e = launch_frag(k, k_strides, w.kp, p->B, p->Hn, pl.gk, p->dtype, false, st);
+        if (e != hipSuccess) return e;
+        return launch_frag(v, v_strides, w.vp, p->B, p->Hn, pl.gk, p->dtype, true, st);
+    }
     // gathering: the pass over k copies the edge chunks of v along with those of k
     e = launch_permute(k, k_strides, w.kp, pool ? w.kc : nullptr, padded_k ? w.valid : nullptr, p->B, p->Hn, pl.gk, p->D,
                        p->dtype, st, pl.direct_kv, nullptr, w.ktiles, pl.direct_kv && padded_k ? v : nullptr, v_strides, w.vp);
@@ -352,6 +370,10 @@ hipError_t attention_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, co
                          const void* k, const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
                          const int64_t o_strides[3], const int32_t* idx, const int32_t* lens, int idx_stride, float* lse,
                          hipStream_t st, bool by_length = false) {
+    if (pl.frag)
+        return launch_fwd_frag(q, w.kp, w.vp, idx, lens, kv_padded(p) ? w.valid : nullptr, o, lse, p->B, p->Hn, pl.Sqp, pl.Skp,
+                               pl.gq.chunk(), pl.gk.chunk(), idx_stride, p->sm_scale, p->dtype, st, w.qrows, q_strides, o_strides,
+                               (int64_t)p->Tq * p->Hq * p->Wq, by_length ? w.order : nullptr, by_length ? w.queue : nullptr);
     FwdLayout L;
     L.q_rows = w.qrows;
     L.k_tiles = w.ktiles;
@@ -521,7 +543,7 @@ int bsa_fwd_3d_static(const bsa_3d_params* p, const void* q, const int64_t q_str
                       const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
                       const int64_t o_strides[3], int32_t* idx_out, int32_t* lens_out, void* score_out, void* stream) {
     Plan pl;
-    BSA_TRY(make_plan(p, &pl));
+    BSA_TRY(make_plan(p, &pl, true));
     if (pl.total > kStaticScratchBytes)
         return set_error(BSA_ERR_WORKSPACE, "fwd_3d_static: this problem needs %zu bytes of scratch memory, the built-in buffer holds %zu; "
                          "use bsa_fwd_3d with a workspace of bsa_workspace_bytes()", pl.total, kStaticScratchBytes);

@@ -131,4 +131,21 @@ hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t
 hipError_t launch_order_by_length(const int32_t* lens, int32_t* order, int BH, int nbq, int tiles_per_block, int max_len,
                                   hipStream_t st);
 
+// queue[0] = 0 (the counter work items are drawn with) and queue[1] = the choice between rounds (0) and the
+// longest-first queue (1), made on the device from the list lengths (see choose_schedule_kernel)
+void launch_schedule_choice(const int32_t* lens, int nbq, int tiles_per_block, int total, int round, int resident,
+                            int max_len, uint32_t* queue, hipStream_t st);
+
+// K or V of a (T, H, W)-ordered tensor in fragment order (bsa_fwd_frag.hip): dst [B*Hn][padded slots / 64][16 KB],
+// padded slots zero; transpose = false for K, true for V.  bf16 / fp16.
+hipError_t launch_frag(const void* src, const int64_t strides[3], void* dst, int B, int Hn, const Grid3& g, int dtype,
+                       bool transpose, hipStream_t st);
+// The attention kernel on fragment-order K and V.  q_rows (optional): token row of every blocked-order query
+// slot, -1 for padding; q_st / o_st: element strides {batch, head, row}; lse_rows: rows per (batch, head) of lse.
+hipError_t launch_fwd_frag(const void* q, const void* kf, const void* vf, const int32_t* idx, const int32_t* lens,
+                           const uint64_t* tile_valid, void* o, float* lse, int B, int Hn, int64_t Sq, int64_t Sk,
+                           int bs_q, int bs_k, int idx_stride, float sm_scale, int dtype, hipStream_t st,
+                           const int32_t* q_rows, const int64_t q_st[3], const int64_t o_st[3], int64_t lse_rows,
+                           const int32_t* order = nullptr, uint32_t* queue = nullptr);
+
 }  // namespace bsa

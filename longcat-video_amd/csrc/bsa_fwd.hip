@@ -608,6 +608,13 @@ __global__ __launch_bounds__(256) void choose_schedule_kernel(const int32_t* __r
     }
 }
 
+void launch_schedule_choice(const int32_t* lens, int nbq, int tiles_per_block, int total, int round, int resident,
+                            int max_len, uint32_t* queue, hipStream_t st) {
+    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, st, queue, 1);
+    hipLaunchKernelGGL(choose_schedule_kernel, dim3(1), dim3(256), 0, st, lens, nbq, tiles_per_block, total, round, resident,
+                       max_len, queue + 1);
+}
+
 hipError_t launch_order_by_length(const int32_t* lens, int32_t* order, int BH, int nbq, int tiles_per_block, int max_len,
                                   hipStream_t st) {
     hipLaunchKernelGGL(order_by_length_kernel, dim3((unsigned)BH), dim3(256), (size_t)(max_len + 1) * sizeof(int), st, lens, order,
@@ -678,9 +685,7 @@ hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t
         // Lists of possibly unequal length.  queue[0] is the counter the items are drawn with, queue[1] the
         // choice between the two schedules, made on the device from the lengths; both are enqueued.
         const int total = B * Hn * per_head;
-        hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, st, queue, 1);
-        hipLaunchKernelGGL(choose_schedule_kernel, dim3(1), dim3(256), 0, st, lens, (int)(Sq / bs_q), bs_q / kTile, total, round, resident,
-                           idx_stride, queue + 1);
+        launch_schedule_choice(lens, (int)(Sq / bs_q), bs_q / kTile, total, round, resident, idx_stride, queue, st);
         gate = queue + 1;
         const dim3 grid((unsigned)(total < resident ? total : resident));
         if (dtype == BSA_BF16)

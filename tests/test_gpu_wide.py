@@ -85,7 +85,10 @@ def test_thw_attention_with_256_token_chunks_equals_the_blocked_route(latent, ch
     op, _ = bi.attn_fwd_bsa_varlen(qp, kp, vp, 0.09, idx, lens, bs, bs, tile_valid=valid)
     want = bi.rearrange_3d_block_to_THW(op, *O.block_grid(latent, chunk), *chunk, 128, latent_shape=latent)
     got = bi.attn_fwd_bsa_thw(q, k, v, latent, latent, chunk, chunk, idx, lens, sm_scale=0.09)
-    assert torch.equal(got, want)
+    # two kernels: P rounded relative to different running maxima, sums in different orders
+    d = (got.float() - want.float()).abs()
+    assert d.max() <= 1.6e-2 and d.mean() <= 1e-3, (float(d.max()), float(d.mean()))
+    assert torch.equal(got == 0, want == 0)
 
 
 # ------------------------------------------------------------------ long index lists

@@ -1,7 +1,9 @@
-"""The entry point that allocates nothing: bsa_fwd_3d_static keeps what bsa_fwd_3d carves from its workspace in
-a buffer built into the library.  It has no counterpart in the reference; it must give the bits of bsa_fwd_3d
-(same kernels), also on a second call with a smaller input that finds the first call's leftovers in the buffer,
-and must reject what does not fit."""
+"""The entry point that allocates nothing: bsa_fwd_3d_static keeps its scratch memory in a buffer built into the
+library.  It has no counterpart in the reference.  It runs the compact route of the operator (k and v gathered
+where they lie), bsa_fwd_3d the route that rewrites k and v in fragment order: the same pooling, score and
+selection kernels, so scores and selection must agree bit for bit, and two attention kernels that agree to fp32
+summation order (fp32 inputs take one route in both).  Checked on calls in a row, the later ones smaller, which
+find the earlier calls' leftovers in the buffer; a problem that does not fit must be rejected."""
 import ctypes as C
 
 import numpy as np
@@ -33,7 +35,11 @@ def same(got, want):
     o2, idx2, lens2, score2 = want
     assert torch.equal(score, score2)
     assert torch.equal(idx, idx2) and torch.equal(lens, lens2)          # integer results: bit-exact
-    assert torch.equal(o, o2)                                           # the same kernels on the same inputs
+    if o.dtype == torch.float32:
+        assert torch.equal(o, o2)                                       # one route, the same kernels
+    else:
+        d = (o.float() - o2.float()).abs()                              # two attention kernels: a couple of bf16 ulps
+        assert d.max() <= 1.6e-2 and d.mean() <= 1e-3, (float(d.max()), float(d.mean()))
     assert torch.isfinite(o.float()).all()
 
 
