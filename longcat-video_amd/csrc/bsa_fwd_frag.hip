@@ -34,14 +34,15 @@
 // dot, exp2, P rounded to the storage type for the P V product, fp32 row sum, one final rounding.
 #include "bsa_mfma.h"
 
+#include <utility>
+
 namespace bsa {
 namespace {
 
 using namespace mfma;
 
 constexpr int kHalfBytes = 8192;      // 32 keys of a fragment-order K (or V) tile
-constexpr int kRing = 2;              // steps of K fragments and of V fragments in flight
-constexpr int kUnroll = 2;            // steps per loop body: one tile (two halves), which is also one turn of the rings
+constexpr int kListEntries = 4096;    // longest list a work item can walk (its staging area in LDS: 17 KB)
 
 // ------------------------------------------------------------------ relayout
 // One workgroup per 64-slot tile of one (batch, head): the 64 rows are gathered from (T, H, W) order
@@ -101,6 +102,17 @@ __global__ __launch_bounds__(256) void frag_kernel(const T* __restrict__ src, in
 }
 
 // ------------------------------------------------------------------ attention
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
+// in every copy of the body (the register arrays of the kernel must never be indexed by a run-time value).
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 // S^T accumulators must sit in ordinary VGPRs, where the softmax reads them, while the (four times larger)
 // output accumulators belong in AGPRs.  For a kernel that may use more than 256 registers the compiler puts
 // the result of every builtin MFMA into AGPRs, so the S^T MFMAs are written as inline assembly with VGPR
@@ -136,7 +148,8 @@ struct FragLayout {
     int64_t q_st[3], o_st[3];     // element strides: batch, head, row
 };
 
-template <typename T>
+// kNsub1: KV blocks of one 64-key tile (bs_k == 64): no division in the walk.
+template <typename T, bool kNsub1>
 __global__ __launch_bounds__(64) void fwd_frag_kernel(
     const T* __restrict__ q, const char* __restrict__ kf, const char* __restrict__ vf,
     const int32_t* __restrict__ idx, const int32_t* __restrict__ lens, const uint64_t* __restrict__ tile_valid,
@@ -145,15 +158,17 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
     const int32_t* __restrict__ order, uint32_t* __restrict__ queue, const uint32_t* __restrict__ gate, uint32_t gate_want) {
     typedef typename Vec8<T>::type V8;
     if (gate != nullptr && *gate != gate_want) return;
-    // output staging: 64 rows of 256 B, 272 B apart
+    // output staging: 64 rows of 256 B, 272 B apart.  During the tile loop the same memory holds the work item's
+    // list of KV blocks (kListEntries words at most), bit 31 of an entry flagging a block with padded keys.
     constexpr int kOutPitch = kD + 8;
     __shared__ __attribute__((aligned(16))) T ost[kTile * kOutPitch];
+    uint32_t* const ents = reinterpret_cast<uint32_t*>(ost);
 
     const int lane = threadIdx.x;
     const int lr = lane & 31, lh = lane >> 5;
     const int nbq = (int)(Sq / bs_q);
     const int nqt = (int)(Sq / kTile);
-    const int nsub = bs_k / kTile;
+    const int nsub = kNsub1 ? 1 : bs_k / kTile;
     const int nbk = (int)(Sk / bs_k);
     const int64_t kv_bh_bytes = (Sk / kTile) * (int64_t)kTileBytes;
     const uint32_t lane_off = (uint32_t)lane * 16u;
@@ -179,8 +194,18 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
     const int64_t q_bh = (int64_t)(bh / Hn) * L.q_st[0] + (int64_t)(bh % Hn) * L.q_st[1];
     const int64_t o_bh = (int64_t)(bh / Hn) * L.o_st[0] + (int64_t)(bh % Hn) * L.o_st[1];
     const int32_t* list = idx + ((int64_t)bh * nbq + qblock) * idx_stride;
-    const int ntiles = min(max(lens[(int64_t)bh * nbq + qblock], 0), idx_stride) * nsub;
+    const int nent = min(min(max(lens[(int64_t)bh * nbq + qblock], 0), idx_stride), kListEntries);
+    const int ntiles = nent * nsub;
     const int nsteps = 2 * ntiles;
+    // the list goes to LDS: clamped block index (a malformed list gives wrong numbers, never a fault) and the flag
+    for (int e = lane; e < nent; e += 64) {
+        const int blk = min(max(list[e], 0), nbk - 1);
+        uint32_t flag = 0;
+        if (tile_valid != nullptr)
+            for (int sub = 0; sub < nsub; ++sub) flag |= tile_valid[blk * nsub + sub] != ~0ull ? 1u : 0u;
+        ents[e] = (uint32_t)blk | (flag << 31);
+    }
+    __syncthreads();
     const char* kbase = kf + (int64_t)bh * kv_bh_bytes;
     const char* vbase = vf + (int64_t)bh * kv_bh_bytes;
 
@@ -205,93 +230,133 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
     float m_i[2] = {-INFINITY, -INFINITY}, l_i[2] = {0.f, 0.f};
 
     if (nsteps > 0) {
-    // Position tp of the tile walk -> byte offset of the tile inside this (batch, head) and its validity
-    // word.  Positions behind the list repeat the last tile with every key masked out, so that the loop
-    // body can run in whole groups of kUnroll steps.  A block index outside [0, nbk) is clamped.
-    auto tile_of = [&](int tp) -> uint32_t {
+    // Position tp of the tile walk -> tile inside this (batch, head) and validity word of its 64 keys.  Positions
+    // behind the list repeat the last tile with every key masked out.  The entry is read from LDS (entry_raw, to
+    // be issued early) and decoded later (entry_tile / entry_mask).
+    auto entry_raw = [&](int tp) -> uint32_t {
         const int tc = min(tp, ntiles - 1);
-        const int blk = min(max(list[tc / nsub], 0), nbk - 1);
-        return (uint32_t)(blk * nsub + tc % nsub);
+        return ents[kNsub1 ? tc : tc / nsub];                   // the same address in every lane
     };
-    auto mask_of = [&](int tp, uint32_t tile) -> uint64_t {
+    auto entry_tile = [&](int tp, uint32_t raw) -> uint32_t {
+        const uint32_t blk = (uint32_t)__builtin_amdgcn_readfirstlane((int)raw) & 0x7fffffffu;
+        if (kNsub1) return blk;
+        return blk * (uint32_t)nsub + (uint32_t)(min(tp, ntiles - 1) % nsub);
+    };
+    auto entry_mask = [&](int tp, uint32_t raw, uint32_t tile) -> uint64_t {
         if (tp >= ntiles) return 0ull;
-        return tile_valid != nullptr ? tile_valid[tile] : ~0ull;
+        if (__builtin_expect(__builtin_amdgcn_readfirstlane((int)raw) < 0, 0)) return tile_valid[tile];
+        return ~0ull;
     };
-    // window of the walk: entries for positions g .. g+3 of loop iteration g (one tile per iteration)
-    uint32_t w_tile[4];
-    uint64_t w_mask[4];
+    // window of the walk: positions g, g + 1, g + 2 of loop iteration g (one tile per iteration)
+    uint32_t w_tile[3];
+    uint64_t w_mask[3];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) { w_tile[r] = tile_of(r); w_mask[r] = mask_of(r, w_tile[r]); }
+    for (int r = 0; r < 3; ++r) {
+        const uint32_t raw = entry_raw(r);
+        w_tile[r] = entry_tile(r, raw);
+        w_mask[r] = entry_mask(r, raw, w_tile[r]);
+    }
 
-    V8 kb[kRing][8], vb[kRing][8];
-    // fragments of step (tile window slot r, half h) into ring slot `slot`
-    auto load_k = [&](auto slot, int r, int h) {
-        constexpr int sl = decltype(slot)::value;
-        const char* p = kbase + (uint64_t)w_tile[r] * kTileBytes + h * kHalfBytes + lane_off;
-#pragma unroll
-        for (int c = 0; c < 8; ++c) kb[sl][c] = *reinterpret_cast<const V8*>(p + c * 1024);
+    // Register rings: K fragments of two steps, V fragments of two steps (each step: 4 fragments for its
+    // first 16 keys, "A", and 4 for its last 16, "B").
+    V8 kb[2][8], vb[2][8];
+    f32x16 s[2][2];                                            // S^T of the current and of the next step
+    V8 pb[2][2];                                               // P^T as B operand: [query half][A | B]
+    auto k_frag = [&](int r, int h, int c) -> V8 {          // window slot r, half h, d step c
+        return *reinterpret_cast<const V8*>(kbase + (uint64_t)w_tile[r] * kTileBytes + h * kHalfBytes + lane_off + c * 1024);
     };
-    auto load_v = [&](auto slot, int r, int h) {
-        constexpr int sl = decltype(slot)::value;
-        const char* p = vbase + (uint64_t)w_tile[r] * kTileBytes + h * kHalfBytes + lane_off;
-#pragma unroll
-        for (int c = 0; c < 8; ++c) vb[sl][c] = *reinterpret_cast<const V8*>(p + c * 1024);
+    auto v_frag = [&](int r, int h, int f) -> V8 {          // f = 4 * key step + d tile
+        return *reinterpret_cast<const V8*>(vbase + (uint64_t)w_tile[r] * kTileBytes + h * kHalfBytes + lane_off + f * 1024);
     };
     // accumulator i <-> key 8 (i / 4) + 4 lh + i % 4 of the step's 32 keys, query lr (+32)
-    auto mask_pair = [&](f32x16 (&s)[2], uint32_t half) {
+    auto mask_pair = [&](f32x16 (&sv)[2], uint32_t half) {
         if (__builtin_expect(half != ~0u, 0)) {
+            asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");       // the MFMAs into these accumulators have retired
 #pragma unroll
             for (int i = 0; i < 16; ++i)
-                if (!((half >> (8 * (i / 4) + 4 * lh + (i % 4))) & 1u)) { s[0][i] = -INFINITY; s[1][i] = -INFINITY; }
+                if (!((half >> (8 * (i / 4) + 4 * lh + (i % 4))) & 1u)) { sv[0][i] = -INFINITY; sv[1][i] = -INFINITY; }
         }
     };
+    // Softmax state per query half: running maximum m_i (scaled, log2 units), its negative for the exponent
+    // (0 while the maximum is -inf), and the unscaled logit above which the maximum has to be raised.
+    float neg_m[2] = {0.f, 0.f}, raise_at[2] = {-INFINITY, -INFINITY};
+    const float inv_scale = 1.0f / qk_scale;
+    // Raising the
+    // maximum has two parts.  Here: the new maximum, the exponent offset, the row sum (which already holds
+    // every probability of the current step).  The output accumulators are rescaled one quarter of a step later
+    // (rescale_out, behind slot 7 of the next step): the product of the current step's P_B, whose
+    // probabilities were taken relative to the old maximum, is only issued in slots 0 .. 7 of that step.
+    float alpha_p[2] = {1.f, 1.f};
+    bool rescale_pending = false;
+    // combine a lane's maximum with the other key group of the same query (lane ^ 32)
+    auto finish_max = [&](float mx) -> float {
+        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+        return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    };
+    // mx0, mx1: this lane's unscaled maxima over its 16 accumulators of the step that comes next.  The test
+    // needs no exchange between the two key groups of a query: some lane exceeds the limit exactly when the
+    // combined maximum does.
     auto raise_max = [&](float mx0, float mx1) {
-        if (__builtin_expect(__any(mx0 > m_i[0] + kLazyTau || mx1 > m_i[1] + kLazyTau), 0)) {
-            const float mx[2] = {mx0, mx1};
-            asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");       // the last MFMA into the accumulators has retired
+        if (__builtin_expect(__any(mx0 > raise_at[0] || mx1 > raise_at[1]), 0)) {
+            const float mx[2] = {finish_max(mx0) * qk_scale, finish_max(mx1) * qk_scale};
 #pragma unroll
             for (int qq = 0; qq < 2; ++qq) {
                 const float m_new = fmaxf(m_i[qq], mx[qq]);
                 const float alpha = __builtin_amdgcn_exp2f(m_i[qq] - ((m_new == -INFINITY) ? 0.f : m_new));
                 m_i[qq] = m_new;
+                neg_m[qq] = (m_new == -INFINITY) ? 0.f : -m_new;
+                raise_at[qq] = (m_new + kLazyTau) * inv_scale;
                 l_i[qq] *= alpha;
-                // The output accumulators live in AGPRs, which the VALU cannot multiply in place.  Written out
-                // register by register through one temporary, so that this rare path does not make the compiler
-                // reserve VGPRs for a copy of the accumulators.
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        float x = oacc[t][qq][i], tmp;
-                        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 1\n\tv_accvgpr_write_b32 %0, %1"
-                                     : "+a"(x), "=&v"(tmp) : "v"(alpha));
-                        oacc[t][qq][i] = x;
-                    }
+                alpha_p[qq] = alpha;
             }
-            asm volatile("s_nop 7" ::: "memory");                    // AGPR writes before the next MFMA reads them
+            rescale_pending = true;
         }
     };
-    // combine a lane's maximum with the other key group of the same query (lane ^ 32) and scale it
-    auto finish_max = [&](float mx) -> float {
-        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
-        return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])) * qk_scale;
+    // The output accumulators live in AGPRs, which the VALU cannot multiply in place.  Written out register by
+    // register through one temporary, so that this rare path does not make the compiler reserve VGPRs for a copy
+    // of the accumulators.
+    auto rescale_out = [&]() {
+        asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMA into the accumulators has retired
+        static_for<128>([&](auto n_c) {
+            constexpr int n = decltype(n_c)::value, qq = n >> 6, t = (n >> 4) & 3, i = n & 15;
+            float x = oacc[t][qq][i], tmp;
+            asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 1\n\tv_accvgpr_write_b32 %0, %1"
+                         : "+a"(x), "=&v"(tmp) : "v"(alpha_p[qq]));
+            oacc[t][qq][i] = x;
+        });
+        asm volatile("s_nop 7" ::: "memory");                        // AGPR writes before the next MFMA reads them
+        rescale_pending = false;
     };
 
-    // ---- prologue: K(0), V(0), K(1), V(1) in flight; S(0) with nothing to overlap; then K(2)
-    load_k(std::integral_constant<int, 0>{}, 0, 0);
-    load_v(std::integral_constant<int, 0>{}, 0, 0);
-    load_k(std::integral_constant<int, 1>{}, 0, 1);
-    load_v(std::integral_constant<int, 1>{}, 0, 1);
-    f32x16 s[2][2];
-#pragma unroll
-    for (int c = 0; c < 8; ++c) {
-        if (c == 0) { mfma_s<true, false>(s[0][0], kb[0][0], qreg[0][0]); mfma_s<true, true>(s[0][1], kb[0][0], qreg[1][0]); }
-        else { mfma_s<false, false>(s[0][0], kb[0][c], qreg[0][c]); mfma_s<false, true>(s[0][1], kb[0][c], qreg[1][c]); }
-    }
-    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");               // MFMA results before the VALU reads them
-    load_k(std::integral_constant<int, 0>{}, 1, 0);                  // K(2)
-    mask_pair(s[0], (uint32_t)w_mask[0]);
+    // ---- prologue.  In flight when the loop starts: K(1), K(2), V_A(0), V_B(0), V_A(1); the ring slot of
+    // V_B(1) holds zeros, which the first step multiplies with P = 0 (there is no step -1).
     {
+        V8 k0[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) k0[c] = k_frag(0, 0, c);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) kb[1][c] = k_frag(0, 1, c);                 // K(1)
+#pragma unroll
+        for (int f = 0; f < 8; ++f) vb[0][f] = v_frag(0, 0, f);                 // V_A(0), V_B(0)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) kb[0][c] = k_frag(1, 0, c);                 // K(2)
+#pragma unroll
+        for (int f = 0; f < 4; ++f) vb[1][f] = v_frag(0, 1, f);                 // V_A(1)
+#pragma unroll
+        for (int f = 4; f < 8; ++f)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) vb[1][f][e] = (T)0.f;
+#pragma unroll
+        for (int qq = 0; qq < 2; ++qq)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pb[qq][1][e] = (T)0.f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            if (c == 0) { mfma_s<true, false>(s[0][0], k0[0], qreg[0][0]); mfma_s<true, true>(s[0][1], k0[0], qreg[1][0]); }
+            else { mfma_s<false, false>(s[0][0], k0[c], qreg[0][c]); mfma_s<false, true>(s[0][1], k0[c], qreg[1][c]); }
+        }
+        asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");           // MFMA results before the VALU reads them
+        mask_pair(s[0], (uint32_t)w_mask[0]);
         float mx[2];
 #pragma unroll
         for (int qq = 0; qq < 2; ++qq) {
@@ -299,112 +364,140 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
 #pragma unroll
             for (int i = 2; i < 16; i += 2) mx[qq] = fmaxf(fmaxf(mx[qq], s[0][qq][i]), s[0][qq][i + 1]);
         }
-        raise_max(finish_max(mx[0]), finish_max(mx[1]));
+        raise_max(mx[0], mx[1]);
+        rescale_pending = false;                                     // nothing accumulated yet
     }
 
-    // Step u = 2 g + j (j static).  S(u) is finished and the running maximum covers it.
-    //   X: S(u+1) = K(u+1) . Q^T from ring slot (j+1) % 2, under the exp2 of the first part of S(u);
-    //      then K(u+3) is requested into that slot.
-    //   Y: O^T += V(u)^T P(u)^T from ring slot j % 2: the MFMAs of the first 16 keys under the exp2 of
-    //      the rest of S(u), those of the last 16 keys under the row maximum of S(u+1);
-    //      then V(u+2) is requested into that slot.
+    // Step u = 2 g + j (j static).  On entry S(u) is complete and the running maximum covers it; P_B(u-1) is
+    // complete.  The 32 MFMAs of a step, in issue order ("slots"):
+    //    0 ..  7   O^T += V_B(u-1)^T P_B(u-1)^T      the last 16 keys of the previous step
+    //    8 .. 23   S(u+1)^T = K(u+1) Q^T
+    //   24 .. 31   O^T += V_A(u)^T P_A(u)^T          the first 16 keys of this step
+    // The VALU work on S(u) - per pair of accumulators two fma, two exp2, two additions for the row sum and one
+    // rounding of the pair to the storage type, 16 pairs - is cut into pieces that go between the MFMAs so that
+    // no gap holds more than an MFMA lasts: the first 14 pairs behind slots 0 .. 23 (the eight pairs of P_A
+    // first: they are complete well before slot 24), the last two behind slots 24 .. 31 together with the row
+    // maximum of S(u+1), which is complete by then.  Fragment registers are reloaded in bursts behind the last
+    // MFMA that reads them: V_B(u+1) behind slot 7, K(u+3) behind slot 23, V_A(u+2) behind slot 31, so that every
+    // fragment is requested two steps before it is used.
     auto step = [&](auto jj) {
         constexpr int j = decltype(jj)::value;
         constexpr int sc = j & 1, sn = sc ^ 1;                 // S(u) and S(u+1) alternate between two register sets
-        constexpr int kslot = (j + 1) % kRing, vslot = j % kRing;
-        float neg_m[2];
-        V8 pb[2][2];                                            // P^T as B operand: [query half][key step]
-        float psum[2];
-#pragma unroll
-        for (int qq = 0; qq < 2; ++qq) neg_m[qq] = (m_i[qq] == -INFINITY) ? 0.f : -m_i[qq];
-        // The exp2 of a pair of accumulators and the use of its results sit in different slots between the
-        // MFMAs: a transcendental result cannot be consumed by the next instruction without a wait state.
-        float pa0, pa1;
-        auto exp_pair = [&](int n) {                            // pair n: query half n & 1, accumulators 2 (n >> 1), + 1
+        constexpr int kslot = (j + 1) & 1;                     // ring slot of K(u+1), then of K(u+3)
+        constexpr int vprev = (j + 1) & 1, vcur = j & 1;       // ring slots of V(u-1) / V(u+1) and of V(u) / V(u+2)
+        // pair n: query half n & 1, accumulators 2 (n >> 1), + 1.  Its arithmetic comes in three pieces of about the
+        // same cost - exponential of the first accumulator (h0), of the second (h1), and the use of both: row sum
+        // and rounding (t) - in the order h0(0) h1(0) h0(1) t(0) h1(1) h0(2) t(1) h1(2) ...: the result of a
+        // transcendental instruction cannot be consumed by the next instruction without a wait state.
+        float pa[2][2];
+        auto piece = [&](int p) {                               // p = 0 .. 47
+            // p = 0: h0(0); p = 1: h1(0); p = 2 + 3 k: h0(k + 1); p = 3 + 3 k: t(k); p = 4 + 3 k: h1(k + 1); p = 47: t(15)
+            const int k = p < 2 ? 0 : (p - 2) / 3, r = p < 2 ? 0 : (p - 2) % 3;
+            const bool is_t = p == 47 || (p >= 2 && r == 1);
+            const int n = p < 2 ? 0 : p == 47 ? 15 : (r == 1 ? k : k + 1);
+            const int e = p < 2 ? p : (r == 0 ? 0 : 1);         // which accumulator of the pair (h0 / h1)
             const int qq = n & 1, i = 2 * (n >> 1);
-            pa0 = __builtin_amdgcn_exp2f(fmaf(s[sc][qq][i], qk_scale, neg_m[qq]));
-            pa1 = __builtin_amdgcn_exp2f(fmaf(s[sc][qq][i + 1], qk_scale, neg_m[qq]));
+            if (is_t) {
+                l_i[qq] += pa[n & 1][0] + pa[n & 1][1];
+                pb[qq][i >> 3][i & 7] = (T)pa[n & 1][0];
+                pb[qq][i >> 3][(i + 1) & 7] = (T)pa[n & 1][1];
+                asm volatile("" : "+v"(l_i[qq]), "+v"(pb[qq][i >> 3]));
+            } else {
+                pa[n & 1][e] = __builtin_amdgcn_exp2f(fmaf(s[sc][qq][i + e], qk_scale, neg_m[qq]));
+                asm volatile("" : "+v"(pa[n & 1][e]));
+            }
         };
-        auto use_pair = [&](int n) {
-            const int qq = n & 1, i = 2 * (n >> 1);
-            if (n < 2) psum[qq] = pa0 + pa1;
-            else psum[qq] += pa0 + pa1;
-            pb[qq][i >> 3][i & 7] = (T)pa0;
-            pb[qq][i >> 3][(i + 1) & 7] = (T)pa1;
-            asm volatile("" : "+v"(psum[qq]), "+v"(pb[qq][i >> 3]));
-        };
-        constexpr int kPairsX = 12;                             // pairs handled under the MFMAs of X; the other 4 under Y
+        float mx[2];
         __builtin_amdgcn_sched_barrier(0);
-        // X: 16 MFMAs
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {
-#pragma unroll
-            for (int qq = 0; qq < 2; ++qq) {
-                if (qq == 0) {
-                    if (c == 0) mfma_s<true, false>(s[sn][0], kb[kslot][0], qreg[0][0]);
+        static_for<32>([&](auto slot_c) {
+            constexpr int slot = decltype(slot_c)::value;
+            // ---- the MFMA of this slot
+            if constexpr (slot < 8) {
+                constexpr int t = slot >> 1, qq = slot & 1;
+                oacc[t][qq] = mfma32(vb[vprev][4 + t], pb[qq][1], oacc[t][qq]);
+            } else if constexpr (slot < 24) {
+                constexpr int c = (slot - 8) >> 1, qq = slot & 1;
+                if constexpr (qq == 0) {
+                    if constexpr (c == 0) mfma_s<true, false>(s[sn][0], kb[kslot][0], qreg[0][0]);
                     else mfma_s<false, false>(s[sn][0], kb[kslot][c], qreg[0][c]);
                 } else {
-                    if (c == 0) mfma_s<true, true>(s[sn][1], kb[kslot][0], qreg[1][0]);
+                    if constexpr (c == 0) mfma_s<true, true>(s[sn][1], kb[kslot][0], qreg[1][0]);
                     else mfma_s<false, true>(s[sn][1], kb[kslot][c], qreg[1][c]);
                 }
-                const int n = 2 * c + qq;                       // 0 .. 15
-                if (n >= 1 && n <= kPairsX) use_pair(n - 1);
-                if (n < kPairsX) exp_pair(n);
-                __builtin_amdgcn_sched_barrier(0);
+            } else {
+                constexpr int t = (slot - 24) >> 1, qq = slot & 1;
+                oacc[t][qq] = mfma32(vb[vcur][t], pb[qq][0], oacc[t][qq]);
             }
-        }
-        // K(u+3): tile window slot (j + 3) / 2, half (j + 1) & 1
-        load_k(std::integral_constant<int, kslot>{}, (j + 3) >> 1, (j + 1) & 1);
-        __builtin_amdgcn_sched_barrier(0);
-        // Y, first 16 keys: 8 MFMAs under the remaining pairs
+            // ---- reloads, in bursts behind the last MFMA that reads the fragments (single loads between the
+            // arithmetic cost more issue time than they take): V_B(u+1), K(u+3), V_A(u+2)
+            if constexpr (slot == 7) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-#pragma unroll
-            for (int qq = 0; qq < 2; ++qq) {
-                oacc[t][qq] = mfma32(vb[vslot][t], pb[qq][0], oacc[t][qq]);
-                const int n = kPairsX + 2 * t + qq;             // 12 .. 19
-                if (n > kPairsX && n <= 16) use_pair(n - 1);
-                if (n < 16) exp_pair(n);
-                __builtin_amdgcn_sched_barrier(0);
+                for (int t = 0; t < 4; ++t) vb[vprev][4 + t] = v_frag((j + 1) >> 1, (j + 1) & 1, 4 + t);
             }
-        }
-        l_i[0] += psum[0];
-        l_i[1] += psum[1];
-        // validity of the keys of step u + 1: tile window slot (j + 1) / 2, half (j + 1) & 1
-        mask_pair(s[sn], (uint32_t)(w_mask[(j + 1) >> 1] >> (32 * ((j + 1) & 1))));
-        // Y, last 16 keys: 8 MFMAs under the row maximum of S(u+1)
-        float mx[2] = {fmaxf(s[sn][0][0], s[sn][0][1]), fmaxf(s[sn][1][0], s[sn][1][1])};
+            if constexpr (slot == 23) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+                for (int c = 0; c < 8; ++c) kb[kslot][c] = k_frag((j + 3) >> 1, (j + 1) & 1, c);
+            }
+            if constexpr (slot == 31) {
 #pragma unroll
-            for (int qq = 0; qq < 2; ++qq) {
-                oacc[t][qq] = mfma32(vb[vslot][4 + t], pb[qq][1], oacc[t][qq]);
-                const int n = 2 * t + qq;                       // 0 .. 7: two of the 14 remaining accumulators each
-                if (n < 7) {
-                    mx[0] = fmaxf(fmaxf(mx[0], s[sn][0][2 * n + 2]), s[sn][0][2 * n + 3]);
-                    mx[1] = fmaxf(fmaxf(mx[1], s[sn][1][2 * n + 2]), s[sn][1][2 * n + 3]);
+                for (int t = 0; t < 4; ++t) vb[vcur][t] = v_frag((j + 2) >> 1, j & 1, t);
+            }
+            if constexpr (slot == 7) {
+                if (__builtin_expect(rescale_pending, 0)) rescale_out();
+            }
+            // ---- VALU pieces: 42 of the 48 (14 pairs) behind slots 0 .. 23, one or two per slot; the other 6 behind
+            // slots 24 .. 31 next to the row maximum of S(u+1).  S(u+1) is first read behind slot 25: its last MFMA
+            // (slot 23) has retired by the time the MFMA of slot 25 has been issued, which the compiler cannot
+            // check for the assembly MFMAs.
+            if constexpr (slot < 24) {
+                constexpr int lo = (slot * 42) / 24, hi = ((slot + 1) * 42) / 24;      // one or two pieces
+                piece(lo);
+                if constexpr (hi - lo > 1) piece(lo + 1);
+            } else {
+                constexpr int r = slot - 24;                    // 0 .. 7
+                if constexpr (r == 0) { piece(42); piece(43); }
+                if constexpr (r == 1) {
+                    // validity of the keys of step u + 1: tile window slot (j + 1) / 2, half (j + 1) & 1
+                    mask_pair(s[sn], (uint32_t)(w_mask[(j + 1) >> 1] >> (32 * ((j + 1) & 1))));
+                    mx[0] = fmaxf(fmaxf(s[sn][0][0], s[sn][0][1]), s[sn][0][2]);
+                    mx[1] = fmaxf(fmaxf(s[sn][1][0], s[sn][1][1]), s[sn][1][2]);
+                    mx[0] = fmaxf(fmaxf(mx[0], s[sn][0][3]), s[sn][0][15]);
+                    mx[1] = fmaxf(fmaxf(mx[1], s[sn][1][3]), s[sn][1][15]);
                 }
-                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (r >= 2 && r < 7) {                // accumulators 4 .. 13, two per slot and query half
+                    mx[0] = fmaxf(fmaxf(mx[0], s[sn][0][2 * r]), s[sn][0][2 * r + 1]);
+                    mx[1] = fmaxf(fmaxf(mx[1], s[sn][1][2 * r]), s[sn][1][2 * r + 1]);
+                }
+                if constexpr (r == 7) {
+                    mx[0] = fmaxf(mx[0], s[sn][0][14]);
+                    mx[1] = fmaxf(mx[1], s[sn][1][14]);
+                }
+                if constexpr (r == 2) piece(44);
+                if constexpr (r == 4) piece(45);
+                if constexpr (r == 6) piece(46);
+                if constexpr (r == 7) piece(47);
             }
-        }
-        // V(u+2): tile window slot (j + 2) / 2, half j & 1
-        load_v(std::integral_constant<int, vslot>{}, (j + 2) >> 1, j & 1);
-        raise_max(finish_max(mx[0]), finish_max(mx[1]));
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        raise_max(mx[0], mx[1]);
     };
 
     for (int g = 0; g < ntiles; ++g) {
-        // entry of the window position that comes in (g + 4), read ahead
-        const uint32_t n_tile = tile_of(g + 4);
+        const uint32_t raw = entry_raw(g + 3);                  // the position that comes into the window, read ahead
         step(std::integral_constant<int, 0>{});
         step(std::integral_constant<int, 1>{});
-#pragma unroll
-        for (int r = 0; r < 3; ++r) {
-            w_tile[r] = w_tile[r + 1];
-            w_mask[r] = w_mask[r + 1];
-        }
-        w_tile[3] = n_tile;
-        w_mask[3] = mask_of(g + 4, n_tile);
+        w_tile[0] = w_tile[1]; w_mask[0] = w_mask[1];
+        w_tile[1] = w_tile[2]; w_mask[1] = w_mask[2];
+        w_tile[2] = entry_tile(g + 3, raw);
+        w_mask[2] = entry_mask(g + 3, raw, w_tile[2]);
     }
+    __syncthreads();                          // the list in LDS has been read: the memory becomes the staging tile
+    // the last 16 keys of the last step (V_B of an odd step sits in ring slot 1)
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int qq = 0; qq < 2; ++qq) oacc[t][qq] = mfma32(vb[1][4 + t], pb[qq][1], oacc[t][qq]);
+    if (rescale_pending) rescale_out();
     }   // nsteps > 0
 
     // ---- epilogue: combine the two key groups of every query, normalise, store through LDS ----
@@ -475,6 +568,7 @@ hipError_t launch_fwd_frag(const void* q, const void* kf, const void* vf, const 
                            int bs_q, int bs_k, int idx_stride, float sm_scale, int dtype, hipStream_t st,
                            const int32_t* q_rows, const int64_t q_st[3], const int64_t o_st[3], int64_t lse_rows,
                            const int32_t* order, uint32_t* queue) {
+    if (idx_stride > kListEntries) return hipErrorInvalidValue;   // the C-ABI layer keeps lists within this limit
     const float qk_scale = sm_scale * kLog2e;
     FragLayout L;
     L.q_rows = q_rows;
@@ -484,16 +578,19 @@ hipError_t launch_fwd_frag(const void* q, const void* kf, const void* vf, const 
     const int resident = resident_wavefronts();
     const dim3 block(64);
     const uint32_t* gate = nullptr;
+#define BSA_FRAG_LAUNCH_T(T, N1, grid, begin, end, ord, que, want)                                                   \
+    hipLaunchKernelGGL((fwd_frag_kernel<T, N1>), grid, block, 0, st, (const T*)q, (const char*)kf, (const char*)vf, idx, \
+                       lens, tile_valid, (T*)o, lse, Sq, Sk, bs_q, bs_k, idx_stride, qk_scale, begin, end, Hn, lse_rows, \
+                       L, ord, que, gate, want)
 #define BSA_FRAG_LAUNCH(grid, begin, end, ord, que, want)                                                             \
     do {                                                                                                               \
-        if (dtype == BSA_BF16)                                                                                         \
-            hipLaunchKernelGGL((fwd_frag_kernel<__bf16>), grid, block, 0, st, (const __bf16*)q, (const char*)kf,       \
-                               (const char*)vf, idx, lens, tile_valid, (__bf16*)o, lse, Sq, Sk, bs_q, bs_k, idx_stride, \
-                               qk_scale, begin, end, Hn, lse_rows, L, ord, que, gate, want);                           \
-        else                                                                                                           \
-            hipLaunchKernelGGL((fwd_frag_kernel<_Float16>), grid, block, 0, st, (const _Float16*)q, (const char*)kf,   \
-                               (const char*)vf, idx, lens, tile_valid, (_Float16*)o, lse, Sq, Sk, bs_q, bs_k,          \
-                               idx_stride, qk_scale, begin, end, Hn, lse_rows, L, ord, que, gate, want);               \
+        if (dtype == BSA_BF16) {                                                                                       \
+            if (bs_k == kTile) BSA_FRAG_LAUNCH_T(__bf16, true, grid, begin, end, ord, que, want);                      \
+            else BSA_FRAG_LAUNCH_T(__bf16, false, grid, begin, end, ord, que, want);                                   \
+        } else {                                                                                                       \
+            if (bs_k == kTile) BSA_FRAG_LAUNCH_T(_Float16, true, grid, begin, end, ord, que, want);                    \
+            else BSA_FRAG_LAUNCH_T(_Float16, false, grid, begin, end, ord, que, want);                                 \
+        }                                                                                                              \
     } while (0)
     if (queue != nullptr) {
         launch_schedule_choice(lens, (int)(Sq / bs_q), bs_q / kTile, total, resident, resident, idx_stride, queue, st);
@@ -507,6 +604,7 @@ hipError_t launch_fwd_frag(const void* q, const void* kf, const void* vf, const 
         BSA_FRAG_LAUNCH(grid, first, end, (const int32_t*)nullptr, (uint32_t*)nullptr, 0u);
     }
 #undef BSA_FRAG_LAUNCH
+#undef BSA_FRAG_LAUNCH_T
     return hipGetLastError();
 }
 
