@@ -29,7 +29,7 @@ int main(int argc, char** argv) {
     p.tq = p.hq = p.wq = p.tk = p.hk = p.wk = 4;
     p.k_sel = 90; p.sm_scale = 0.088388f; p.cdf_threshold = 0.f;
     const size_t ws = workspace_bytes(&p);
-    if (ws < (size_t)100 << 20 || ws > (size_t)1 << 30) return 7;      /* a few hundred MB at 720p */
+    if (ws < (size_t)1 << 30 || ws > (size_t)2 << 30) return 7;        /* k and v in fragment order (1.5 GB) + a few hundred MB at 720p */
     p.D = 96;
     if (workspace_bytes(&p) != 0) return 8;                            /* unsupported head dim: 0 and an error text */
     if (strlen(last_error()) == 0) return 9;

@@ -101,10 +101,10 @@ def test_fwd_3d_plan_and_workspace():
     lib = _capi.load()
     prm = _capi.Bsa3dParams(1, 32, 128, _capi.BSA_BF16, 24, 45, 80, 24, 45, 80, 4, 4, 4, 4, 4, 4, 90, 0.0883883)
     need = lib.bsa_workspace_bytes(C.byref(prm))
-    # q, o, k and v are used where they lie; only the chunks of the padded h edge of k and v
-    # (1/12 of the grid) are copied, plus pooled vectors, the score matrix and the lists
-    edge = 2 * 32 * (92160 // 12) * 128 * 2
-    assert need > edge and need < edge + 300 * 2 ** 20
+    # q and o are used where they lie; k and v are rewritten once, in fragment order, at their padded size;
+    # plus pooled vectors, the score matrix and the lists
+    kv = 2 * 32 * 92160 * 128 * 2
+    assert need > kv and need < kv + 300 * 2 ** 20
     prm32 = _capi.Bsa3dParams(1, 32, 128, _capi.BSA_F32, 24, 45, 80, 24, 45, 80, 4, 4, 4, 4, 4, 4, 90, 0.0883883)
     assert lib.bsa_workspace_bytes(C.byref(prm32)) > 4 * 32 * 92160 * 128 * 4     # fp32: blocked copies of all four
     st = _capi.strides3([32 * 86400 * 128, 86400 * 128, 128])

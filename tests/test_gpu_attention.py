@@ -257,3 +257,39 @@ def test_random_lists_lengths_and_masks(seed):
     fin = torch.isfinite(want_lse)
     assert torch.allclose(lse[fin], want_lse[fin], atol=2e-3)
     assert torch.all(torch.isinf(lse[~fin]) & (lse[~fin] < 0)) and torch.all(o[~fin] == 0)
+
+
+@pytest.mark.parametrize("case", ["scaled", "late", "late_within_bound", "nan_free_zero_keys"])
+def test_thw_kernel_keeps_its_exponentials_finite(case):
+    """The (T,H,W)-order kernel raises its running maximum lazily and rescales its accumulators a quarter of a step
+    after the maximum has moved.  Inputs that drive that path hard: logits scaled far beyond the usual range; a list
+    whose first blocks give tiny logits and whose last blocks give huge ones (the maximum moves late and far); the same
+    with a milder slope; all-zero keys."""
+    bi = I()
+    latent, chunk = (8, 8, 16), (4, 4, 4)
+    S, nb = 1024, 16
+    q, k, v = seeded_qkv(90, 1, 2, S, S, 128, torch.bfloat16)
+    kp = O.rearrange_thw_to_3d_block(k, latent, chunk).float()
+    if case == "scaled":
+        q = (q.float() * 30).bfloat16()
+    elif case in ("late", "late_within_bound"):
+        # keys of the low blocks shrink, keys of the high blocks grow: ascending lists meet the large logits last
+        gain = torch.linspace(-6, 5 if case == "late" else 1.5, nb).exp2().repeat_interleave(64).view(1, 1, -1, 1)
+        k = O.rearrange_3d_block_to_thw((kp * gain).bfloat16(), latent, chunk)
+        q = (q.float() * (6 if case == "late" else 1)).bfloat16()
+    else:
+        k = torch.zeros_like(k)
+    g = torch.Generator().manual_seed(91)
+    idx = torch.stack([torch.randperm(nb, generator=g)[:8].sort().values for _ in range(2 * nb)]).view(1, 2, nb, 8)
+    lens = torch.full((1, 2, nb), 8, dtype=torch.int32)
+    o, lse = bi.attn_fwd_bsa_thw(q.cuda(), k.cuda(), v.cuda(), latent, latent, chunk, chunk, idx.int().cuda(), lens.cuda(),
+                                 return_lse=True)
+    qp = O.rearrange_thw_to_3d_block(q, latent, chunk)
+    kp = O.rearrange_thw_to_3d_block(k, latent, chunk)
+    vp = O.rearrange_thw_to_3d_block(v, latent, chunk)
+    want, want_lse = O.masked_dense_attention(qp, kp, vp, O.block_mask_from_indices(idx, lens, nb), 64, 64, 1 / math.sqrt(128))
+    got = O.rearrange_thw_to_3d_block(o.cpu(), latent, chunk)
+    got_lse = O.rearrange_thw_to_3d_block(lse.cpu().unsqueeze(-1), latent, chunk)[..., 0]
+    assert torch.isfinite(got.float()).all() and torch.isfinite(got_lse).all()
+    close(got, want, torch.bfloat16)
+    assert torch.allclose(got_lse, want_lse, rtol=1e-4, atol=2e-3)
