@@ -482,14 +482,22 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
         raise_max(mx[0], mx[1]);
     };
 
+    // The entry that comes into the window is read from LDS one iteration before it is decoded.  The read is
+    // issued behind everything else of an iteration that waits on the scalar / LDS counter (the rare validity
+    // word), so that no wait for it lands in front of the MFMAs.
+    uint32_t raw = entry_raw(3);
     for (int g = 0; g < ntiles; ++g) {
-        const uint32_t raw = entry_raw(g + 3);                  // the position that comes into the window, read ahead
         step(std::integral_constant<int, 0>{});
         step(std::integral_constant<int, 1>{});
         w_tile[0] = w_tile[1]; w_mask[0] = w_mask[1];
         w_tile[1] = w_tile[2]; w_mask[1] = w_mask[2];
         w_tile[2] = entry_tile(g + 3, raw);
         w_mask[2] = entry_mask(g + 3, raw, w_tile[2]);
+        asm volatile("" : "+s"(w_tile[0]), "+s"(w_tile[1]), "+s"(w_tile[2]));
+        asm volatile("" : "+s"(w_mask[0]), "+s"(w_mask[1]), "+s"(w_mask[2]));
+        __builtin_amdgcn_sched_barrier(0);
+        raw = entry_raw(g + 4);
+        __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();                          // the list in LDS has been read: the memory becomes the staging tile
     // the last 16 keys of the last step (V_B of an odd step sits in ring slot 1)
