@@ -345,7 +345,14 @@ hipError_t prepare_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, cons
         e = launch_permute(q, q_strides, nullptr, nullptr, nullptr, 1, 1, pl.gq, p->D, p->dtype, st, false, w.qrows, nullptr);
     if (e != hipSuccess) return e;
     if (pl.frag) {
-        // pooled means and validity words of k (one read of k), then k and v in fragment order
+        // 64-slot chunks: one pass over k gives its fragment order, its chunk means and the validity words
+        if (pl.gk.chunk() == 64) {
+            e = launch_frag(k, k_strides, w.kp, p->B, p->Hn, pl.gk, p->dtype, false, st, pool ? w.kc : nullptr,
+                            padded_k ? w.valid : nullptr);
+            if (e != hipSuccess) return e;
+            return launch_frag(v, v_strides, w.vp, p->B, p->Hn, pl.gk, p->dtype, true, st);
+        }
+        // larger chunks: pooled means and validity words of k by the pooling pass, then k and v in fragment order
         if (pool || padded_k) {
             if (pool)
                 e = launch_permute(k, k_strides, nullptr, w.kc, padded_k ? w.valid : nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st);

@@ -138,8 +138,10 @@ void launch_schedule_choice(const int32_t* lens, int nbq, int tiles_per_block, i
 
 // K or V of a (T, H, W)-ordered tensor in fragment order (bsa_fwd_frag.hip): dst [B*Hn][padded slots / 64][16 KB],
 // padded slots zero; transpose = false for K, true for V.  bf16 / fp16.
+// For K (transpose = false) of 64-slot chunks the pass can also write the chunk means (pooled, [B*Hn][blocks][128],
+// the bits launch_permute's pooling gives) and the tile validity words; both optional.
 hipError_t launch_frag(const void* src, const int64_t strides[3], void* dst, int B, int Hn, const Grid3& g, int dtype,
-                       bool transpose, hipStream_t st);
+                       bool transpose, hipStream_t st, void* pooled = nullptr, uint64_t* tile_valid = nullptr);
 // The attention kernel on fragment-order K and V.  q_rows (optional): token row of every blocked-order query
 // slot, -1 for padding; q_st / o_st: element strides {batch, head, row}; lse_rows: rows per (batch, head) of lse.
 hipError_t launch_fwd_frag(const void* q, const void* kf, const void* vf, const int32_t* idx, const int32_t* lens,

@@ -48,9 +48,13 @@ constexpr int kListEntries = 4096;    // longest list a work item can walk (its 
 // One workgroup per 64-slot tile of one (batch, head): the 64 rows are gathered from (T, H, W) order
 // (padded slots: zeros) into LDS and written out as 16 fragments of 1 KB.  K (TRANSPOSE = false) moves
 // 16-byte pieces; V (TRANSPOSE = true) gathers 8 keys of one d per piece.
+// For K of 64-slot chunks the same pass can also produce what the pooling pass of bsa_permute.hip would: the chunk
+// mean (pooled, in the storage type given by is_bf16; the summation order of permute_kernel is reproduced, so the
+// two routes give the same bits) and the validity word of the tile.
 template <typename T, bool TRANSPOSE>
 __global__ __launch_bounds__(256) void frag_kernel(const T* __restrict__ src, int64_t sB, int64_t sH, int64_t sS,
-                                                   char* __restrict__ dst, Grid3 g, int Hn) {
+                                                   char* __restrict__ dst, Grid3 g, int Hn, T* __restrict__ pooled,
+                                                   uint64_t* __restrict__ tile_valid, int is_bf16) {
     // rows padded to 264 B: the transposing reads below walk down a column
     constexpr int kPitch = kD + 4;
     __shared__ __attribute__((aligned(16))) T tile[kTile * kPitch];
@@ -71,6 +75,44 @@ __global__ __launch_bounds__(256) void frag_kernel(const T* __restrict__ src, in
             x = *reinterpret_cast<const uint4*>(sbase + (((int64_t)tt * g.H + hh) * g.W + ww) * sS + c16 * 8);
         val[i][0] = make_uint2(x.x, x.y);
         val[i][1] = make_uint2(x.z, x.w);
+    }
+    if (!TRANSPOSE && tile_valid != nullptr && bh == 0 && threadIdx.x < 64) {
+        const int r = sub * kTile + threadIdx.x;
+        const int wi = r % g.w, hi = (r / g.w) % g.h, ti = r / (g.w * g.h);
+        const uint64_t m = __ballot(nt * g.t + ti < g.T && nh * g.h + hi < g.H && nw * g.w + wi < g.W);
+        if (threadIdx.x == 0) tile_valid[blockIdx.x] = m;
+    }
+    if (!TRANSPOSE && pooled != nullptr) {
+        // permute_kernel's order: a thread sums its rows rg, rg + 16, rg + 32, rg + 48 per element, then the 16
+        // partial sums of a column are added in ascending rg; mean = sum * (1 / 64), rounded once
+        __shared__ float red[16 * kD];
+        float acc[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w[4] = {val[i][0].x, val[i][0].y, val[i][1].x, val[i][1].y};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float lo, hi;
+                if (is_bf16) { lo = __uint_as_float(w[e] << 16); hi = __uint_as_float(w[e] & 0xffff0000u); }
+                else { lo = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[e] & 0xffffu)); hi = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[e] >> 16)); }
+                acc[2 * e] += lo;
+                acc[2 * e + 1] += hi;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) red[rg * kD + c16 * 8 + e] = acc[e];
+        __syncthreads();
+        if (threadIdx.x < kD) {
+            float sum = 0.f;
+            for (int gq = 0; gq < 16; ++gq) sum += red[gq * kD + threadIdx.x];
+            sum *= 1.0f / 64.0f;
+            uint16_t bits;
+            if (is_bf16) bits = __builtin_bit_cast(uint16_t, (__bf16)sum);
+            else bits = __builtin_bit_cast(uint16_t, (_Float16)sum);
+            reinterpret_cast<uint16_t*>(pooled)[((int64_t)bh * gridDim.x + blockIdx.x) * kD + threadIdx.x] = bits;
+        }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -617,16 +659,15 @@ hipError_t launch_fwd_frag(const void* q, const void* kf, const void* vf, const 
 }
 
 hipError_t launch_frag(const void* src, const int64_t st3[3], void* dst, int B, int Hn, const Grid3& g, int dtype,
-                       bool transpose, hipStream_t st) {
+                       bool transpose, hipStream_t st, void* pooled, uint64_t* tile_valid) {
     const dim3 grid((unsigned)(g.blocks() * (g.chunk() / kTile)), (unsigned)(B * Hn)), block(256);
     // 16-bit types move as raw bits
     if (transpose)
         hipLaunchKernelGGL((frag_kernel<uint16_t, true>), grid, block, 0, st, (const uint16_t*)src, st3[0], st3[1], st3[2],
-                           (char*)dst, g, Hn);
+                           (char*)dst, g, Hn, (uint16_t*)nullptr, (uint64_t*)nullptr, 0);
     else
         hipLaunchKernelGGL((frag_kernel<uint16_t, false>), grid, block, 0, st, (const uint16_t*)src, st3[0], st3[1], st3[2],
-                           (char*)dst, g, Hn);
-    (void)dtype;
+                           (char*)dst, g, Hn, (uint16_t*)pooled, tile_valid, dtype == BSA_BF16 ? 1 : 0);
     return hipGetLastError();
 }
 
