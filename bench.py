@@ -34,10 +34,32 @@ WORKLOADS = {
     "c2": ((24, 30, 52), 0.9375, 1, False, "480p layer: 32 heads x 128, grid 24x30x52 (37440 tokens), density 1/16"),
     "c3": ((24, 45, 80), 0.9375, 2, True, "720p layer: 32 heads x 128, grid 24x45x80 (86400 tokens), density 1/16"),
 }
-# Bytes that leave L2 per layer in the attention kernel (all of its launches), from rocprofv3 --pmc
-# FETCH_SIZE (x2) and WRITE_SIZE (x1) as recorded in profiles/bsa_operator_c3_720p.md: 45 launches
-# x (1286.6 MB + 15.7 MB).  Re-measure after kernel changes.
-ATTENTION_TRAFFIC_BYTES = {"c3": 45 * (1286.6e6 + 15.7e6)}
+ATTENTION_KERNEL = "fwd_frag_kernel<bf16> (all launches of one layer)"
+ATTENTION_SOURCE = os.path.join(ROOT, "longcat-video_amd", "csrc", "bsa_fwd_frag.hip")
+
+
+def source_sha16(path=ATTENTION_SOURCE):
+    import hashlib
+    with open(path, "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def recorded_traffic(workload):
+    """HBM-side bytes per layer of the attention kernel (rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled as the profile
+    summary says), as recorded in profiles/bsa_operator_<workload>_*.md on a line
+    `traffic_record: {"workload": ..., "source_sha16": ..., "bytes_per_layer": ...}` - or None when there is no
+    record for this workload or the kernel source has changed since it was taken (a stale figure is not reported)."""
+    import glob
+    for path in glob.glob(os.path.join(ROOT, "profiles", "bsa_operator_%s_*.md" % workload)):
+        with open(path) as f:
+            for line in f:
+                if line.startswith("traffic_record:"):
+                    rec = json.loads(line[len("traffic_record:"):])
+                    if rec.get("workload") == workload and rec.get("source_sha16") == source_sha16():
+                        return float(rec["bytes_per_layer"])
+    return None
+
+
 CHUNK = (4, 4, 4)
 HEADS, D = 32, 128
 
@@ -86,32 +108,23 @@ def time_events(torch, fn, steps, warmup):
     return start.elapsed_time(stop) / steps      # ms per call
 
 
-def cpu_baseline(torch, latent, sparsity, seed, rms, budget_s):
-    """The oracle's masked-dense evaluation of the same layer on the host cores:
-    pool -> score -> top-k -> block mask -> fp32 softmax(QK^T/sqrt(D) + mask)V.
-    One head is prepared in full; query blocks are evaluated until the time
-    budget is spent, then scaled linearly to all heads and query blocks."""
+def cpu_attention_sample(torch, q, k, v, latent_q, latent_k, sparsity, budget_s):
+    """One head of one operator call on the host cores through the oracle: permute, pool, score, top-k in full,
+    then masked-dense fp32 attention on as many query blocks as the time budget allows.  q [1,1,Sq,D], k, v
+    [1,1,Sk,D].  Returns (seconds for the whole head, extrapolated linearly over its query blocks; set-up seconds;
+    attention seconds spent; query blocks evaluated; query blocks in all; blocks kept per row)."""
     from oracle import bsa_oracle as O
-    cores = os.cpu_count() or 1
-    torch.set_num_threads(cores)
-    S = latent[0] * latent[1] * latent[2]
-    g = torch.Generator().manual_seed(seed)
-    q, k, v = (torch.randn(1, 1, S, D, generator=g) for _ in range(3))
-    if rms:
-        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + 1e-6)
-        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + 1e-6)
-    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
     t0 = time.perf_counter()
-    qp = O.rearrange_thw_to_3d_block(q, latent, CHUNK)
-    kp = O.rearrange_thw_to_3d_block(k, latent, CHUNK)
-    vp = O.rearrange_thw_to_3d_block(v, latent, CHUNK)
+    qp = O.rearrange_thw_to_3d_block(q, latent_q, CHUNK)
+    kp = O.rearrange_thw_to_3d_block(k, latent_k, CHUNK)
+    vp = O.rearrange_thw_to_3d_block(v, latent_k, CHUNK)
     score = O.cal_score(O.mean_pooling_compression(qp, 64), O.mean_pooling_compression(kp, 64))
     nbq, nbk = score.shape[-2:]
     k_sel = O.num_selected(sparsity, nbk)
     idx, lens = O.select_topk(score, k_sel)
     mask = O.block_mask_from_indices(idx, lens, nbk)
-    kvalid = torch.from_numpy(O.slot_validity(latent, CHUNK))
-    t_head_setup = time.perf_counter() - t0
+    kvalid = torch.from_numpy(O.slot_validity(latent_k, CHUNK))
+    t_setup = time.perf_counter() - t0
     done, t_attn = 0, 0.0
     O.masked_dense_attention(qp, kp, vp, mask, 64, 64, 1 / math.sqrt(D), key_valid=kvalid, q_blocks=[0])   # warm-up
     while done < nbq and t_attn < budget_s:
@@ -120,15 +133,45 @@ def cpu_baseline(torch, latent, sparsity, seed, rms, budget_s):
         O.masked_dense_attention(qp, kp, vp, mask, 64, 64, 1 / math.sqrt(D), key_valid=kvalid, q_blocks=blocks)
         t_attn += time.perf_counter() - t0
         done += len(blocks)
-    layer_s = HEADS * (t_head_setup + t_attn * nbq / done)
+    return t_setup + t_attn * nbq / done, t_setup, t_attn, done, nbq, k_sel
+
+
+def host_inputs(torch, S, seed, rms):
+    """One head of q, k, v drawn on the host: the same distribution as the GPU leg's inputs, a separate draw."""
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = (torch.randn(1, 1, S, D, generator=g) for _ in range(3))
+    if rms:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + 1e-6)
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + 1e-6)
+    return q.bfloat16(), k.bfloat16(), v.bfloat16()
+
+
+def cpu_baseline(torch, latent, sparsity, seed, rms, budget_s):
+    """The oracle's masked-dense evaluation of the same layer on the host cores:
+    pool -> score -> top-k -> block mask -> fp32 softmax(QK^T/sqrt(D) + mask)V.
+    One head is prepared in full; query blocks are evaluated until the time
+    budget is spent, then scaled linearly to all heads and query blocks."""
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    q, k, v = host_inputs(torch, latent[0] * latent[1] * latent[2], seed, rms)
+    head_s, t_setup, t_attn, done, nbq, k_sel = cpu_attention_sample(torch, q, k, v, latent, latent, sparsity, budget_s)
+    layer_s = HEADS * head_s
     flop = HEADS * nbq * k_sel * 4 * 64 * 64 * D
     return {
-        "value": flop / layer_s / 1e12, "unit": "TFLOP/s (sparse-actual)", "cores": cores, "kind": "port",
-        "ms_per_layer": layer_s * 1e3,
-        "sample": "1 of %d heads: permute+pool+score+top-k in full (%.2f s), masked-dense fp32 attention on %d of %d "
-                  "query blocks against all keys (%.2f s); scaled linearly to %d heads x %d query blocks"
-                  % (HEADS, t_head_setup, done, nbq, t_attn, HEADS, nbq),
+        "value": round(flop / layer_s / 1e12, 5), "unit": "TFLOP/s (sparse-actual)", "cores": cores, "kind": "port",
+        "ms_per_layer": round(layer_s * 1e3, 1),
+        "sample": "1 of %d heads, inputs drawn on the host from the same distribution as the GPU leg's (a separate "
+                  "draw, not the same tensors): permute+pool+score+top-k in full (%.2f s), masked-dense fp32 attention "
+                  "on %d of %d query blocks against all keys (%.2f s); scaled linearly to %d heads x %d query blocks"
+                  % (HEADS, t_setup, done, nbq, t_attn, HEADS, nbq),
     }
+
+
+def attention_roofline(flop, ms, workload, coherent=False):
+    tflops = flop / (ms * 1e-3) / 1e12
+    return {"kernel": ATTENTION_KERNEL, "bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s", "frac": round(tflops / PEAK_BF16_TFLOPS, 4),
+            "traffic": None if coherent else recorded_traffic(workload), "ms": round(ms, 4)}
 
 
 def run_c4(torch, args):
@@ -139,10 +182,12 @@ def run_c4(torch, args):
     S, n = T * Hh * W, cond * Hh * W
     q, k, v = make_inputs(torch, (T, Hh, W), 3, False)
     out = torch.empty(1, S, HEADS, D, dtype=torch.bfloat16, device="cuda").permute(0, 2, 1, 3)
+    calls = [((q[:, :, :n], k[:, :, :n], v[:, :, :n]), (cond, Hh, W), (cond, Hh, W), out[:, :, :n]),
+             ((q[:, :, n:], k, v), (T - cond, Hh, W), (T, Hh, W), out[:, :, n:])]
 
     def step():
-        I._bsa_3d(q[:, :, :n], k[:, :, :n], v[:, :, :n], (cond, Hh, W), (cond, Hh, W), 0.875, CHUNK, CHUNK, out=out[:, :, :n])
-        I._bsa_3d(q[:, :, n:], k, v, (T - cond, Hh, W), (T, Hh, W), 0.875, CHUNK, CHUNK, out=out[:, :, n:])
+        for (a, b, c), lq, lk, o in calls:
+            I._bsa_3d(a, b, c, lq, lk, 0.875, CHUNK, CHUNK, out=o)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -151,16 +196,44 @@ def run_c4(torch, args):
         step()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    want = out.clone()
+    # the attention kernel of both calls on its own, with the operator's lists
+    ms_attn = 0.0
+    for (a, b, c), lq, lk, o in calls:
+        _, idx, lens, _ = I._bsa_3d(a, b, c, lq, lk, 0.875, CHUNK, CHUNK, want_selection=True)
+        idx = idx.sort(dim=-1).values.contiguous()
+        attend = I.ThwAttention(b, c, lq, lk, CHUNK, CHUNK)
+        ms_attn += time_events(torch, lambda: attend(a, idx, lens, out=o), max(args.steps, 5), 2)
+        del attend
+    assert torch.equal(out, want), "the separately timed attention kernel must reproduce the operator's output"
     pairs = HEADS * (312 * 39 + 936 * 156)
     flop = pairs * 4 * 64 * 64 * D
-    print(json.dumps({
+    result = {
         "metric": "BSA fwd ms/layer + sparse TFLOPS, long-video continuation (cond/noise split)", "value": round(flop / ms / 1e9, 2),
         "unit": "TFLOP/s (sparse-actual, both operator calls)", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic N(0,1) q/k/v, seeded on the GPU",
         "config": {"workload": "c4: 32 heads x 128, grid 48x30x52 (74880 tokens), 12 conditioning frames, density 1/8",
                    "block_pairs": pairs},
-        "pct_of_bf16_peak_whole_operator": round(100 * flop / ms / 1e9 / PEAK_BF16_TFLOPS, 2)}))
+        "pct_of_bf16_peak_whole_operator": round(100 * flop / ms / 1e9 / PEAK_BF16_TFLOPS, 2),
+        "kernels_ms": {"attention (both calls)": round(ms_attn, 4), "everything else (step - attention)": round(ms - ms_attn, 4)},
+        "roofline": attention_roofline(flop, ms_attn, "c4")}
+    if not args.no_cpu_baseline:
+        cores = os.cpu_count() or 1
+        torch.set_num_threads(cores)
+        hq, hk, hv = host_inputs(torch, S, 3, False)
+        half = args.cpu_seconds / 2
+        a = cpu_attention_sample(torch, hq[:, :, :n], hk[:, :, :n], hv[:, :, :n], (cond, Hh, W), (cond, Hh, W), 0.875, half)
+        b = cpu_attention_sample(torch, hq[:, :, n:], hk, hv, (T - cond, Hh, W), (T, Hh, W), 0.875, half)
+        layer_s = HEADS * (a[0] + b[0])
+        result["cpu_baseline"] = {
+            "value": round(flop / layer_s / 1e12, 5), "unit": "TFLOP/s (sparse-actual)", "cores": cores, "kind": "port",
+            "ms_per_layer": round(layer_s * 1e3, 1),
+            "sample": "1 of %d heads, inputs drawn on the host from the same distribution (a separate draw): both operator "
+                      "calls with permute+pool+score+top-k in full (%.2f s + %.2f s) and masked-dense fp32 attention on %d of %d "
+                      "conditioning and %d of %d noise query blocks (%.2f s + %.2f s); scaled linearly to all query blocks and %d heads"
+                      % (HEADS, a[1], b[1], a[3], a[4], b[3], b[4], a[2], b[2], HEADS)}
+    print(json.dumps(result))
 
 
 def run_c5(torch, args):
@@ -191,17 +264,80 @@ def run_c5(torch, args):
     assert torch.isfinite(y.float()).all()
     bsa_flop = HEADS * 1440 * 90 * 4 * 64 * 64 * D
     gemm_flop = 2 * N * C * 3 * C + 2 * N * C * C
+    # ---- the module's kernels on their own, on the module's own tensors
     ms_qkv = time_events(torch, lambda: M.linear_bf16(x, attn.qkv.weight, attn.qkv.bias), 5, 2)
-    print(json.dumps({
+    ms_proj = time_events(torch, lambda: M.linear_bf16(x, attn.proj.weight, attn.proj.bias, residual=x), 5, 2)
+    qs, ks, vs = attn._project_qkv(M.rms_norm(x, w_pre, 1e-6))
+    new = lambda: torch.empty(1, HEADS, N, D, dtype=x.dtype, device=x.device)
+    qd, kd, vd = new(), new(), new()
+    ms_norm_rope = time_events(torch, lambda: M.norm_rope(qs, qd, attn.q_norm.weight, latent), 5, 2)
+    M.norm_rope(ks, kd, attn.k_norm.weight, latent)
+    M.norm_rope(vs, vd)
+    from longcat_video_amd.block_sparse_attention import bsa_interface as I
+    _, idx, lens, _ = I._bsa_3d(qd, kd, vd, latent, latent, 0.9375, CHUNK, CHUNK, want_selection=True)
+    idx = idx.sort(dim=-1).values.contiguous()
+    attend = I.ThwAttention(kd, vd, latent, latent, CHUNK, CHUNK)
+    o_buf = torch.empty(1, N, HEADS, D, dtype=x.dtype, device=x.device).permute(0, 2, 1, 3)
+    ms_attn = time_events(torch, lambda: attend(qd, idx, lens, out=o_buf), 5, 2)
+    del attend
+    qkv_tflops = 2 * N * C * 3 * C / ms_qkv / 1e9
+    norm_rope_gbs = 2 * N * C * 2 / ms_norm_rope / 1e6          # one tensor: 708 MB read + 708 MB written
+    result = {
         "metric": "attention sub-chain of a DiT block, ms/layer + TFLOPS (GEMMs + sparse-actual attention)",
         "value": round((bsa_flop + gemm_flop) / ms / 1e9, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic N(0,1) activations, N(0,0.02) weights, zero biases, unit norm weights",
         "config": {"workload": "c5: x [1, 86400, 4096] bf16, 32 heads x 128, grid 24x45x80, density 1/16"},
-        "qkv_gemm_ms": round(ms_qkv, 4), "qkv_gemm_tflops": round(2 * N * C * 3 * C / ms_qkv / 1e9, 1),
+        "kernels_ms": {"attention": round(ms_attn, 4), "qkv_gemm": round(ms_qkv, 4), "proj_gemm_with_residual": round(ms_proj, 4),
+                       "norm_rope_move_one_tensor": round(ms_norm_rope, 4)},
+        "qkv_gemm_ms": round(ms_qkv, 4), "qkv_gemm_tflops": round(qkv_tflops, 1),
         "gemm_tuning": {"qkv": {"algorithms_timed": tuned[0][0], "default_ms": round(tuned[0][1], 4), "chosen_ms": round(tuned[0][2], 4)},
                         "proj": {"algorithms_timed": tuned[1][0], "default_ms": round(tuned[1][1], 4), "chosen_ms": round(tuned[1][2], 4)}},
-        "pct_of_bf16_peak": round(100 * (bsa_flop + gemm_flop) / ms / 1e9 / PEAK_BF16_TFLOPS, 2)}))
+        "pct_of_bf16_peak": round(100 * (bsa_flop + gemm_flop) / ms / 1e9 / PEAK_BF16_TFLOPS, 2),
+        # the dominant kernel of the module is still the attention kernel; the other two kinds of kernel beside it
+        "roofline": attention_roofline(bsa_flop, ms_attn, "c5"),
+        "roofline_qkv_gemm": {"kernel": "hipBLASLt bf16 GEMM [86400,4096]x[4096,12288]^T + bias (library kernel)", "bound": "mfma",
+                              "achieved": round(qkv_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                              "frac": round(qkv_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None, "ms": round(ms_qkv, 4)},
+        "roofline_norm_rope": {"kernel": "norm_rope_kernel<bf16> (per-head RMSNorm + 3-D RoPE + move of one tensor)", "bound": "hbm",
+                               "achieved": round(norm_rope_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                               "frac": round(norm_rope_gbs / PEAK_HBM_GBS, 4), "traffic": None, "ms": round(ms_norm_rope, 4)},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline_c5(torch, latent, N, C, args.cpu_seconds, bsa_flop + gemm_flop)
+    print(json.dumps(result))
+
+
+def cpu_baseline_c5(torch, latent, N, C, budget_s, flop):
+    """The module on the host cores through the oracle, on a bounded sample: both projections in fp32 on a slice of the
+    tokens (with the pre-norm, the per-head norm and the rotation of that slice), and the attention of one head as in
+    cpu_baseline; each part scaled linearly to the layer."""
+    from oracle import bsa_oracle as O
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(4)
+    n_tok = 1024
+    x = torch.randn(1, n_tok, C, generator=g).bfloat16()
+    w_qkv = (torch.randn(3 * C, C, generator=g) * 0.02).bfloat16()
+    w_proj = (torch.randn(C, C, generator=g) * 0.02).bfloat16()
+    t0 = time.perf_counter()
+    y = O.rms_norm_fp32(x, torch.ones(C, dtype=torch.bfloat16))
+    qkv = (y.reshape(n_tok, C).float() @ w_qkv.float().t()).bfloat16().view(1, n_tok, 3, HEADS, D).permute(2, 0, 3, 1, 4)
+    qh, kh = O.rms_norm_fp32(qkv[0], torch.ones(D, dtype=torch.bfloat16)), O.rms_norm_fp32(qkv[1], torch.ones(D, dtype=torch.bfloat16))
+    ang = O.rope_3d_angles(latent, D)[:n_tok]
+    qh, kh = O.rope_3d_apply(qh, ang), O.rope_3d_apply(kh, ang)
+    o = qkv[2].transpose(1, 2).reshape(n_tok, C)
+    _ = (o.float() @ w_proj.float().t() + x.reshape(n_tok, C).float()).bfloat16()
+    t_glue = time.perf_counter() - t0
+    hq, hk, hv = host_inputs(torch, N, 2, True)
+    head_s, t_setup, t_attn, done, nbq, _ = cpu_attention_sample(torch, hq, hk, hv, latent, latent, 0.9375, budget_s)
+    layer_s = t_glue * N / n_tok + HEADS * head_s
+    return {"value": round(flop / layer_s / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "ms_per_layer": round(layer_s * 1e3, 1),
+            "sample": "inputs drawn on the host from the same distributions (separate draws): pre-norm, both projections in fp32, "
+                      "per-head norm and rotation on %d of %d tokens (%.2f s, scaled linearly); attention of 1 of %d heads with "
+                      "permute+pool+score+top-k in full (%.2f s) and masked-dense fp32 attention on %d of %d query blocks (%.2f s), "
+                      "scaled linearly to all query blocks and heads" % (n_tok, N, t_glue, HEADS, t_setup, done, nbq, t_attn)}
 
 
 def main():
@@ -210,8 +346,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4", "c5"],
-                    help="c3 is the headline (default); c2 the same operator at 480p; c4 and c5 print a reduced line "
-                         "for the cond/noise split and for the attention module")
+                    help="c3 is the headline (default); c2 the same operator at 480p; c4 the cond/noise split of a long "
+                         "video; c5 the attention module around the operator")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the CPU baseline's attention sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm-tuning", action="store_true", help="c5: leave the GEMM algorithm choice to hipBLASLt's first proposal")
@@ -295,18 +431,14 @@ def main():
         "pct_of_bf16_peak_whole_operator": round(100 * tflops_step / PEAK_BF16_TFLOPS, 2),
         "dense_equivalent_tflops": round(dense_flop / (ms_step * 1e-3) / 1e12, 1),
         "kernels_ms": {"attention": round(ms_attn, 4), "score_topk": round(ms_select, 4),
-                       "pool_q_k_and_edge_copies (step - attention - score_topk)": round(ms_step - ms_attn - ms_select, 4)},
+                       "pool_q_and_fragment_order_k_v (step - attention - score_topk)": round(ms_step - ms_attn - ms_select, 4)},
         "standalone_ms": {"permute_pool_one_tensor": round(ms_permute, 4), "unpermute": round(ms_unpermute, 4)},
         "permute_gbs": round(permute_bytes / (ms_permute * 1e-3) / 1e9, 1),
-        "roofline": {"kernel": "fwd_mfma_kernel<bf16> (all launches of one layer)", "bound": "mfma", "achieved": round(tflops_attn, 2),
-                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops_attn / PEAK_BF16_TFLOPS, 4),
-                     "traffic": None if coherent else ATTENTION_TRAFFIC_BYTES.get(args.workload), "ms": round(ms_attn, 4)},
+        "roofline": attention_roofline(flop, ms_attn, args.workload, coherent),
     }
     del o
     if not args.no_cpu_baseline and not coherent:
         result["cpu_baseline"] = cpu_baseline(torch, latent, sparsity, seed, rms, args.cpu_seconds)
-        result["cpu_baseline"]["value"] = round(result["cpu_baseline"]["value"], 5)
-        result["cpu_baseline"]["ms_per_layer"] = round(result["cpu_baseline"]["ms_per_layer"], 1)
     print(json.dumps(result))
 
 
