@@ -35,13 +35,17 @@ WORKLOADS = {
     "c3": ((24, 45, 80), 0.9375, 2, True, "720p layer: 32 heads x 128, grid 24x45x80 (86400 tokens), density 1/16"),
 }
 ATTENTION_KERNEL = "fwd_frag_kernel<bf16> (all launches of one layer)"
-ATTENTION_SOURCE = os.path.join(ROOT, "longcat-video_amd", "csrc", "bsa_fwd_frag.hip")
+# what the attention kernel's traffic depends on: the kernel itself and the visiting order of the lists it walks
+ATTENTION_SOURCES = [os.path.join(ROOT, "longcat-video_amd", "csrc", f) for f in ("bsa_fwd_frag.hip", "bsa_select.hip")]
 
 
-def source_sha16(path=ATTENTION_SOURCE):
+def source_sha16(paths=ATTENTION_SOURCES):
     import hashlib
-    with open(path, "rb") as f:
-        return hashlib.sha256(f.read()).hexdigest()[:16]
+    h = hashlib.sha256()
+    for path in paths:
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def recorded_traffic(workload):
@@ -62,6 +66,15 @@ def recorded_traffic(workload):
 
 CHUNK = (4, 4, 4)
 HEADS, D = 32, 128
+
+
+def kv_blocks(latent):
+    return math.prod(-(-n // c) for n, c in zip(latent, CHUNK))
+
+
+def operator_lists(I, idx_score_order, lens, latent_k):
+    """The lists as the operator hands them to its attention kernel: ascending block order, then its visiting order."""
+    return I.visit_order(idx_score_order.sort(dim=-1).values.int().contiguous(), lens, kv_blocks(latent_k))
 
 
 def make_inputs(torch, latent, seed, rms):
@@ -201,7 +214,7 @@ def run_c4(torch, args):
     ms_attn = 0.0
     for (a, b, c), lq, lk, o in calls:
         _, idx, lens, _ = I._bsa_3d(a, b, c, lq, lk, 0.875, CHUNK, CHUNK, want_selection=True)
-        idx = idx.sort(dim=-1).values.contiguous()
+        idx = operator_lists(I, idx, lens, lk)
         attend = I.ThwAttention(b, c, lq, lk, CHUNK, CHUNK)
         ms_attn += time_events(torch, lambda: attend(a, idx, lens, out=o), max(args.steps, 5), 2)
         del attend
@@ -275,7 +288,7 @@ def run_c5(torch, args):
     M.norm_rope(vs, vd)
     from longcat_video_amd.block_sparse_attention import bsa_interface as I
     _, idx, lens, _ = I._bsa_3d(qd, kd, vd, latent, latent, 0.9375, CHUNK, CHUNK, want_selection=True)
-    idx = idx.sort(dim=-1).values.contiguous()
+    idx = operator_lists(I, idx, lens, latent)
     attend = I.ThwAttention(kd, vd, latent, latent, CHUNK, CHUNK)
     o_buf = torch.empty(1, N, HEADS, D, dtype=x.dtype, device=x.device).permute(0, 2, 1, 3)
     ms_attn = time_events(torch, lambda: attend(qd, idx, lens, out=o_buf), 5, 2)
@@ -384,10 +397,10 @@ def main():
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
     # ---- per-kernel timing with events on the launch stream ----
-    # the attention kernel exactly as the operator runs it: same lists (ascending block order), same
+    # the attention kernel exactly as the operator runs it: same lists in the same visiting order, same
     # THW-order addressing, workspace prepared once outside the timed region
     _, idx_score, lens, _ = I._bsa_3d(q, k, v, latent, latent, sparsity, CHUNK, CHUNK, want_selection=True)
-    idx = idx_score.sort(dim=-1).values.contiguous()
+    idx = operator_lists(I, idx_score, lens, latent)
     del idx_score
     nbq, k_sel = idx.shape[2], idx.shape[3]
     ksteps, kwarm = max(args.steps, 5), max(min(args.warmup, 3), 1)

@@ -139,6 +139,23 @@ int bsa_topk_from_score(const void* score, int32_t* idx_out, int32_t* idx_sorted
                         int B, int Hn, int nbq, int nbk, int k_sel, int dtype, void* stream);
 
 /*
+ * The order in which bsa_fwd_3d's attention kernel visits each query block's selected KV blocks.  No
+ * counterpart in the reference: its kernel visits the blocks in list order (vmask:249-285), and softmax
+ * attention depends on that order only through floating-point rounding, so the engine chooses the order that
+ * keeps the query tiles running side by side at the same place of the KV sequence (they then share K/V tiles
+ * in the L2 cache).  The attention entry points (bsa_fwd, bsa_fwd_thw) visit a caller's list in the order it
+ * is given; this entry point gives callers that build their own lists the operator's order.
+ *
+ *   idx_sorted [rows, idx_stride] i32, lens[row] blocks in ascending order per row; idx_out the same shape
+ *   (may be idx_sorted itself); nbk KV blocks in the sequence.  Slot groups of 8: group g takes the blocks b
+ *   with g == min(b*n/(nbk*8), groups-1), n = lens[row], up to its number of slots; the blocks over that
+ *   number fill the slots left empty, both in ascending order; every group's slots end in ascending block
+ *   order.  Rows of at most 8 blocks stay as they are.  idx_stride <= 4096.
+ */
+int bsa_visit_order(const int32_t* idx_sorted, const int32_t* lens, int32_t* idx_out, int64_t rows, int nbk,
+                    int idx_stride, void* stream);
+
+/*
  * R5 + R6.  Block-sparse flash-attention forward over blocked-order tensors.
  * Replaces attn_fwd_bsa_varlen_triton (bsa:290-341) and the kernel
  * _attn_fwd_bsa_varlen_align (vmask:172-285).

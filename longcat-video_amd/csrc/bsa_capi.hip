@@ -144,6 +144,16 @@ int bsa_topk_from_score(const void* score, int32_t* idx_out, int32_t* idx_sorted
     return e == hipSuccess ? BSA_OK : hip_fail(e, "top-k launch");
 }
 
+int bsa_visit_order(const int32_t* idx_sorted, const int32_t* lens, int32_t* idx_out, int64_t rows, int nbk,
+                    int idx_stride, void* stream) {
+    if (!idx_sorted || !lens || !idx_out) return set_error(BSA_ERR_BAD_ARG, "visit_order: null pointer");
+    if (rows < 0 || rows > 0x7fffffff || nbk <= 0 || idx_stride <= 0 || idx_stride > 4096)
+        return set_error(BSA_ERR_BAD_ARG, "visit_order: rows in [0, 2^31), nbk > 0 and 0 < idx_stride <= 4096 wanted");
+    const hipError_t e = launch_pace_order(idx_sorted, idx_out, lens, rows, nbk, idx_stride, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "visit order");
+    return BSA_OK;
+}
+
 int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32_t* idx_sorted_out, int32_t* lens_out,
                    void* score_out, int B, int Hn, int nbq, int nbk, int D, int k_sel, int dtype, void* stream) {
     if (!q_cmp || !k_cmp || !lens_out || (!idx_out && !idx_sorted_out)) return set_error(BSA_ERR_BAD_ARG, "score_topk: null pointer");
@@ -478,8 +488,9 @@ int fwd_3d_impl(const Plan& pl, const bsa_3d_params* p, const void* q, const int
         BSA_HIP(launch_permute(v, v_strides, w.vp, nullptr, nullptr, p->B, p->Hn, pl.gk, p->D, p->dtype, st), "permute v");
     }
     BSA_HIP(launch_score(w.qc, w.kc, w.score, p->B * p->Hn, pl.nbq, pl.nbk, p->D, p->dtype, st), "score");
-    // the attention kernel walks each list in ascending block order (L2 locality); the score
-    // order is only produced when the caller asks for the selection
+    // the lists the attention kernel walks come out in ascending block order and, for the fragment-order
+    // kernel, are then put in its visiting order (L2 locality); the score order is only produced when the
+    // caller asks for the selection
     const int64_t sel_rows = (int64_t)p->B * p->Hn * pl.nbq;
     if (pl.cdf) {
         BSA_HIP(launch_cdf_count(w.score, w.lens, sel_rows, pl.nbk, p->cdf_threshold, p->sm_scale, p->k_sel < pl.sel_width ? p->k_sel : pl.sel_width,
@@ -488,6 +499,8 @@ int fwd_3d_impl(const Plan& pl, const bsa_3d_params* p, const void* q, const int
     } else {
         BSA_HIP(launch_topk(w.score, idx_out ? w.idx : nullptr, w.idx_sorted, w.lens, sel_rows, pl.nbk, p->k_sel, p->dtype, st), "top-k");
     }
+    if (pl.frag && pl.sel_width > 0)
+        BSA_HIP(launch_pace_order(w.idx_sorted, w.idx_sorted, w.lens, sel_rows, pl.nbk, pl.sel_width, st), "visit order");
     if (pl.direct_qo) {
         // lists of unequal length: one launch whose workgroups draw the items, longest lists first
         if (pl.cdf)

@@ -124,6 +124,10 @@ hipError_t launch_fwd(const void* q, const void* k, const void* v, const int32_t
                       float sm_scale, int dtype, hipStream_t st, const FwdLayout* layout = nullptr,
                       int64_t layout_lse_rows = 0, int64_t layout_edge_bytes = 0, const int32_t* order = nullptr,
                       uint32_t* queue = nullptr);
+// Rewrites every row's ascending list of KV blocks into the order the attention kernel visits them in (see
+// pace_order_kernel).  rows of `stride` entries, lens[row] of them in use; in == out allowed; stride <= 5000.
+hipError_t launch_pace_order(const int32_t* in, int32_t* out, const int32_t* lens, int64_t rows, int nbk, int stride,
+                             hipStream_t st);
 // order: for every (batch, head) its 64-row query tiles by descending list length (lens is per query
 // block of tiles_per_block tiles, clamped to [0, max_len]); with `order` and a two-word `queue`
 // launch_fwd enqueues the 16-bit kernel both as rounds and as one launch whose workgroups draw items

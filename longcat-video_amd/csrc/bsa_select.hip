@@ -226,6 +226,86 @@ __global__ __launch_bounds__(256) void topk_kernel(const S* __restrict__ score,
     }
 }
 
+// ---------------------------------------------------------------- visiting order
+// The order in which the attention kernel visits one row's selected KV blocks.  Softmax attention does not
+// depend on it beyond rounding, so it is chosen for the L2 cache: the query tiles that run side by side walk
+// the KV sequence together when slot s of every list holds a block near s/n of the sequence, and then share
+// the K/V tiles they have in common while those are still cached.  A plain ascending list drifts from that
+// pace wherever it holds more or fewer blocks than the average in a stretch of the sequence.
+//
+// One wavefront per row.  in: n = lens[row] blocks in ascending order.  Visit slots are cut into groups of
+// kPaceWidth; group g belongs to the blocks b with g == min(b * n / (nbk * kPaceWidth), groups - 1).  A group
+// takes its own blocks in ascending order up to its number of slots; the blocks over that number (ascending
+// over the whole list) fill the slots left empty (ascending); every group's slots are then put in ascending
+// block order.  in == out is allowed.  A malformed list (unsorted, repeated or out-of-range blocks) still
+// gives a permutation of the blocks clamped to the valid range.
+constexpr int kPaceWidth = 8;
+__global__ __launch_bounds__(64) void pace_order_kernel(const int32_t* in, int32_t* out, const int32_t* __restrict__ lens, int nbk, int stride) {
+    extern __shared__ int32_t pace_lds[];
+    int32_t* const lst = pace_lds;               // [stride] the row, ascending
+    int32_t* const slots = lst + stride;         // [stride] block per visit slot, -1 = empty
+    int32_t* const spare = slots + stride;       // [stride] blocks over their group's room, ascending
+    int32_t* const first = spare + stride;       // [groups] position of a group's first block in lst
+    const int lane = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    const int32_t* src = in + row * stride;
+    int32_t* dst = out + row * stride;
+    const int n = min(max(lens[row], 0), stride);
+    if (src != dst)
+        for (int e = n + lane; e < stride; e += 64) dst[e] = src[e];
+    if (n <= kPaceWidth) {
+        if (src != dst)
+            for (int e = lane; e < n; e += 64) dst[e] = src[e];
+        return;
+    }
+    const int groups = (n + kPaceWidth - 1) / kPaceWidth;
+    const int64_t span = (int64_t)nbk * kPaceWidth;
+    auto group_of = [&](int32_t b) { return (int)min((int64_t)b * n / span, (int64_t)groups - 1); };
+    for (int e = lane; e < n; e += 64) {
+        lst[e] = min(max(src[e], 0), nbk - 1);
+        slots[e] = -1;
+    }
+    for (int g = lane; g < groups; g += 64) first[g] = 0;
+    __syncthreads();
+    for (int e = lane; e < n; e += 64) {
+        const int g = group_of(lst[e]);
+        if (e == 0 || group_of(lst[e - 1]) != g) first[g] = e;
+    }
+    __syncthreads();
+    const uint64_t below = ((uint64_t)1 << lane) - 1;
+    int taken = 0;
+    for (int base = 0; base < n; base += 64) {
+        const int e = base + lane;
+        bool over = false;
+        if (e < n) {
+            const int g = group_of(lst[e]), rank = e - first[g];
+            const int room = min(kPaceWidth, n - g * kPaceWidth);
+            if (rank >= 0 && rank < room) slots[g * kPaceWidth + rank] = lst[e];
+            else over = true;
+        }
+        const uint64_t m = __ballot(over);
+        if (over) spare[taken + __popcll(m & below)] = lst[e];
+        taken += __popcll(m);
+    }
+    __syncthreads();
+    taken = 0;
+    for (int base = 0; base < n; base += 64) {
+        const int s = base + lane;
+        const bool empty = s < n && slots[s] < 0;
+        const uint64_t m = __ballot(empty);
+        if (empty) slots[s] = spare[taken + __popcll(m & below)];
+        taken += __popcll(m);
+    }
+    __syncthreads();
+    for (int s = lane; s < n; s += 64) {
+        const int lo = s / kPaceWidth * kPaceWidth, hi = min(lo + kPaceWidth, n);
+        const int32_t b = slots[s];
+        int rank = 0;
+        for (int t = lo; t < hi; ++t) rank += (slots[t] < b || (slots[t] == b && t < s)) ? 1 : 0;
+        dst[lo + rank] = b;
+    }
+}
+
 // ---------------------------------------------------------------- CDF rule
 __device__ inline float score_value(uint16_t s, int dtype) {
     if (dtype == BSA_F16) return (float)__builtin_bit_cast(_Float16, s);
@@ -376,6 +456,16 @@ hipError_t launch_topk(const void* score, int32_t* idx, int32_t* idx_sorted, int
     if (dtype == BSA_F32)
         return launch_topk_t<uint32_t>((const uint32_t*)score, idx, idx_sorted, lens, rows, nbk, k_sel, k_rows, stride, st);
     return launch_topk_t<uint16_t>((const uint16_t*)score, idx, idx_sorted, lens, rows, nbk, k_sel, k_rows, stride, st);
+}
+
+hipError_t launch_pace_order(const int32_t* in, int32_t* out, const int32_t* lens, int64_t rows, int nbk, int stride,
+                             hipStream_t st) {
+    if (rows <= 0 || stride <= 0) return hipSuccess;
+    const int groups = (stride + kPaceWidth - 1) / kPaceWidth;
+    const size_t lds = ((size_t)3 * stride + groups) * sizeof(int32_t);
+    if (lds > 64 * 1024 || rows > 0x7fffffff) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(pace_order_kernel, dim3((unsigned)rows), dim3(64), lds, st, in, out, lens, nbk, stride);
+    return hipGetLastError();
 }
 
 hipError_t launch_cdf_count(const void* score, int32_t* lens, int64_t rows, int nbk, float threshold, float scale,

@@ -41,6 +41,7 @@ SIGNATURES = {
     "bsa_mean_pool": (_i, [_p, _p, _i, _i, _i64, _i, _i, _i, _p]),
     "bsa_score_topk": (_i, [_p, _p, _p, _p, _p, _p] + [_i] * 7 + [_p]),
     "bsa_topk_from_score": (_i, [_p, _p, _p, _p] + [_i] * 6 + [_p]),
+    "bsa_visit_order": (_i, [_p, _p, _p, _i64, _i, _i, _p]),
     "bsa_score_cdf": (_i, [_p, _p, _p, _p, _p, _p] + [_i] * 5 + [_f, _f, _i, _i, _i, _p]),
     "bsa_cdf_from_score": (_i, [_p, _p, _p, _p] + [_i] * 4 + [_f, _f, _i, _i, _i, _p]),
     "bsa_fwd": (_i, [_p] * 8 + [_i, _i, _i64, _i64, _i, _i, _i, _i, _f, _i, _p]),

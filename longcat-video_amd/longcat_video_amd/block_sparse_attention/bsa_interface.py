@@ -155,6 +155,23 @@ def _score_topk(q_cmp, k_cmp, k_sel, order="score"):
     return idx, lens, score
 
 
+def visit_order(idx_sorted: torch.Tensor, lens: torch.Tensor, n_kv_blocks: int) -> torch.Tensor:
+    """The operator's visiting order for lists given in ascending block order (bsa_visit_order): [..., rows, width]
+    int32 lists with lens[...] entries in use.  No counterpart in the reference, whose kernel visits the blocks in
+    list order; attention depends on the order only through rounding."""
+    _need_gpu(idx_sorted, lens)
+    assert idx_sorted.dtype == torch.int32 and lens.dtype == torch.int32 and idx_sorted.shape[:-1] == lens.shape
+    idx_sorted, lens = idx_sorted.contiguous(), lens.contiguous()
+    out = torch.empty_like(idx_sorted)
+    if idx_sorted.numel() == 0:
+        return out
+    lib = _capi.load()
+    with torch.cuda.device(idx_sorted.device):
+        _capi.check(lib.bsa_visit_order(_ptr(idx_sorted), _ptr(lens), _ptr(out), lens.numel(), int(n_kv_blocks),
+                                        idx_sorted.shape[-1], _stream(idx_sorted)), "visit_order")
+    return out
+
+
 def cal_score(q: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
     """bsa_interface.py:180-184: unscaled ``q @ k^T`` in the input dtype."""
     return _score_topk(q, k, 0)[2]

@@ -49,6 +49,14 @@ fixtures for this path, so the pins are mathematical; see tests/test_oracle_*):
                                     W + m*a*U.D exactly; split up-projection ==
                                     one block-diagonal matrix; torch F.linear
 
+  paced_visit_order                 (no reference counterpart: the reference
+                                    visits the selected blocks in list order,
+                                    and the result does not depend on that
+                                    order beyond rounding) permutation
+                                    property, identity on evenly spread lists,
+                                    a hand-worked example, a brute-force
+                                    sequential restatement
+
 What no CPU check can pin ("parity unpinned", because the reference executes
 them inside un-vendored third parties - Triton and ATen/Inductor of torch 2.6 -
 and holds no recorded outputs): torch.topk's order among exactly tied scores,
@@ -325,6 +333,42 @@ def blockwise_attention(q, k, v, idx, lens, bs_q: int, bs_k: int, sm_scale: floa
                 M[b, h, mblk * bs_q:(mblk + 1) * bs_q] = m_i + torch.log2(l_i)
                 o[b, h, mblk * bs_q:(mblk + 1) * bs_q] = (acc / l_i.unsqueeze(1)).to(dt)
     return o, M * LN2
+
+
+PACE_WIDTH = 8
+
+
+def paced_visit_order(blocks: np.ndarray, n_kv_blocks: int, width: int = PACE_WIDTH) -> np.ndarray:
+    """Order in which the engine's attention kernel visits one query block's selected KV blocks.  The
+    reference visits them in list order (vmask:249-285) and softmax(QK^T)V does not depend on the
+    order beyond fp rounding, so the engine is free to choose one; it chooses the order that keeps
+    the query blocks that run side by side on the GPU at the same place of the KV sequence, which is
+    what lets them share K/V tiles in the L2 cache.
+
+    `blocks`: the n selected block indices in ascending order.  Visit slots are cut into groups of
+    `width`; group g belongs to the blocks whose index b falls in the g-th n/width-th of the KV
+    sequence, g = min(b*n // (n_kv_blocks*width), groups-1).  A group takes its own blocks in
+    ascending order up to its number of slots; the blocks over that number, in ascending order over
+    the whole list, fill the slots that groups with too few blocks leave empty, in ascending slot
+    order; finally every group's slots are put in ascending block order.  Lists of at most `width`
+    blocks stay as they are."""
+    blocks = np.asarray(blocks)
+    n = len(blocks)
+    if n <= width:
+        return blocks.copy()
+    groups = -(-n // width)
+    g = np.minimum(blocks.astype(np.int64) * n // (n_kv_blocks * width), groups - 1)
+    slots = np.full(n, -1, dtype=np.int64)
+    spare = []
+    for grp in range(groups):
+        own = blocks[g == grp]
+        room = min(width, n - grp * width)
+        slots[grp * width:grp * width + min(len(own), room)] = own[:room]
+        spare.extend(own[room:])
+    slots[slots < 0] = spare
+    for grp in range(groups):
+        slots[grp * width:(grp + 1) * width] = np.sort(slots[grp * width:(grp + 1) * width])
+    return slots.astype(blocks.dtype)
 
 
 def merge_partial_attention(o_a, lse_a, o_b, lse_b):

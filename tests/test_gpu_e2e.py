@@ -309,7 +309,7 @@ def test_cdf_lists_of_unequal_length_schedule(spread):
     """With the CDF rule the operator enqueues two schedules of the attention kernel (rounds of equal work items,
     and one launch whose workgroups draw the items longest list first) and picks one on the device from the list
     lengths.  Whatever it picks, the output must equal, bit for bit, what the kernel gives in plain rounds on the
-    same lists (ThwAttention), here with more work items (640) than one round holds: 'wide' has lists from a few
+    same lists in the same visiting order (ThwAttention), here with more work items (640) than one round holds: 'wide' has lists from a few
     blocks to most of them, 'narrow' lists of nearly equal length."""
     latent, heads = (8, 32, 32), 5
     S = int(np.prod(latent))
@@ -340,6 +340,7 @@ def test_cdf_lists_of_unequal_length_schedule(spread):
     big = idx.shape[-1] + 1
     asc = torch.where(idx < 0, torch.full_like(idx, big), idx).sort(dim=-1).values
     asc = torch.where(asc == big, torch.zeros_like(asc), asc)
+    asc = I().visit_order(asc.int(), lens, int(np.prod(O.block_grid(latent, (4, 4, 4)))))      # the operator's visiting order
     rounds = I().ThwAttention(kg, vg, latent, latent, (4, 4, 4), (4, 4, 4))(qg, asc, lens)
     assert torch.equal(o, rounds)
     # the same choice of schedule for a caller's own lists
