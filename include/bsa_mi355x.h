@@ -221,10 +221,15 @@ int bsa_fwd_3d(const bsa_3d_params* p,
  * capture, tight serving loops, harnesses that forbid hipMalloc.  What bsa_fwd_3d carves from its workspace
  * lives in a buffer of BSA_STATIC_SCRATCH_BYTES that is part of the library's code object, so every GPU the
  * library is used on holds that much memory from the first call on it until the process ends.
- *   - Arguments and results are those of bsa_fwd_3d (same kernels, same bits).
- *   - A problem whose bsa_workspace_bytes() exceeds BSA_STATIC_SCRATCH_BYTES is rejected with
- *     BSA_ERR_WORKSPACE before anything is launched (64 MiB covers, in bf16 with 4x4x4 chunks, the 720p
- *     grid at up to 6 heads or the 480p grid at up to 17 heads: one GPU's share of a head-sharded layer).
+ *   - Arguments and results are those of bsa_fwd_3d: the same selection bit for bit.  To fit the buffer it
+ *     makes no fragment-order copies of k and v; its attention kernel reads them where they lie (the
+ *     LDS-tiled kernel), so the output agrees with bsa_fwd_3d's within the rounding of a different
+ *     summation order (bf16 / fp16: max-abs 1.6e-2, mean-abs 1e-3 on unit-variance inputs; fp32: equal).
+ *   - A problem that needs more scratch than BSA_STATIC_SCRATCH_BYTES - pooled means, scores, lists, tables and
+ *     the zero-filled copies of the KV chunks at the padded edge of the grid, i.e. bsa_workspace_bytes() less
+ *     the two fragment-order copies - is rejected with BSA_ERR_WORKSPACE before anything is launched (64 MiB
+ *     covers, in bf16 with 4x4x4 chunks, the 720p grid at up to 6 heads or the 480p grid at up to 17 heads:
+ *     one GPU's share of a head-sharded layer).
  *   - The call itself makes no hipMalloc / hipFree and calls no allocating library routine.  The first call
  *     on a device looks up the buffer's address (hipGetSymbolAddress); make that call outside graph capture.
  *   - All calls on one GPU share the one buffer, which keeps the previous call's contents; nothing in it
