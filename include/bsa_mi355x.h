@@ -108,7 +108,7 @@ int bsa_mean_pool(const void* x, void* out, int B, int Hn, int64_t S, int block,
  *             idx_out / idx_sorted_out must be given
  *   lens_out  int32 [B, Hn, nbq], every entry k_sel (bsa:217-222)
  *   score_out optional [B, Hn, nbq, nbk] in `dtype`
- * Limits: D == 128, 0 <= k_sel <= nbk <= 4096, k_sel <= 1024.
+ * Limits: D == 128, 0 <= k_sel <= nbk <= 4096.
  * NaN scores order above +inf, as torch.topk orders them.
  */
 int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32_t* idx_sorted_out,
@@ -125,7 +125,7 @@ int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32
  *   (the reference returns all nbk sorted columns, of which the attention kernel reads the first lens).
  * The weights are fp32 for every storage type and the running sum is kept in double precision: a row may
  * differ from an fp32 running sum only where that sum comes within rounding of the threshold.
- * Limits as for bsa_score_topk; idx_stride <= min(nbk, 1024).
+ * Limits as for bsa_score_topk; idx_stride <= nbk.
  */
 int bsa_score_cdf(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32_t* idx_sorted_out,
                   int32_t* lens_out, void* score_out, int B, int Hn, int nbq, int nbk, int D,
@@ -185,7 +185,7 @@ int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, con
  *   q [B, Hn, Tq*Hq*Wq, D] with element strides q_strides = {B, Hn, S}; same
  *   for k, v; o likewise with o_strides.  k_sel from bsa_num_selected() on the
  *   padded KV block count.  With p->cdf_threshold > 0 the selection follows
- *   bsa_score_cdf instead (bsa:268-277 dispatch), at most min(nbk, 1024) blocks per
+ *   bsa_score_cdf instead (bsa:268-277 dispatch), at most nbk blocks per
  *   row, and idx_out has that many columns.  workspace: bsa_workspace_bytes() bytes, 256-byte
  *   aligned.  idx_out/lens_out/score_out are optional copies for inspection
  *   (shapes as in bsa_score_topk).  With cdf_threshold the lists differ in length: the work is then also

@@ -132,7 +132,6 @@ static int check_topk(int B, int Hn, int nbq, int nbk, int k_sel, int dtype) {
         return set_error(BSA_ERR_BAD_ARG, "top-k: sizes must be positive (B=%d heads=%d nbq=%d nbk=%d)", B, Hn, nbq, nbk);
     if (k_sel < 0 || k_sel > nbk) return set_error(BSA_ERR_SHAPE, "top-k: k_sel=%d outside [0, %d]", k_sel, nbk);
     if (nbk > 4096) return set_error(BSA_ERR_UNSUPPORTED, "top-k: %d KV blocks exceed the limit of 4096", nbk);
-    if (k_sel > 1024) return set_error(BSA_ERR_UNSUPPORTED, "top-k: k_sel=%d exceeds the limit of 1024", k_sel);
     return BSA_OK;
 }
 
@@ -171,8 +170,8 @@ int bsa_score_topk(const void* q_cmp, const void* k_cmp, int32_t* idx_out, int32
 static int check_cdf(float thr, float scale, int k_min, int idx_stride, int nbk) {
     if (!(thr > 0.f) || !std::isfinite(thr)) return set_error(BSA_ERR_BAD_ARG, "cdf: threshold must be positive and finite");
     if (!(scale > 0.f) || !std::isfinite(scale)) return set_error(BSA_ERR_BAD_ARG, "cdf: sm_scale must be positive and finite");
-    if (idx_stride <= 0 || idx_stride > nbk || idx_stride > 1024)
-        return set_error(BSA_ERR_SHAPE, "cdf: idx_stride=%d outside [1, min(%d, 1024)]", idx_stride, nbk);
+    if (idx_stride <= 0 || idx_stride > nbk || idx_stride > 4096)
+        return set_error(BSA_ERR_SHAPE, "cdf: idx_stride=%d outside [1, min(%d, 4096)]", idx_stride, nbk);
     if (k_min < 0 || k_min > idx_stride) return set_error(BSA_ERR_SHAPE, "cdf: k_min=%d outside [0, %d]", k_min, idx_stride);
     return BSA_OK;
 }
@@ -259,7 +258,7 @@ int make_plan(const bsa_3d_params* p, Plan* pl, bool compact = false) {
     pl->nbk = pl->gk.blocks();
     BSA_TRY(check_topk(p->B, p->Hn, pl->nbq, pl->nbk, p->k_sel, p->dtype));
     pl->cdf = p->cdf_threshold > 0.f;
-    pl->sel_width = pl->cdf ? (pl->nbk < 1024 ? pl->nbk : 1024) : p->k_sel;
+    pl->sel_width = pl->cdf ? pl->nbk : p->k_sel;       // the CDF rule may keep every block of a row (nbk <= 4096)
     if (pl->cdf && !std::isfinite(p->cdf_threshold)) return set_error(BSA_ERR_BAD_ARG, "cdf_threshold must be finite");
     if (!(p->sm_scale > 0.f) || !std::isfinite(p->sm_scale)) return set_error(BSA_ERR_BAD_ARG, "sm_scale must be positive and finite");
     pl->Sqp = (int64_t)pl->nbq * pl->gq.chunk();

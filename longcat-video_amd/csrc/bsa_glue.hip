@@ -7,6 +7,7 @@
 
 #include <map>
 #include <mutex>
+#include <shared_mutex>
 #include <tuple>
 
 namespace bsa {
@@ -270,24 +271,34 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(const T* __restrict__ sr
 }
 
 // ------------------------------------------------------------- linear (GEMM)
-// Shape of a linear call -> the algorithm bsa_linear_bf16_tune measured to be the fastest for it.
+// Shape of a linear call on a device -> the algorithm it runs with: the one bsa_linear_bf16_tune measured to be
+// the fastest, else hipBLASLt's first proposal that fits the workspace (asked for once per shape, not per call).
 struct LinearKey {
     int64_t M, ldx, ldw, ldo;
-    int N, K, bias, residual;
+    int N, K, bias, residual, device;
     bool operator<(const LinearKey& o) const {
-        return std::tie(M, ldx, ldw, ldo, N, K, bias, residual) < std::tie(o.M, o.ldx, o.ldw, o.ldo, o.N, o.K, o.bias, o.residual);
+        return std::tie(M, ldx, ldw, ldo, N, K, bias, residual, device) <
+               std::tie(o.M, o.ldx, o.ldw, o.ldo, o.N, o.K, o.bias, o.residual, o.device);
     }
 };
 struct TunedAlgo {
     hipblasLtMatmulAlgo_t algo;
     size_t workspace;
 };
+// Calls from several threads do not serialise: every thread has its own hipBLASLt handle per device, and the
+// table of chosen algorithms is read under a shared lock (written once per shape, and by the tuning call).
 struct LtState {
-    std::mutex mu;
-    hipblasLtHandle_t handle = nullptr;
-    std::map<LinearKey, TunedAlgo> tuned;
+    std::shared_mutex mu;
+    std::map<LinearKey, TunedAlgo> chosen;
 };
 LtState& lt_state() { static LtState s; return s; }
+constexpr int kMaxLtDevices = 64;
+hipblasLtHandle_t thread_handle(int device) {
+    thread_local hipblasLtHandle_t handles[kMaxLtDevices] = {};
+    if (device < 0 || device >= kMaxLtDevices) return nullptr;
+    if (!handles[device] && hipblasLtCreate(&handles[device]) != HIPBLAS_STATUS_SUCCESS) handles[device] = nullptr;
+    return handles[device];
+}
 
 }  // namespace
 }  // namespace bsa
@@ -458,9 +469,10 @@ static int linear_impl(const void* x, int64_t ldx, const void* w, int64_t ldw, c
     if (!workspace || workspace_bytes < ((size_t)64 << 20))
         return set_error(BSA_ERR_WORKSPACE, "linear: a workspace of at least 64 MiB is required (got %zu bytes)", workspace_bytes);
     LtState& st = lt_state();
-    std::lock_guard<std::mutex> lock(st.mu);
-    if (!st.handle && hipblasLtCreate(&st.handle) != HIPBLAS_STATUS_SUCCESS)
-        return set_error(BSA_ERR_HIP, "linear: hipblasLtCreate failed");
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return set_error(BSA_ERR_HIP, "linear: hipGetDevice failed");
+    const hipblasLtHandle_t handle = thread_handle(device);
+    if (!handle) return set_error(BSA_ERR_HIP, "linear: hipblasLtCreate failed");
 #define BSA_LT(call)                                                                        \
     do {                                                                                    \
         const hipblasStatus_t s_ = (call);                                                  \
@@ -490,17 +502,25 @@ static int linear_impl(const void* x, int64_t ldx, const void* w, int64_t ldw, c
         BSA_LT(hipblasLtMatmulPreferenceCreate(&pref));
         const uint64_t wsb = workspace_bytes;
         BSA_LT(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &wsb, sizeof(wsb)));
-        const LinearKey key{M, ldx, ldw, ldo, N, K, bias ? 1 : 0, residual ? 1 : 0};
-        const auto hit = st.tuned.find(key);
-        if (!tune && hit != st.tuned.end() && hit->second.workspace <= workspace_bytes) {
-            BSA_LT(hipblasLtMatmul(st.handle, desc, &alpha, w, la, x, lb, &beta, residual ? residual : out, lc, out, lc,
-                                   &hit->second.algo, workspace, workspace_bytes, (hipStream_t)stream));
-            goto done;
+        const LinearKey key{M, ldx, ldw, ldo, N, K, bias ? 1 : 0, residual ? 1 : 0, device};
+        if (!tune) {
+            TunedAlgo known;
+            bool have = false;
+            {
+                std::shared_lock<std::shared_mutex> lock(st.mu);
+                const auto hit = st.chosen.find(key);
+                if (hit != st.chosen.end() && hit->second.workspace <= workspace_bytes) { known = hit->second; have = true; }
+            }
+            if (have) {
+                BSA_LT(hipblasLtMatmul(handle, desc, &alpha, w, la, x, lb, &beta, residual ? residual : out, lc, out, lc,
+                                       &known.algo, workspace, workspace_bytes, (hipStream_t)stream));
+                goto done;
+            }
         }
         constexpr int kMaxAlgos = 32;
         hipblasLtMatmulHeuristicResult_t heur[kMaxAlgos];
         int found = 0, pick = -1;
-        BSA_LT(hipblasLtMatmulAlgoGetHeuristic(st.handle, desc, la, lb, lc, lc, pref, tune ? kMaxAlgos : 8, heur, &found));
+        BSA_LT(hipblasLtMatmulAlgoGetHeuristic(handle, desc, la, lb, lc, lc, pref, tune ? kMaxAlgos : 8, heur, &found));
         // never hand the library less workspace than the algorithm says it uses
         for (int i = 0; i < found && pick < 0; ++i)
             if (heur[i].state == HIPBLAS_STATUS_SUCCESS && heur[i].workspaceSize <= workspace_bytes) pick = i;
@@ -520,7 +540,7 @@ static int linear_impl(const void* x, int64_t ldx, const void* w, int64_t ldw, c
                 bool ok = true;
                 for (int r = 0; r < 4 && ok; ++r) {
                     if (r == 1) ok = hipEventRecord(e0, (hipStream_t)stream) == hipSuccess;
-                    ok = ok && hipblasLtMatmul(st.handle, desc, &alpha, w, la, x, lb, &beta, residual ? residual : out, lc, out, lc,
+                    ok = ok && hipblasLtMatmul(handle, desc, &alpha, w, la, x, lb, &beta, residual ? residual : out, lc, out, lc,
                                                &heur[i].algo, workspace, workspace_bytes, (hipStream_t)stream) == HIPBLAS_STATUS_SUCCESS;
                 }
                 float ms = 0.f;
@@ -537,12 +557,19 @@ static int linear_impl(const void* x, int64_t ldx, const void* w, int64_t ldw, c
             if (best_i < 0) { rc = set_error(BSA_ERR_HIP, "linear tune: no candidate ran"); goto done; }
             // three runs each are a noisy measurement: the library's own first choice stays unless it is beaten by 2 %
             if (dflt > 0.f && best > 0.98f * dflt) { best_i = pick; best = dflt; }
-            st.tuned[key] = TunedAlgo{heur[best_i].algo, heur[best_i].workspaceSize};
+            {
+                std::unique_lock<std::shared_mutex> lock(st.mu);
+                st.chosen[key] = TunedAlgo{heur[best_i].algo, heur[best_i].workspaceSize};
+            }
             if (best_ms) *best_ms = best;
             rc = tried;
             goto done;
         }
-        BSA_LT(hipblasLtMatmul(st.handle, desc, &alpha, w, la, x, lb, &beta, residual ? residual : out, lc, out, lc,
+        {
+            std::unique_lock<std::shared_mutex> lock(st.mu);
+            st.chosen.emplace(key, TunedAlgo{heur[pick].algo, heur[pick].workspaceSize});      // a measured choice stays
+        }
+        BSA_LT(hipblasLtMatmul(handle, desc, &alpha, w, la, x, lb, &beta, residual ? residual : out, lc, out, lc,
                                &heur[pick].algo, workspace, workspace_bytes, (hipStream_t)stream));
     }
 done:

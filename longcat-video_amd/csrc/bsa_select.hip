@@ -133,18 +133,124 @@ template <> struct KeyOf<uint32_t> {   // fp32 bit patterns
     __device__ static int index(uint64_t k) { return (int)(0xFFFFFFFFu - (uint32_t)k); }
 };
 
-constexpr int kMaxSel = 1024;   // winners kept in LDS per wavefront
+constexpr int kMaxSel = 4096;   // longest list: the score-order ranking keeps a row's winners in LDS
 
 // Order-preserving image of a score alone (ties stay ties).
 __device__ inline uint32_t ord_of(uint16_t s) { return ord16(s); }
 __device__ inline uint32_t ord_of(uint32_t s) { return ord32(s); }
 
-// One wavefront per score row; lane l holds columns l, l + 64, ... in registers.
-//   1. bitwise binary search for the k-th largest score value t (counting = ballot + popcount);
+// Selection of one score row by one wavefront; lane l holds the order-preserving images of columns l, l + 64,
+// ... in registers (0 for columns past the end of the row).
+//   1. the k-th largest score value t: for 16-bit scores from a histogram of the codes just below the row
+//      maximum, otherwise (and for rows whose winners reach further down) by a bitwise binary search whose
+//      counting step is a ballot + popcount;
 //   2. every score above t wins, and of the scores equal to t the ones with the lowest column
 //      index, as many as are still needed; walking the registers in column order hands out the
 //      positions of the ascending-block-order list at the same time (no sort);
 //   3. only when the score-order list is wanted: rank the winners by (score desc, index asc).
+// raw_at(i): the stored score of column i.  mine: one key of LDS per list entry (SCORE_ORDER only); h: 256 words of LDS.
+template <typename S, int NPL, bool SCORE_ORDER, typename RawAt>
+__device__ inline void select_row(const uint32_t (&val)[NPL], RawAt raw_at, int lane, int nbk, int k_sel,
+                                  int32_t* __restrict__ idx_row, int32_t* __restrict__ idx_sorted_row,
+                                  typename KeyOf<S>::type* mine, uint32_t* h) {
+    typedef typename KeyOf<S>::type K;
+    constexpr int kValueBits = 8 * (int)sizeof(S);
+    // The k-th largest score value t: every column above it wins, and of the columns equal to it the first
+    // need_eq in column order.
+    uint32_t thr = 0;
+    int cnt_gt = 0;
+    bool found = false;
+    if (kValueBits == 16) {
+        // 16-bit scores: the winners of a row usually lie within a few hundred codes of the row maximum, so one
+        // histogram of (maximum - ord) over 255 bins, built with LDS atomics by the columns that fall into it,
+        // and one scan find t.  Rows whose k_sel largest values reach further down take the search below.
+        uint32_t mx = 0;
+#pragma unroll
+        for (int j = 0; j < NPL; ++j) mx = max(mx, val[j]);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, o));
+        *reinterpret_cast<uint4*>(h + 4 * lane) = make_uint4(0u, 0u, 0u, 0u);
+        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < NPL; ++j) {
+            const uint32_t d = mx - val[j];
+            if (j * 64 + lane < nbk && d < 255u) atomicAdd(h + d, 1u);
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_wave_barrier();
+        const uint4 c = *reinterpret_cast<const uint4*>(h + 4 * lane);
+        const int own = (int)(c.x + c.y + c.z + c.w);
+        int upto = own;                                    // columns within bins 0 .. 4 lane + 3
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int t = __shfl_up(upto, o);
+            if (lane >= o) upto += t;
+        }
+        const int before = upto - own;
+        const uint64_t holder = __ballot(before < k_sel && k_sel <= upto);
+        if (holder != 0) {
+            int bin = 4 * lane, run = before;
+            if (run + (int)c.x < k_sel) { run += (int)c.x; ++bin;
+                if (run + (int)c.y < k_sel) { run += (int)c.y; ++bin;
+                    if (run + (int)c.z < k_sel) { run += (int)c.z; ++bin; } } }
+            const int src = __builtin_ctzll(holder);
+            thr = mx - (uint32_t)__shfl(bin, src);
+            cnt_gt = __shfl(run, src);
+            found = true;
+        }
+    }
+    if (!found) {
+        // Largest t with count(ord >= t) >= k_sel, t = 0 if there is none above, by a bitwise binary search
+        // whose counting step is a ballot + popcount.  Every candidate is at least 1, so the zeros past the end
+        // of the row never count.  Leaving early with exactly k_sel columns at or above t is fine: the winners
+        // are then all columns at or above t.
+        for (int bit = kValueBits - 1; bit >= 0; --bit) {
+            const uint32_t cand = thr | (1u << bit);
+            int cnt = 0;
+#pragma unroll
+            for (int j = 0; j < NPL; ++j) cnt += __popcll(__ballot(val[j] >= cand));
+            if (cnt >= k_sel) {
+                thr = cand;
+                if (cnt == k_sel) break;
+            }
+        }
+        cnt_gt = 0;
+#pragma unroll
+        for (int j = 0; j < NPL; ++j) cnt_gt += __popcll(__ballot(val[j] > thr));
+    }
+    const int need_eq = k_sel - cnt_gt;
+
+    int pos = 0, eq_seen = 0;
+    const uint64_t lt = ((uint64_t)1 << lane) - 1;
+#pragma unroll
+    for (int j = 0; j < NPL; ++j) {
+        const int i = j * 64 + lane;
+        const bool eq = val[j] == thr && i < nbk;          // thr may be 0, like the padding of val
+        const uint64_t meq = __ballot(eq);
+        const bool win = val[j] > thr || (eq && eq_seen + __popcll(meq & lt) < need_eq);
+        const uint64_t m = __ballot(win);
+        if (win) {
+            const int p = pos + __popcll(m & lt);
+            if (idx_sorted_row) idx_sorted_row[p] = i;                        // column order = ascending block order
+            if (SCORE_ORDER) mine[p] = KeyOf<S>::make(raw_at(i), i);
+        }
+        pos += __popcll(m);
+        eq_seen += __popcll(meq);
+    }
+    if (!SCORE_ORDER) return;
+    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): LDS writes of this wavefront landed
+    __builtin_amdgcn_wave_barrier();
+    // descending score, ties towards the lowest index: the order of the combined keys
+    for (int e = lane; e < k_sel; e += 64) {
+        const K me = mine[e];
+        int rank = 0;
+        for (int o = 0; o < k_sel; ++o) rank += mine[o] > me;
+        idx_row[rank] = KeyOf<S>::index(me);
+    }
+}
+
+// Top-k from a score matrix in memory: one wavefront per score row.
 template <typename S, int NPL, bool SCORE_ORDER>
 __global__ __launch_bounds__(256) void topk_kernel(const S* __restrict__ score,
                                                    int32_t* __restrict__ idx_out,
@@ -153,8 +259,8 @@ __global__ __launch_bounds__(256) void topk_kernel(const S* __restrict__ score,
                                                    int nbk, int k_all, const int32_t* __restrict__ k_rows,
                                                    int stride) {
     typedef typename KeyOf<S>::type K;
-    constexpr int kValueBits = 8 * (int)sizeof(S);
-    __shared__ K sel[4][kMaxSel];
+    extern __shared__ __attribute__((aligned(16))) unsigned char topk_keys[];    // SCORE_ORDER: 4 x stride keys
+    __shared__ __attribute__((aligned(16))) uint32_t hist[4][256];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + wave;
     if (row >= rows) return;
@@ -176,54 +282,10 @@ __global__ __launch_bounds__(256) void topk_kernel(const S* __restrict__ score,
         const S raw = srow[min(i, nbk - 1)];               // unconditional load, masked afterwards
         val[j] = i < nbk ? ord_of(raw) : 0u;
     }
-    // Largest t with count(ord >= t) >= k_sel, t = 0 if there is none above.  Every candidate is at
-    // least 1, so the zeros past the end of the row never count.  Leaving early with exactly k_sel
-    // columns at or above t is fine: the winners are then all columns at or above t.
-    uint32_t thr = 0;
-    for (int bit = kValueBits - 1; bit >= 0; --bit) {
-        const uint32_t cand = thr | (1u << bit);
-        int cnt = 0;
-#pragma unroll
-        for (int j = 0; j < NPL; ++j) cnt += __popcll(__ballot(val[j] >= cand));
-        if (cnt >= k_sel) {
-            thr = cand;
-            if (cnt == k_sel) break;
-        }
-    }
-    // every column above thr wins; of the real columns equal to thr, the first need_eq in column order
-    int cnt_gt = 0;
-#pragma unroll
-    for (int j = 0; j < NPL; ++j) cnt_gt += __popcll(__ballot(val[j] > thr));
-    const int need_eq = k_sel - cnt_gt;
-
-    K* mine = sel[wave];
-    int pos = 0, eq_seen = 0;
-    const uint64_t lt = ((uint64_t)1 << lane) - 1;
-#pragma unroll
-    for (int j = 0; j < NPL; ++j) {
-        const int i = j * 64 + lane;
-        const bool eq = val[j] == thr && i < nbk;          // thr may be 0, like the padding of val
-        const uint64_t meq = __ballot(eq);
-        const bool win = val[j] > thr || (eq && eq_seen + __popcll(meq & lt) < need_eq);
-        const uint64_t m = __ballot(win);
-        if (win) {
-            const int p = pos + __popcll(m & lt);
-            if (idx_sorted_out) idx_sorted_out[row * stride + p] = i;         // column order = ascending block order
-            if (SCORE_ORDER) mine[p] = KeyOf<S>::make(srow[i], i);
-        }
-        pos += __popcll(m);
-        eq_seen += __popcll(meq);
-    }
-    if (!SCORE_ORDER) return;
-    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): LDS writes of this wavefront landed
-    __builtin_amdgcn_wave_barrier();
-    // descending score, ties towards the lowest index: the order of the combined keys
-    for (int e = lane; e < k_sel; e += 64) {
-        const K me = mine[e];
-        int rank = 0;
-        for (int o = 0; o < k_sel; ++o) rank += mine[o] > me;
-        idx_out[row * stride + rank] = KeyOf<S>::index(me);
-    }
+    select_row<S, NPL, SCORE_ORDER>(val, [&](int i) { return srow[i]; }, lane, nbk, k_sel,
+                                    idx_out ? idx_out + row * stride : nullptr,
+                                    idx_sorted_out ? idx_sorted_out + row * stride : nullptr,
+                                    reinterpret_cast<K*>(topk_keys) + (SCORE_ORDER ? (size_t)wave * stride : 0), hist[wave]);
 }
 
 // ---------------------------------------------------------------- visiting order
@@ -413,12 +475,19 @@ template <typename S>
 hipError_t launch_topk_t(const S* score, int32_t* idx, int32_t* idx_sorted, int32_t* lens, int64_t rows,
                          int nbk, int k_sel, const int32_t* k_rows, int stride, hipStream_t st) {
     dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    // the score-order ranking keeps the winners of the workgroup's four rows in LDS
+    const size_t lds = idx != nullptr ? (size_t)4 * stride * sizeof(typename KeyOf<S>::type) : 0;
 #define BSA_TOPK(N)                                                                                \
     do {                                                                                           \
-        if (idx != nullptr)                                                                        \
-            hipLaunchKernelGGL((topk_kernel<S, N, true>), grid, block, 0, st, score, idx, idx_sorted, lens, rows, nbk, k_sel, k_rows, stride);  \
-        else                                                                                       \
+        if (idx != nullptr) {                                                                      \
+            if (lds > 64 * 1024) {                                                                 \
+                const hipError_t ea = hipFuncSetAttribute((const void*)topk_kernel<S, N, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+                if (ea != hipSuccess) return ea;                                                   \
+            }                                                                                      \
+            hipLaunchKernelGGL((topk_kernel<S, N, true>), grid, block, lds, st, score, idx, idx_sorted, lens, rows, nbk, k_sel, k_rows, stride);  \
+        } else {                                                                                   \
             hipLaunchKernelGGL((topk_kernel<S, N, false>), grid, block, 0, st, score, idx, idx_sorted, lens, rows, nbk, k_sel, k_rows, stride); \
+        }                                                                                          \
     } while (0)
     if (nbk <= 4 * 64) BSA_TOPK(4);
     else if (nbk <= 8 * 64) BSA_TOPK(8);

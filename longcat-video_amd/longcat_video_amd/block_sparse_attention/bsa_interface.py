@@ -201,7 +201,7 @@ def get_select_indices_topk(q: torch.Tensor, k: torch.Tensor, sparsity: float):
 
 
 def _cdf_width(nbk: int) -> int:
-    return min(int(nbk), 1024)       # columns kept per row at most
+    return min(int(nbk), 4096)       # columns kept per row at most: all of them (the engine's lists hold 4096 entries)
 
 
 def _select_cdf(score, q_cmp, k_cmp, cdf_threshold, sm_scale, k_min, order="score"):
@@ -235,7 +235,7 @@ def _select_cdf(score, q_cmp, k_cmp, cdf_threshold, sm_scale, k_min, order="scor
 
 
 def get_select_indices_cdf_from_score(score: torch.Tensor, cdf_threshold: float, sm_scale: float):
-    """bsa_interface.py:233-243.  Indices int64 [B,H,nbq,min(nbk,1024)]: row m holds its selection in
+    """bsa_interface.py:233-243.  Indices int64 [B,H,nbq,nbk]: row m holds its selection in
     descending score order up to lens[m] and -1 behind (the reference returns all nbk sorted columns, of
     which only the first lens[m] are ever read); lens int32."""
     idx, lens, _ = _select_cdf(score, None, None, cdf_threshold, sm_scale, 0)

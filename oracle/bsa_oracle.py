@@ -190,7 +190,7 @@ def select_cdf(score: torch.Tensor, cdf_threshold: float, sm_scale: float, k_min
     leaves ties unspecified; the softmax is monotone in the score); the weights are fp32 for every score
     dtype (the reference's bf16 route stops at a dtype check inside torch.searchsorted, bsa:236-241); the
     running sum is kept in float64, so a row can differ from an fp32 running sum only where that sum comes
-    within rounding of the threshold.  `cap` limits lens (the engine keeps at most 1024 blocks per row)."""
+    within rounding of the threshold.  `cap` limits lens (the engine's own entry points take a list width)."""
     s = score.float()
     w = torch.softmax(s * sm_scale, dim=-1)
     order = np.argsort(-s.numpy(), axis=-1, kind="stable")

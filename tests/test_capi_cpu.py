@@ -72,7 +72,7 @@ def test_topk_rejects_bad_arguments():
     lib = _capi.load()
     assert lib.bsa_topk_from_score(FAKE, FAKE, None, FAKE, 1, 1, 4, 4, 5, _capi.BSA_BF16, None) == _capi.BSA_ERR_SHAPE
     assert lib.bsa_topk_from_score(FAKE, FAKE, None, FAKE, 1, 1, 4, 5000, 5, _capi.BSA_BF16, None) == _capi.BSA_ERR_UNSUPPORTED
-    assert lib.bsa_topk_from_score(FAKE, FAKE, None, FAKE, 1, 1, 4, 4096, 2000, _capi.BSA_BF16, None) == _capi.BSA_ERR_UNSUPPORTED
+    assert lib.bsa_topk_from_score(FAKE, FAKE, None, FAKE, 1, 1, 4, 4096, 4097, _capi.BSA_BF16, None) == _capi.BSA_ERR_SHAPE
     assert lib.bsa_topk_from_score(None, FAKE, None, FAKE, 1, 1, 4, 4, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_BAD_ARG
     assert lib.bsa_score_topk(FAKE, FAKE, FAKE, None, FAKE, FAKE, 1, 1, 4, 4, 100, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_UNSUPPORTED
     assert lib.bsa_score_topk(FAKE, FAKE, FAKE, None, FAKE, None, 1, 1, 4, 4, 128, 2, _capi.BSA_BF16, None) == _capi.BSA_ERR_BAD_ARG

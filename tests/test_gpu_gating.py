@@ -53,7 +53,7 @@ def test_score_random_within_one_ulp(dtype, ulp):
 
 
 @pytest.mark.parametrize("nbq,nbk,k_sel", [(4, 4, 2), (5, 37, 9), (3, 64, 64), (2, 65, 1), (7, 200, 0), (3, 624, 39),
-                                             (2, 1440, 90), (2, 1248, 156), (1, 2047, 300), (1, 4096, 1024)])
+                                             (2, 1440, 90), (2, 1248, 156), (1, 2047, 300), (1, 4096, 1024), (5, 4096, 3000)])
 def test_topk_bit_exact_with_ties(nbq, nbk, k_sel):
     g = torch.Generator().manual_seed(nbk)
     # few distinct values => many exact ties, resolved towards the lowest index
@@ -73,6 +73,49 @@ def test_topk_random_scores_all_dtypes(dtype):
     assert torch.equal(got, want)
     vals = torch.gather(score.float(), -1, got)
     assert torch.equal(vals, torch.topk(score.float(), 41).values)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_topk_rows_on_both_sides_of_the_histogram_window(dtype):
+    """For 16-bit scores the kernel first looks for the k-th largest value within 254 codes below the row maximum
+    (a histogram) and otherwise searches bit by bit.  Rows built from bit patterns so that the k-th largest value
+    lies 0, 1, 253, 254, 255, 256 and thousands of codes below the maximum, with ties at the threshold, across
+    zero, and with a maximum so small that its distance to the padding code would fit the window."""
+    nbk, k = 333, 20
+    base = 0x3C00 if dtype == torch.float16 else 0x3F80          # 1.0
+    rows = []
+    for gap in (0, 1, 253, 254, 255, 256, 5000):
+        codes = np.full(nbk, base - gap - 300, dtype=np.int64)       # the crowd, far below
+        codes[5:5 + k - 4] = base                                    # k - 4 columns at the maximum
+        codes[100:110] = base - gap                                  # ten tied columns of which four win (lowest index)
+        rows.append(codes)
+    # positive and negative values around zero: codes of -x sort below every positive code
+    mixed = np.full(nbk, 0x8000 | (base - 7), dtype=np.int64)        # about -1
+    mixed[::17] = 3                                                  # tiny positives: the winners, all tied
+    rows.append(mixed)
+    # a row of tiny values: maximum = code 2 (a denormal), the rest zero or negative zero
+    tiny = np.zeros(nbk, dtype=np.int64)
+    tiny[50] = 2
+    tiny[51::3] = 0x8000
+    rows.append(tiny)
+    bits = torch.from_numpy(np.stack(rows).astype(np.uint16).view(np.int16))
+    score = bits.view(dtype).view(1, 1, len(rows), nbk)
+    for kk in (k, 1, 150):
+        got, lens = topk_gpu(score, kk)
+        want, want_lens = O.select_topk(score, kk)
+        assert torch.equal(lens, want_lens)
+        assert torch.equal(got, want), kk
+
+
+def test_topk_long_lists_of_fp32_scores():
+    """2 500 of 4 096 columns of fp32 scores in score order: the ranking keeps 64-bit keys of four rows in LDS,
+    more than the 64 KB a kernel gets without asking."""
+    g = torch.Generator().manual_seed(13)
+    score = torch.randn(1, 1, 6, 4096, generator=g)
+    score[0, 0, 2] = (score[0, 0, 2] * 4).round() / 4                  # a row full of ties
+    got, lens = topk_gpu(score, 2500)
+    want, want_lens = O.select_topk(score, 2500)
+    assert torch.equal(lens, want_lens) and torch.equal(got, want)
 
 
 def test_block_ordered_list_is_the_same_set_in_ascending_order():
@@ -134,7 +177,7 @@ def check_cdf_selection(score, idx, lens, thr, scale, k_min=0):
     """idx/lens from the GPU against the oracle on the same scores: the count may only differ where the
     running sum comes within rounding of the threshold; given the count, the list is the oracle's order."""
     nbk = score.shape[-1]
-    cap = min(nbk, 1024)
+    cap = nbk                                           # a row may keep every block
     want_idx, want_lens, cdf = O.select_cdf(score, thr, scale, k_min=k_min, cap=cap)
     lens = lens.cpu().long()
     near = (cdf - float(np.float32(thr))).abs().min(-1).values < 1e-5
@@ -178,7 +221,7 @@ def test_cdf_selection_edge_cases():
     big = torch.randn(1, 1, 3, 1440, generator=torch.Generator().manual_seed(22)).bfloat16()
     idx, lens = I().get_select_indices_cdf_from_score(big.cuda(), 0.95, 1.0)
     check_cdf_selection(big, idx, lens, 0.95, 1.0)
-    assert idx.shape[-1] == 1024 and int(lens.max()) <= 1024               # at most 1024 blocks per row
+    assert idx.shape[-1] == 1440 and 1024 < int(lens.max()) <= 1440        # rows that keep more than 1 024 blocks
 
 
 def test_cdf_selection_from_pooled_vectors_and_dispatch():

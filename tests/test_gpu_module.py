@@ -66,6 +66,44 @@ def test_linear_with_bias_and_residual():
     assert torch.all((got_nb.float() - (want - b.float())).abs() <= (want - b.float()).abs() * BF16_ULP + 2e-3)
 
 
+def test_linear_from_several_threads_on_their_own_streams():
+    """Linear layers called from four host threads at once, each on its own stream and with its own shapes, give
+    what they give when called alone (the GEMM wrapper keeps one library handle per thread and shares only its
+    table of chosen algorithms)."""
+    import threading
+    g = torch.Generator().manual_seed(40)
+    jobs = []
+    for n_out, rows in ((384, 200), (512, 333), (640, 128), (384, 200)):
+        x = torch.randint(-2, 3, (rows, 512), generator=g).bfloat16().cuda()          # small integers: exact
+        w = torch.randint(-2, 3, (n_out, 512), generator=g).bfloat16().cuda()
+        b = torch.randint(-2, 3, (n_out,), generator=g).bfloat16().cuda()
+        jobs.append((x, w, b, M().linear_bf16(x, w, b)))
+    torch.cuda.synchronize()
+    failures = []
+
+    def worker(job):
+        x, w, b, want = job
+        stream = torch.cuda.Stream()
+        try:
+            with torch.cuda.stream(stream):
+                for _ in range(25):
+                    got = M().linear_bf16(x, w, b)
+                    stream.synchronize()
+                    if not torch.equal(got, want):
+                        failures.append("mismatch")
+                        return
+        except Exception as exc:                                       # noqa: BLE001 - reported through the list
+            failures.append(repr(exc))
+
+    threads = [threading.Thread(target=worker, args=(j,)) for j in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+    assert not failures, failures
+    assert all(not t.is_alive() for t in threads)
+
+
 def test_qk_norm_rope_against_the_oracle():
     grid = (3, 5, 7)
     S = 105
