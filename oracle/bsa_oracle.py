@@ -49,6 +49,13 @@ fixtures for this path, so the pins are mathematical; see tests/test_oracle_*):
                                     W + m*a*U.D exactly; split up-projection ==
                                     one block-diagonal matrix; torch F.linear
 
+  inverse_block_lists               brute-force loop over the mask
+  blockwise_attention_backward      torch.autograd through an fp32 masked-dense
+                                    softmax attention written with plain torch
+                                    ops (an independent derivation): equal to
+                                    rounding in fp32, within the stated bf16
+                                    tolerance otherwise; finite differences on
+                                    a tiny case; delta == rowsum(o * do)
   paced_visit_order                 (no reference counterpart: the reference
                                     visits the selected blocks in list order,
                                     and the result does not depend on that
@@ -333,6 +340,99 @@ def blockwise_attention(q, k, v, idx, lens, bs_q: int, bs_k: int, sm_scale: floa
                 M[b, h, mblk * bs_q:(mblk + 1) * bs_q] = m_i + torch.log2(l_i)
                 o[b, h, mblk * bs_q:(mblk + 1) * bs_q] = (acc / l_i.unsqueeze(1)).to(dt)
     return o, M * LN2
+
+
+# --------------------------------------------------------------------------
+# backward (bsa:341-461, vmask:288-945)
+# --------------------------------------------------------------------------
+RCP_LN2 = 1.4426950408889634     # bsa:359, 369
+
+
+def inverse_block_lists(idx: torch.Tensor, lens: torch.Tensor, n_kv_blocks: int):
+    """create_indices_k_from_indices_q_varlen, bsa:152-165: for every KV block the query blocks that selected it,
+    ascending.  Returns (lists [B,H,nbk,nbq] int64 padded with nbq, counts [B,H,nbk])."""
+    mask = block_mask_from_indices(idx, lens, n_kv_blocks)              # [B,H,nbq,nbk]
+    B, H, nbq, nbk = mask.shape
+    mk = mask.permute(0, 1, 3, 2)
+    ids = torch.arange(nbq).view(1, 1, 1, -1).expand_as(mk)
+    lists = torch.where(mk, ids, torch.full_like(ids, nbq)).sort(dim=-1).values
+    return lists, (lists < nbq).sum(dim=-1)
+
+
+def blockwise_attention_backward(q, k, v, o, do, lse, idx, lens, bs_q: int, bs_k: int, sm_scale: float,
+                                 key_valid: Optional[torch.Tensor] = None):
+    """Restatement of the reference backward's numerics (bsa:341-461; kernels vmask:288-360, 428-462, wrappers
+    vmask:630-642, 943-945):
+      M2 = lse * RCP_LN2 (fp32); k_s = k * (sm_scale * RCP_LN2) in k's dtype (one rounding, bsa:369-370);
+      delta = rowsum(o * do) in fp32 (common.py:105-109);
+      per (query block, selected KV block): s = q . k_s^T (fp32), p = exp2(s - M2), dp = do . v^T (fp32),
+      ds = p * (dp - delta) rounded to the storage type, p rounded to the storage type for dV;
+      dV = sum p^T do, dK = (sum ds^T q) * sm_scale, dQ = (sum ds k_s) * LN2, fp32 accumulators, one final rounding.
+    dQ walks a row's blocks in list order, dK / dV walk the query blocks of a KV block in ascending order
+    (bsa:389-392); fp32 summation order inside a product is free.  Padded keys (extension) have p = 0.
+    Returns (dq, dk, dv) in the input dtype."""
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    nbq, nbk = Sq // bs_q, Sk // bs_k
+    dt = q.dtype
+    ln2 = 0.6931471824645996                                  # vmask:943 (tl.constexpr LN2)
+    m2 = lse.float() * RCP_LN2
+    k_s = k * (sm_scale * RCP_LN2)                            # stays in k's dtype
+    delta = (o.float() * do.float()).sum(-1)
+    dq = torch.zeros(B, H, Sq, D, dtype=torch.float32)
+    dk = torch.zeros(B, H, Sk, D, dtype=torch.float32)
+    dv = torch.zeros(B, H, Sk, D, dtype=torch.float32)
+    inv, inv_n = inverse_block_lists(idx, lens, nbk)
+
+    def pair(b, h, m, j):
+        qs = q[b, h, m * bs_q:(m + 1) * bs_q]
+        ks = k_s[b, h, j * bs_k:(j + 1) * bs_k]
+        vs = v[b, h, j * bs_k:(j + 1) * bs_k]
+        dos = do[b, h, m * bs_q:(m + 1) * bs_q]
+        s = qs.float() @ ks.float().t()
+        p = torch.exp2(s - m2[b, h, m * bs_q:(m + 1) * bs_q].unsqueeze(1))
+        if key_valid is not None:
+            p = torch.where(key_valid[j * bs_k:(j + 1) * bs_k].unsqueeze(0), p, torch.zeros_like(p))
+        dp = dos.float() @ vs.float().t()
+        ds = (p * (dp - delta[b, h, m * bs_q:(m + 1) * bs_q].unsqueeze(1))).to(dt)
+        return qs, ks, dos, p.to(dt), ds
+
+    for b in range(B):
+        for h in range(H):
+            for m in range(nbq):                                            # dQ: list order (vmask:469-499)
+                seen = set()
+                for i in range(int(lens[b, h, m])):
+                    j = int(idx[b, h, m, i])
+                    if j in seen:                                           # a mask has no duplicates
+                        continue
+                    seen.add(j)
+                    qs, ks, dos, p, ds = pair(b, h, m, j)
+                    dq[b, h, m * bs_q:(m + 1) * bs_q] += ds.float() @ ks.float()
+            for j in range(nbk):                                            # dK, dV: ascending query blocks (vmask:327-356)
+                for i in range(int(inv_n[b, h, j])):
+                    m = int(inv[b, h, j, i])
+                    qs, ks, dos, p, ds = pair(b, h, m, j)
+                    dv[b, h, j * bs_k:(j + 1) * bs_k] += p.float().t() @ dos.float()
+                    dk[b, h, j * bs_k:(j + 1) * bs_k] += ds.float().t() @ qs.float()
+    return (dq * ln2).to(dt), (dk * sm_scale).to(dt), dv.to(dt)
+
+
+def masked_dense_attention_autograd(q, k, v, do, block_mask, bs_q: int, bs_k: int, sm_scale: float,
+                                    key_valid: Optional[torch.Tensor] = None):
+    """The tolerance oracle of the backward: gradients of fp32 softmax(Q K^T * sm_scale + mask) V by
+    torch.autograd.  Returns (dq, dk, dv) fp32."""
+    qf, kf, vf = (t.detach().float().requires_grad_(True) for t in (q, k, v))
+    allow = block_mask.repeat_interleave(bs_q, dim=2).repeat_interleave(bs_k, dim=3)
+    if key_valid is not None:
+        allow = allow & key_valid.view(1, 1, 1, -1)
+    logits = (qf @ kf.transpose(-1, -2)) * sm_scale
+    logits = logits.masked_fill(~allow, -math.inf)
+    none = ~allow.any(-1, keepdim=True)
+    p = torch.softmax(logits.masked_fill(none, 0.0), dim=-1)
+    p = torch.where(allow, p, torch.zeros_like(p))
+    out = p @ vf
+    out.backward(do.float())
+    return qf.grad, kf.grad, vf.grad
 
 
 PACE_WIDTH = 8
