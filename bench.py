@@ -1,6 +1,6 @@
 """Benchmark of the block-sparse attention forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|bwd]
 
 A step is one pass of the whole operator (chunk mean pooling of q and k, pooled
 scores, top-k, block-sparse flash attention that gathers its tiles from the
@@ -249,6 +249,68 @@ def run_c4(torch, args):
     print(json.dumps(result))
 
 
+def run_bwd(torch, args):
+    """Backward of the blocked-order operator (bsa_bwd) at the c3 geometry: 32 heads x 128, 1440 query and KV blocks of
+    64 tokens, 90 selected blocks per row from the operator's own gating.  A step is one backward pass (row sums,
+    scaled k, bit matrix, seven fragment-order passes, dQ kernel, dK/dV kernel); the forward is not in it."""
+    from longcat_video_amd.block_sparse_attention import bsa_interface as I
+    latent, sparsity, seed, rms, desc = WORKLOADS["c3"]
+    q, k, v = make_inputs(torch, latent, seed, rms)
+    qp, kp, vp = (I._permute(t, latent, CHUNK)[0] for t in (q, k, v))
+    del q, k, v
+    sm = 1 / math.sqrt(D)
+    idx, lens = I._select_blocked(qp, kp, 64, 64, sparsity, None)
+    o, lse = I.attn_fwd_bsa_varlen(qp, kp, vp, sm, idx, lens, 64, 64)
+    do = torch.randn(o.shape, generator=torch.Generator(device="cuda").manual_seed(seed + 100), device="cuda").bfloat16()
+    dq, dk, dv = (torch.empty_like(t) for t in (qp, kp, vp))
+    step = lambda: I.attn_bwd_bsa_varlen(do, qp, kp, vp, o, dq, dk, dv, sm, lse, idx, lens, 64, 64)
+    for _ in range(min(args.warmup, 2)):
+        step()
+    torch.cuda.synchronize()
+    steps = min(args.steps, 5)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    assert all(bool(torch.isfinite(t.float()).all()) for t in (dq, dk, dv))
+    pairs = HEADS * idx.shape[2] * idx.shape[3]
+    flop = pairs * 7 * 2 * 64 * 64 * D       # q.k_s and do.v (each in both kernels), dV, dK, dQ
+    tflops = flop / ms / 1e9
+    result = {
+        "metric": "BSA bwd ms/layer + TFLOPS at 720p 86.4k tokens (blocked order)", "value": round(tflops, 2),
+        "unit": "TFLOP/s (seven 64x64x128 products per selected block pair)", "n_gpus": 1, "steps": steps, "warmup": min(args.warmup, 2),
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic N(0,1) q/k/v with per-head RMS-normalised q/k and N(0,1) output gradient, seeded on the GPU",
+        "config": {"workload": "bwd: backward of the c3 layer in blocked order, 32 heads x 128, 1440 x 1440 blocks of 64, 90 per row",
+                   "block_pairs": pairs},
+        "roofline": {"kernel": "bwd_dq_kernel<bf16> + bwd_dkdv_kernel<bf16> (with the passes before them)", "bound": "mfma",
+                     "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": None, "ms": round(ms, 4)}}
+    if not args.no_cpu_baseline:
+        from oracle import bsa_oracle as O
+        cores = os.cpu_count() or 1
+        torch.set_num_threads(cores)
+        hq, hk, hv = host_inputs(torch, qp.shape[2], seed, rms)
+        hdo = torch.randn(hq.shape, generator=torch.Generator().manual_seed(seed + 100)).bfloat16()
+        score = O.cal_score(O.mean_pooling_compression(hq, 64), O.mean_pooling_compression(hk, 64))
+        hidx, hlens = O.select_topk(score, idx.shape[3])
+        nq = 128                                                         # query blocks of the sample
+        mask = O.block_mask_from_indices(hidx[:, :, :nq], hlens[:, :, :nq], score.shape[-1])
+        ho, hlse = O.masked_dense_attention(hq[:, :, :nq * 64], hk, hv, mask, 64, 64, sm)
+        t0 = time.perf_counter()
+        O.blockwise_attention_backward(hq[:, :, :nq * 64], hk, hv, ho.bfloat16(), hdo[:, :, :nq * 64], hlse, hidx[:, :, :nq], hlens[:, :, :nq],
+                                       64, 64, sm)
+        sec = time.perf_counter() - t0
+        layer_s = sec * pairs / (nq * idx.shape[3])
+        result["cpu_baseline"] = {
+            "value": round(flop / layer_s / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port", "ms_per_layer": round(layer_s * 1e3, 1),
+            "sample": "1 of %d heads, inputs drawn on the host from the same distribution (a separate draw): the oracle's backward "
+                      "of %d of 1440 query blocks with their %d selected blocks each (%.2f s), scaled linearly to all block pairs"
+                      % (HEADS, nq, idx.shape[3], sec)}
+    print(json.dumps(result))
+
+
 def run_c5(torch, args):
     """benchmark configuration 5: the attention sub-chain of one DiT block at 720p: RMSNorm -> QKV projection ->
     per-head RMSNorm + 3-D RoPE -> block-sparse attention -> output projection + residual (dim 4096)."""
@@ -358,9 +420,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4", "c5"],
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4", "c5", "bwd"],
                     help="c3 is the headline (default); c2 the same operator at 480p; c4 the cond/noise split of a long "
-                         "video; c5 the attention module around the operator")
+                         "video; c5 the attention module around the operator; bwd the backward of the c3 layer")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the CPU baseline's attention sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm-tuning", action="store_true", help="c5: leave the GEMM algorithm choice to hipBLASLt's first proposal")
@@ -381,6 +443,8 @@ def main():
         return run_c4(torch, args)
     if args.workload == "c5":
         return run_c5(torch, args)
+    if args.workload == "bwd":
+        return run_bwd(torch, args)
     latent, sparsity, seed, rms, desc = WORKLOADS[args.workload]
     coherent = args.data == "coherent"
     q, k, v = make_coherent_inputs(torch, latent, seed) if coherent else make_inputs(torch, latent, seed, rms)

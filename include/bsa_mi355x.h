@@ -216,6 +216,26 @@ int bsa_fwd_3d(const bsa_3d_params* p,
                int32_t* idx_out, int32_t* lens_out, void* score_out, void* stream);
 
 /*
+ * Backward of bsa_fwd: gradients of the block-sparse attention with respect to q, k and v.
+ * Replaces attn_bwd_bsa_varlen_triton (bsa:341-461) and the kernels _attn_bwd_preprocess (common.py:94-111),
+ * _attn_bwd_dkdv_bsa_varlen_wrapper (vmask:505-642) and _attn_bwd_dq_bsa_varlen(_align)_wrapper (vmask:665-945),
+ * including create_indices_k_from_indices_q_varlen (bsa:152-165), with their rounding points: k pre-scaled by
+ * sm_scale*log2(e) and rounded once to the storage type, p = exp2(q.k_s - lse*log2(e)) in fp32, p and
+ * dS = p*(dP - delta) rounded to the storage type for the products, fp32 accumulators, dK scaled by sm_scale and dQ
+ * by ln 2 before the final rounding.
+ *   q, o, d_o, dq [B, Hn, Sq, D]; k, v, dk, dv [B, Hn, Sk, D]: contiguous, blocked order, bf16 / fp16, D == 128.
+ *   lse [B, Hn, Sq] fp32 (natural log) and idx / lens as bsa_fwd took and returned them (a row names a block at
+ *   most once); tile_valid as in bsa_fwd (padded keys get no gradient and give none).
+ *   workspace: bsa_bwd_workspace_bytes() bytes, 256-byte aligned (seven fragment-order copies of q / k / v / d_o
+ *   sized tensors, the scaled k, two fp32 vectors per query row, a bit matrix [kv block][query block]).
+ */
+size_t bsa_bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int D, int bs_q, int bs_k, int dtype);
+int bsa_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+            const int32_t* idx, const int32_t* lens, const uint64_t* tile_valid, void* dq, void* dk, void* dv, int B,
+            int Hn, int64_t Sq, int64_t Sk, int D, int bs_q, int bs_k, int idx_stride, float sm_scale, int dtype,
+            void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * bsa_fwd_3d without a workspace argument and without any allocation.  It has no counterpart in the
  * reference; it is for callers that cannot allocate device memory around the call: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  What bsa_fwd_3d carves from its workspace

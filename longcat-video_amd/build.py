@@ -21,12 +21,12 @@ OUT_DIR = os.path.join(HERE, "longcat_video_amd", "lib")
 LIB = os.path.join(OUT_DIR, "libbsa_mi355x.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["bsa_capi.hip", "bsa_permute.hip", "bsa_select.hip", "bsa_fwd.hip", "bsa_fwd_frag.hip", "bsa_glue.hip"]
+SOURCES = ["bsa_capi.hip", "bsa_permute.hip", "bsa_select.hip", "bsa_fwd.hip", "bsa_fwd_frag.hip", "bsa_bwd.hip", "bsa_glue.hip"]
 # The attention kernel never produces a NaN by construction (the -inf cases are guarded), so its
 # maxima need no NaN-quieting extra instructions.  Infinities keep their IEEE meaning.
 # The glue kernels restate eager fp32 expressions (x * cos + rot * sin, x * (scale + 1) + shift, x + gate * y)
 # whose products and sums are rounded one by one: no contraction into FMAs there (explicit fmaf stays an FMA).
-EXTRA_FLAGS = {"bsa_fwd.hip": ["-fno-honor-nans"], "bsa_fwd_frag.hip": ["-fno-honor-nans"], "bsa_glue.hip": ["-ffp-contract=off"]}
+EXTRA_FLAGS = {"bsa_fwd.hip": ["-fno-honor-nans"], "bsa_fwd_frag.hip": ["-fno-honor-nans"], "bsa_bwd.hip": ["-fno-honor-nans"], "bsa_glue.hip": ["-ffp-contract=off"]}
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -1,0 +1,451 @@
+// Block-sparse flash-attention backward for gfx950 (bf16 / fp16 MFMA), blocked-order tensors.
+//
+// Follows the reference's backward (bsa_interface.py:341-461; kernels flash_attn_bsa_varlen_mask.py:288-360
+// for dK/dV and :428-462 for dQ, wrappers :630-642 and :943-945) with the same rounding points:
+//   M2 = lse * log2(e);  k_s = k * (sm_scale * log2(e)) rounded once to the storage type;
+//   delta = rowsum(o * do) in fp32;
+//   per (query block, selected KV block): s = q . k_s^T, p = exp2(s - M2), dp = do . v^T (all fp32),
+//   ds = p * (dp - delta) rounded to the storage type, p rounded to the storage type for dV;
+//   dV = sum p^T do,  dK = sm_scale * sum ds^T q,  dQ = ln 2 * sum ds k_s  (fp32 accumulators, one final rounding).
+//
+// Data movement as in bsa_fwd_frag.hip: every operand that an MFMA reads from memory is first rewritten into
+// fragment order (frag_kernel), so a wavefront loads it with one coalesced 16-byte load per lane and fragment and
+// LDS carries nothing.  "row layout" = the K layout of that file (A operand whose rows are tokens), "transposed
+// layout" = its V layout (A operand whose rows are head-dim columns, contraction over 16 tokens in accumulator
+// order).  Needed: k_s in both layouts and v in row layout (dQ); q and do in both layouts (dK, dV).
+//
+// dQ: one wavefront per 32 query rows.  S^T = K_s Q^T and dP^T = V dO^T (Q and dO rows in registers as B operands)
+// put one query per lane, so M2 and delta are one scalar per lane and dS^T in the accumulator registers is already
+// the B operand of dQ^T += K_s^T dS^T.
+// dK, dV: one wavefront per 32 keys.  S = Q K_s^T and dP = dO V^T (K_s and V rows in registers as B operands) put
+// one key per lane; P and dS in the accumulator registers are the B operands of dV^T += dO^T P and dK^T += Q^T dS.
+// The query blocks of a KV block come from a bit matrix [KV block][query block] that a small kernel fills from
+// the forward's lists (ascending order for free).  Lists are expected to name a block at most once, as a
+// selection does; for a repeated block dQ follows the list (as the forward does) and dK / dV the bit matrix, like
+// the reference.
+#include "bsa_mfma.h"
+
+namespace bsa {
+namespace {
+
+using namespace mfma;
+
+constexpr float kRcpLn2 = 1.4426950408889634f;
+
+// ------------------------------------------------------------------ small passes
+// delta[row] = sum_d o * do (fp32), m2[row] = lse * log2(e), +inf for rows without any key (their p is then 0).
+// One 16-lane group per row.
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_rows_kernel(const T* __restrict__ o, const T* __restrict__ dout,
+                                                       const float* __restrict__ lse, float* __restrict__ delta,
+                                                       float* __restrict__ m2, int64_t rows) {
+    typedef typename Vec8<T>::type V8;
+    const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int c = threadIdx.x & 15;
+    float s = 0.f;
+    if (row < rows) {
+        const V8 a = *reinterpret_cast<const V8*>(o + row * kD + c * 8);
+        const V8 b = *reinterpret_cast<const V8*>(dout + row * kD + c * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s += (float)a[e] * (float)b[e];
+    }
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off);
+    if (row < rows && c == 0) {
+        delta[row] = s;
+        const float l = lse[row];
+        m2[row] = l == -INFINITY ? INFINITY : l * kRcpLn2;
+    }
+}
+
+// k_s = k * c, rounded once to the storage type (the product is formed in fp32, as torch does for a tensor times
+// a Python scalar).
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_scale_kernel(const T* __restrict__ k, T* __restrict__ ks, float c, int64_t n8) {
+    typedef typename Vec8<T>::type V8;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n8) return;
+    V8 x = *reinterpret_cast<const V8*>(k + i * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * c);
+    *reinterpret_cast<V8*>(ks + i * 8) = x;
+}
+
+__global__ void bwd_zero_kernel(uint32_t* p, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+// bits[bh][kv block][query block / 32] |= 1 << (query block % 32) for every list entry; block indices are clamped
+// to the valid range as the forward kernels do.
+__global__ __launch_bounds__(256) void bwd_mask_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ lens,
+                                                       uint32_t* __restrict__ bits, int nbq, int nbk, int stride,
+                                                       int words, int64_t rows) {
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const int64_t bh = row / nbq;
+    const int m = (int)(row % nbq);
+    const int n = min(max(lens[row], 0), stride);
+    for (int e = lane; e < n; e += 64) {
+        const int j = min(max(idx[row * stride + e], 0), nbk - 1);
+        atomicOr(bits + (bh * nbk + j) * words + (m >> 5), 1u << (m & 31));
+    }
+}
+
+// ------------------------------------------------------------------ fragment access
+// row layout: [tile][half h][d step c][lane][8];  transposed layout: [tile][half h][16-row step s][d tile t][lane][8]
+template <typename V8>
+__device__ __forceinline__ V8 frag_row(const char* base, int64_t tile, int h, int c, uint32_t lane_off) {
+    return *reinterpret_cast<const V8*>(base + tile * kTileBytes + h * (kTileBytes / 2) + c * 1024 + lane_off);
+}
+template <typename V8>
+__device__ __forceinline__ V8 frag_tr(const char* base, int64_t tile, int h, int s, int t, uint32_t lane_off) {
+    return *reinterpret_cast<const V8*>(base + tile * kTileBytes + h * (kTileBytes / 2) + (4 * s + t) * 1024 + lane_off);
+}
+
+template <typename T, typename V8>
+__device__ __forceinline__ V8 pack8(const f32x16& x, int s) {
+    V8 r;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[j] = (T)x[8 * s + j];
+    return r;
+}
+
+// ------------------------------------------------------------------ dQ
+template <typename T>
+__global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, const T* __restrict__ dout,
+                                                    const char* __restrict__ ks_row, const char* __restrict__ ks_tr,
+                                                    const char* __restrict__ v_row, const float* __restrict__ m2,
+                                                    const float* __restrict__ delta, const int32_t* __restrict__ idx,
+                                                    const int32_t* __restrict__ lens,
+                                                    const uint64_t* __restrict__ tile_valid, T* __restrict__ dq,
+                                                    int64_t Sq, int64_t Sk, int bs_q, int bs_k, int stride) {
+    typedef typename Vec8<T>::type V8;
+    const int lane = threadIdx.x, lr = lane & 31, lh = lane >> 5;
+    const uint32_t lane_off = (uint32_t)lane * 16u;
+    const int64_t groups = Sq / 32;
+    const int64_t item = blockIdx.x;
+    const int64_t bh = item / groups;
+    const int64_t qrow0 = (item % groups) * 32;
+    const int nbq = (int)(Sq / bs_q), nbk = (int)(Sk / bs_k), nsub = bs_k / kTile;
+    const int64_t lrow = bh * nbq + qrow0 / bs_q;
+    const int n = min(max(lens[lrow], 0), stride);
+    const int32_t* list = idx + lrow * stride;
+    const int64_t kv_tiles = Sk / kTile;
+    const char* ksr = ks_row + bh * kv_tiles * kTileBytes;
+    const char* kst = ks_tr + bh * kv_tiles * kTileBytes;
+    const char* vr = v_row + bh * kv_tiles * kTileBytes;
+
+    const int64_t row = bh * Sq + qrow0 + lr;
+    V8 qreg[8], doreg[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        qreg[c] = *reinterpret_cast<const V8*>(q + row * kD + 16 * c + 8 * lh);
+        doreg[c] = *reinterpret_cast<const V8*>(dout + row * kD + 16 * c + 8 * lh);
+    }
+    const float m_row = m2[row], d_row = delta[row];
+    f32x16 acc[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+
+    // The fragments of a half tile (K_s rows, V rows, K_s transposed: 24 KB) are requested one half ahead of their
+    // use, into two register buffers that take turns.
+    struct Frags { V8 k[8], v[8], t[8]; };
+    auto load = [&](Frags& f, int64_t tile, int h) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) f.k[c] = frag_row<V8>(ksr, tile, h, c, lane_off);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) f.v[c] = frag_row<V8>(vr, tile, h, c, lane_off);
+#pragma unroll
+        for (int x = 0; x < 8; ++x) f.t[x] = frag_tr<V8>(kst, tile, h, x >> 2, x & 3, lane_off);
+    };
+    auto compute = [&](const Frags& f, uint32_t hv) {
+        f32x16 s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { s[i] = 0.f; dp[i] = 0.f; }
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            s = mfma32(f.k[c], qreg[c], s);
+            dp = mfma32(f.v[c], doreg[c], dp);
+        }
+        // accumulator i <-> key 8 (i / 4) + 4 lh + i % 4 of the half, query lr
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int key = 8 * (i / 4) + 4 * lh + (i % 4);
+            float p = __builtin_amdgcn_exp2f(s[i] - m_row);
+            if (!((hv >> key) & 1u)) p = 0.f;
+            s[i] = p * (dp[i] - d_row);
+        }
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+            const V8 ds = pack8<T, V8>(s, st);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc[t] = mfma32(f.t[4 * st + t], ds, acc[t]);
+        }
+    };
+    const int ntiles = n * nsub;
+    auto tile_at = [&](int tp) -> int64_t {
+        const int tc = min(tp, ntiles - 1);
+        return (int64_t)min(max(list[tc / nsub], 0), nbk - 1) * nsub + tc % nsub;
+    };
+    if (ntiles > 0) {
+        Frags fa, fb;
+        int64_t tile = tile_at(0);
+        load(fa, tile, 0);
+        for (int tp = 0; tp < ntiles; ++tp) {
+            const uint64_t valid = tile_valid != nullptr ? tile_valid[tile] : ~0ull;
+            load(fb, tile, 1);
+            compute(fa, (uint32_t)valid);
+            const int64_t next = tile_at(tp + 1);
+            load(fa, next, 0);                            // behind the last tile: loaded again, not used
+            compute(fb, (uint32_t)(valid >> 32));
+            tile = next;
+        }
+    }
+    // accumulator i of d tile t <-> d = 32 t + 8 (i / 4) + 4 lh + i % 4, query lr
+    T* out = dq + row * kD;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            T x[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) x[j] = (T)(acc[t][4 * g4 + j] * kLn2);
+            *reinterpret_cast<uint2*>(out + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(x);
+        }
+}
+
+// ------------------------------------------------------------------ dK, dV
+template <typename T>
+__global__ __launch_bounds__(64) void bwd_dkdv_kernel(const T* __restrict__ ks, const T* __restrict__ v,
+                                                      const char* __restrict__ q_row, const char* __restrict__ q_tr,
+                                                      const char* __restrict__ do_row, const char* __restrict__ do_tr,
+                                                      const float* __restrict__ m2, const float* __restrict__ delta,
+                                                      const uint32_t* __restrict__ bits,
+                                                      const uint64_t* __restrict__ tile_valid, T* __restrict__ dk,
+                                                      T* __restrict__ dv, int64_t Sq, int64_t Sk, int bs_q, int bs_k,
+                                                      int words, float sm_scale) {
+    typedef typename Vec8<T>::type V8;
+    const int lane = threadIdx.x, lr = lane & 31, lh = lane >> 5;
+    const uint32_t lane_off = (uint32_t)lane * 16u;
+    const int64_t groups = Sk / 32;
+    const int64_t item = blockIdx.x;
+    const int64_t bh = item / groups;
+    const int64_t krow0 = (item % groups) * 32;
+    const int nbq = (int)(Sq / bs_q), nbk = (int)(Sk / bs_k), qsub = bs_q / kTile;
+    const int kblk = (int)(krow0 / bs_k);
+    const uint32_t* mask_row = bits + (bh * nbk + kblk) * words;
+    const int64_t q_tiles = Sq / kTile;
+    const char* qr = q_row + bh * q_tiles * kTileBytes;
+    const char* qt = q_tr + bh * q_tiles * kTileBytes;
+    const char* dor = do_row + bh * q_tiles * kTileBytes;
+    const char* dot = do_tr + bh * q_tiles * kTileBytes;
+
+    const int64_t row = bh * Sk + krow0 + lr;
+    V8 kreg[8], vreg[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        kreg[c] = *reinterpret_cast<const V8*>(ks + row * kD + 16 * c + 8 * lh);
+        vreg[c] = *reinterpret_cast<const V8*>(v + row * kD + 16 * c + 8 * lh);
+    }
+    bool key_ok = true;
+    if (tile_valid != nullptr) key_ok = (tile_valid[krow0 / kTile] >> ((krow0 % kTile) + lr)) & 1ull;
+    f32x16 adv[4], adk[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { adv[t][i] = 0.f; adk[t][i] = 0.f; }
+
+    // the query blocks of this KV block, ascending, from the bit matrix into LDS
+    extern __shared__ int32_t qlist[];
+    int count = 0;
+    for (int w0 = 0; w0 < words; w0 += 64) {
+        const int w = w0 + lane;
+        uint32_t word = w < words ? mask_row[w] : 0u;
+        if (w == words - 1 && (nbq & 31)) word &= (1u << (nbq & 31)) - 1u;
+        int mine = __popc(word), upto = mine;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int t = __shfl_up(upto, off);
+            if (lane >= off) upto += t;
+        }
+        int pos = count + upto - mine;
+        while (word != 0u) {
+            qlist[pos++] = 32 * w + __builtin_ctz(word);
+            word &= word - 1u;
+        }
+        count += __shfl(upto, 63);
+    }
+    __syncthreads();
+    // Row fragments of a half tile of queries (Q rows, dO rows: 16 KB) are requested one half ahead of their use,
+    // into two register buffers that take turns; the transposed fragments at the start of the half that uses them.
+    struct Rows { V8 q[8], d[8]; };
+    auto load = [&](Rows& f, int64_t tile, int h) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) f.q[c] = frag_row<V8>(qr, tile, h, c, lane_off);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) f.d[c] = frag_row<V8>(dor, tile, h, c, lane_off);
+    };
+    auto compute = [&](const Rows& f, int64_t tile, int h) {
+        V8 tq[8], td[8];
+#pragma unroll
+        for (int x = 0; x < 8; ++x) td[x] = frag_tr<V8>(dot, tile, h, x >> 2, x & 3, lane_off);
+#pragma unroll
+        for (int x = 0; x < 8; ++x) tq[x] = frag_tr<V8>(qt, tile, h, x >> 2, x & 3, lane_off);
+        // accumulator i <-> query 8 (i / 4) + 4 lh + i % 4 of the half, key lr
+        const int64_t qrow = bh * Sq + tile * kTile + 32 * h + 4 * lh;
+        float4 mm[4], dd[4];
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            mm[g4] = *reinterpret_cast<const float4*>(m2 + qrow + 8 * g4);
+            dd[g4] = *reinterpret_cast<const float4*>(delta + qrow + 8 * g4);
+        }
+        f32x16 s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { s[i] = 0.f; dp[i] = 0.f; }
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            s = mfma32(f.q[c], kreg[c], s);
+            dp = mfma32(f.d[c], vreg[c], dp);
+        }
+        f32x16 p;
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            const float mv[4] = {mm[g4].x, mm[g4].y, mm[g4].z, mm[g4].w}, dl[4] = {dd[g4].x, dd[g4].y, dd[g4].z, dd[g4].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int i = 4 * g4 + j;
+                float pi = __builtin_amdgcn_exp2f(s[i] - mv[j]);
+                if (!key_ok) pi = 0.f;
+                p[i] = pi;
+                s[i] = pi * (dp[i] - dl[j]);
+            }
+        }
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+            const V8 pb = pack8<T, V8>(p, st), dsb = pack8<T, V8>(s, st);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                adv[t] = mfma32(td[4 * st + t], pb, adv[t]);
+                adk[t] = mfma32(tq[4 * st + t], dsb, adk[t]);
+            }
+        }
+    };
+    const int ntiles = count * qsub;
+    auto tile_at = [&](int tp) -> int64_t {
+        const int tc = min(tp, ntiles - 1);
+        return (int64_t)qlist[tc / qsub] * qsub + tc % qsub;
+    };
+    if (ntiles > 0) {
+        Rows fa, fb;
+        int64_t tile = tile_at(0);
+        load(fa, tile, 0);
+        for (int tp = 0; tp < ntiles; ++tp) {
+            load(fb, tile, 1);
+            compute(fa, tile, 0);
+            const int64_t next = tile_at(tp + 1);
+            load(fa, next, 0);                            // behind the last tile: loaded again, not used
+            compute(fb, tile, 1);
+            tile = next;
+        }
+    }
+    // accumulator i of d tile t <-> d = 32 t + 8 (i / 4) + 4 lh + i % 4, key lr
+    T* okk = dk + row * kD;
+    T* ovv = dv + row * kD;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            T x[4], y[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { x[j] = (T)(adk[t][4 * g4 + j] * sm_scale); y[j] = (T)adv[t][4 * g4 + j]; }
+            *reinterpret_cast<uint2*>(okk + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(x);
+            *reinterpret_cast<uint2*>(ovv + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(y);
+        }
+}
+
+}  // namespace
+
+// Workspace of the backward, in bytes: seven fragment-order copies ([B*Hn][S/64][16 KB]: q and do in both
+// layouts, k_s in both, v in row layout), k_s in blocked order, delta and M2, the bit matrix.
+size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k) {
+    const size_t bh = (size_t)B * Hn;
+    auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+    const size_t words = (size_t)((Sq / bs_q + 31) / 32);
+    return 4 * up(bh * Sq * kD * 2) + 4 * up(bh * Sk * kD * 2) + 2 * up(bh * Sq * 4) + up(bh * (Sk / bs_k) * words * 4);
+}
+
+hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
+                      const int32_t* idx, const int32_t* lens, const uint64_t* tile_valid, void* dq, void* dk, void* dv,
+                      int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride, float sm_scale, int dtype,
+                      void* workspace, hipStream_t st) {
+    const size_t bh = (size_t)B * Hn;
+    auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+    char* ws = static_cast<char*>(workspace);
+    auto take = [&](size_t n) { char* p = ws; ws += up(n); return p; };
+    char* q_row = take(bh * Sq * kD * 2);
+    char* q_tr = take(bh * Sq * kD * 2);
+    char* do_row = take(bh * Sq * kD * 2);
+    char* do_tr = take(bh * Sq * kD * 2);
+    char* ks_row = take(bh * Sk * kD * 2);
+    char* ks_tr = take(bh * Sk * kD * 2);
+    char* v_row = take(bh * Sk * kD * 2);
+    char* ks = take(bh * Sk * kD * 2);
+    float* delta = reinterpret_cast<float*>(take(bh * Sq * 4));
+    float* m2 = reinterpret_cast<float*>(take(bh * Sq * 4));
+    const int nbq = (int)(Sq / bs_q), nbk = (int)(Sk / bs_k);
+    const int words = (nbq + 31) / 32;
+    uint32_t* bits = reinterpret_cast<uint32_t*>(take(bh * nbk * (size_t)words * 4));
+
+    const int64_t qrows = (int64_t)bh * Sq, krows = (int64_t)bh * Sk;
+    const float c = sm_scale * kRcpLn2;
+    if (dtype == BSA_BF16) {
+        hipLaunchKernelGGL((bwd_rows_kernel<__bf16>), dim3((unsigned)((qrows + 15) / 16)), dim3(256), 0, st, (const __bf16*)o,
+                           (const __bf16*)dout, lse, delta, m2, qrows);
+        hipLaunchKernelGGL((bwd_scale_kernel<__bf16>), dim3((unsigned)((krows * 16 + 255) / 256)), dim3(256), 0, st,
+                           (const __bf16*)k, (__bf16*)ks, c, krows * 16);
+    } else {
+        hipLaunchKernelGGL((bwd_rows_kernel<_Float16>), dim3((unsigned)((qrows + 15) / 16)), dim3(256), 0, st, (const _Float16*)o,
+                           (const _Float16*)dout, lse, delta, m2, qrows);
+        hipLaunchKernelGGL((bwd_scale_kernel<_Float16>), dim3((unsigned)((krows * 16 + 255) / 256)), dim3(256), 0, st,
+                           (const _Float16*)k, (_Float16*)ks, c, krows * 16);
+    }
+    const int64_t nwords = (int64_t)bh * nbk * words;
+    hipLaunchKernelGGL(bwd_zero_kernel, dim3((unsigned)((nwords + 255) / 256)), dim3(256), 0, st, bits, nwords);
+    const int64_t lrows = (int64_t)bh * nbq;
+    hipLaunchKernelGGL(bwd_mask_kernel, dim3((unsigned)((lrows + 3) / 4)), dim3(256), 0, st, idx, lens, bits, nbq, nbk, idx_stride,
+                       words, lrows);
+    // blocked-order tensors as a grid of 64-token chunks along one axis
+    const Grid3 gq = make_grid((int)(Sq / kTile), 1, kTile, 1, 1, kTile), gk = make_grid((int)(Sk / kTile), 1, kTile, 1, 1, kTile);
+    const int64_t stq[3] = {(int64_t)Hn * Sq * kD, Sq * kD, kD}, stk[3] = {(int64_t)Hn * Sk * kD, Sk * kD, kD};
+    hipError_t e;
+    if ((e = launch_frag(q, stq, q_row, B, Hn, gq, dtype, false, st)) != hipSuccess) return e;
+    if ((e = launch_frag(q, stq, q_tr, B, Hn, gq, dtype, true, st)) != hipSuccess) return e;
+    if ((e = launch_frag(dout, stq, do_row, B, Hn, gq, dtype, false, st)) != hipSuccess) return e;
+    if ((e = launch_frag(dout, stq, do_tr, B, Hn, gq, dtype, true, st)) != hipSuccess) return e;
+    if ((e = launch_frag(ks, stk, ks_row, B, Hn, gk, dtype, false, st)) != hipSuccess) return e;
+    if ((e = launch_frag(ks, stk, ks_tr, B, Hn, gk, dtype, true, st)) != hipSuccess) return e;
+    if ((e = launch_frag(v, stk, v_row, B, Hn, gk, dtype, false, st)) != hipSuccess) return e;
+
+    const dim3 block(64);
+    const size_t lds = (size_t)nbq * sizeof(int32_t);         // a KV block's query blocks (bwd_dkdv_kernel)
+    const dim3 grid_q((unsigned)(bh * (Sq / 32))), grid_k((unsigned)(bh * (Sk / 32)));
+    if (dtype == BSA_BF16) {
+        hipLaunchKernelGGL((bwd_dq_kernel<__bf16>), grid_q, block, 0, st, (const __bf16*)q, (const __bf16*)dout, ks_row, ks_tr, v_row,
+                           m2, delta, idx, lens, tile_valid, (__bf16*)dq, Sq, Sk, bs_q, bs_k, idx_stride);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<__bf16>), grid_k, block, lds, st, (const __bf16*)ks, (const __bf16*)v, q_row, q_tr, do_row,
+                           do_tr, m2, delta, bits, tile_valid, (__bf16*)dk, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words, sm_scale);
+    } else {
+        hipLaunchKernelGGL((bwd_dq_kernel<_Float16>), grid_q, block, 0, st, (const _Float16*)q, (const _Float16*)dout, ks_row, ks_tr,
+                           v_row, m2, delta, idx, lens, tile_valid, (_Float16*)dq, Sq, Sk, bs_q, bs_k, idx_stride);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<_Float16>), grid_k, block, lds, st, (const _Float16*)ks, (const _Float16*)v, q_row, q_tr,
+                           do_row, do_tr, m2, delta, bits, tile_valid, (_Float16*)dk, (_Float16*)dv, Sq, Sk, bs_q, bs_k, words,
+                           sm_scale);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace bsa

@@ -228,6 +228,45 @@ int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, con
     return e == hipSuccess ? BSA_OK : hip_fail(e, "fwd launch");
 }
 
+static int check_bwd_shape(int B, int Hn, int64_t Sq, int64_t Sk, int D, int bs_q, int bs_k, int dtype) {
+    if (dtype != BSA_BF16 && dtype != BSA_F16) return set_error(BSA_ERR_UNSUPPORTED, "bwd: dtype %d is not built (bf16, fp16)", dtype);
+    if (D != 128) return set_error(BSA_ERR_UNSUPPORTED, "bwd: head dim %d is not built (only 128)", D);
+    if (B <= 0 || Hn <= 0 || Sq <= 0 || Sk <= 0)
+        return set_error(BSA_ERR_BAD_ARG, "bwd: sizes must be positive (B=%d heads=%d Sq=%lld Sk=%lld)", B, Hn, (long long)Sq, (long long)Sk);
+    if ((int64_t)B * Hn > 65535) return set_error(BSA_ERR_UNSUPPORTED, "B*heads exceeds 65535");
+    if (bs_q <= 0 || bs_k <= 0 || bs_q % 64 != 0 || bs_k % 64 != 0)
+        return set_error(BSA_ERR_UNSUPPORTED, "bwd: chunk sizes %d/%d must be multiples of 64", bs_q, bs_k);
+    if (Sq % bs_q != 0 || Sk % bs_k != 0)
+        return set_error(BSA_ERR_SHAPE, "bwd: Sq=%lld / Sk=%lld are not multiples of the chunk sizes %d / %d", (long long)Sq, (long long)Sk, bs_q, bs_k);
+    if ((Sq / 32) * (int64_t)B * Hn > 0x7fffffffLL || (Sk / 32) * (int64_t)B * Hn > 0x7fffffffLL)
+        return set_error(BSA_ERR_UNSUPPORTED, "bwd: problem too large (32-bit work item indices)");
+    return BSA_OK;
+}
+
+size_t bsa_bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int D, int bs_q, int bs_k, int dtype) {
+    if (check_bwd_shape(B, Hn, Sq, Sk, D, bs_q, bs_k, dtype) != BSA_OK) return 0;
+    return bwd_workspace_bytes(B, Hn, Sq, Sk, bs_q, bs_k);
+}
+
+int bsa_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+            const int32_t* idx, const int32_t* lens, const uint64_t* tile_valid, void* dq, void* dk, void* dv, int B,
+            int Hn, int64_t Sq, int64_t Sk, int D, int bs_q, int bs_k, int idx_stride, float sm_scale, int dtype,
+            void* workspace, size_t workspace_bytes, void* stream) {
+    if (!q || !k || !v || !o || !d_o || !lse || !idx || !lens || !dq || !dk || !dv || !workspace)
+        return set_error(BSA_ERR_BAD_ARG, "bwd: null pointer");
+    BSA_TRY(check_bwd_shape(B, Hn, Sq, Sk, D, bs_q, bs_k, dtype));
+    if (idx_stride <= 0 || idx_stride > 4096) return set_error(BSA_ERR_BAD_ARG, "bwd: idx_stride=%d outside [1, 4096]", idx_stride);
+    if (!(sm_scale > 0.f) || !std::isfinite(sm_scale)) return set_error(BSA_ERR_BAD_ARG, "bwd: sm_scale must be positive and finite");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) ||
+        !aligned16(dv) || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return set_error(BSA_ERR_BAD_ARG, "bwd: tensors must be 16-byte aligned, the workspace 256-byte aligned");
+    const size_t need = bwd_workspace_bytes(B, Hn, Sq, Sk, bs_q, bs_k);
+    if (workspace_bytes < need) return set_error(BSA_ERR_WORKSPACE, "bwd: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+    const hipError_t e = launch_bwd(q, k, v, o, d_o, lse, idx, lens, tile_valid, dq, dk, dv, B, Hn, Sq, Sk, bs_q, bs_k, idx_stride,
+                                    sm_scale, dtype, workspace, (hipStream_t)stream);
+    return e == hipSuccess ? BSA_OK : hip_fail(e, "bwd launch");
+}
+
 // ---- whole operator -------------------------------------------------------
 namespace {
 struct Plan {

@@ -45,11 +45,6 @@ def _need_gpu(*tensors: torch.Tensor) -> None:
             raise RuntimeError("the block-sparse attention engine runs on the GPU only; got a %s tensor" % t.device)
 
 
-def _no_grad(*tensors: torch.Tensor) -> None:
-    if torch.is_grad_enabled() and any(t.requires_grad for t in tensors):
-        raise RuntimeError("block-sparse attention is forward-only here; call it under torch.no_grad()")
-
-
 def _stream(t: torch.Tensor) -> C.c_void_p:
     return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
@@ -314,14 +309,42 @@ def attn_fwd_bsa_varlen(q, k, v, sm_scale, block_indices, block_indices_lens, ch
 attn_fwd_bsa_varlen_triton = attn_fwd_bsa_varlen   # the reference's name for the same entry
 
 
-def flash_attn_bsa(q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold, sm_scale,
-                   tile_valid: Optional[torch.Tensor] = None):
-    """bsa_interface.py:535-568, 598 (``_attention_bsa.apply``) on blocked-order
-    tensors: pool, score, top-k, attention.  Returns ``o`` only, like the reference."""
-    _no_grad(q, k, v)
+def attn_bwd_bsa_varlen(do, q, k, v, o, dq, dk, dv, sm_scale, M, block_indices, block_indices_lens, chunk_size_q,
+                        chunk_size_k, sparsity=None, tile_valid: Optional[torch.Tensor] = None):
+    """bsa_interface.py:343-461 (attn_bwd_bsa_varlen_triton): gradients of the blocked-order attention into the
+    caller's ``dq``, ``dk``, ``dv``.  ``M`` is the natural-log sum-exp the forward returned.  bf16 / fp16."""
+    _need_gpu(do, q, k, v, o, dq, dk, dv, M, block_indices, block_indices_lens)
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    if q.dtype == torch.float32:
+        raise NotImplementedError("the backward is built for bf16 and fp16")
+    for t, like in ((do, q), (o, q), (dq, q), (dk, k), (dv, k), (v, k)):
+        assert t.shape == like.shape and t.dtype == q.dtype
+    for t in (dq, dk, dv):
+        assert t.is_contiguous(), "dq, dk, dv are written in place and must be contiguous"
+    do, q, k, v, o = (t.contiguous() for t in (do, q, k, v, o))
+    lse = M.to(torch.float32).contiguous()
+    idx = block_indices.to(torch.int32).contiguous()
+    lens = block_indices_lens.to(torch.int32).contiguous()
+    assert idx.shape[:3] == (B, H, Sq // chunk_size_q) and lens.shape == idx.shape[:3] and lse.shape == (B, H, Sq)
+    lib = _capi.load()
+    need = lib.bsa_bwd_workspace_bytes(B, H, Sq, Sk, D, int(chunk_size_q), int(chunk_size_k), _code(q))
+    if need == 0:
+        raise RuntimeError("bsa_bwd: " + lib.bsa_last_error().decode())
+    ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        _capi.check(lib.bsa_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(idx), _ptr(lens),
+                                _ptr(tile_valid), _ptr(dq), _ptr(dk), _ptr(dv), B, H, Sq, Sk, D, int(chunk_size_q),
+                                int(chunk_size_k), idx.shape[3], float(sm_scale), _code(q), _ptr(ws), need, _stream(q)),
+                    "bsa_bwd")
+
+
+attn_bwd_bsa_varlen_triton = attn_bwd_bsa_varlen   # the reference's name for the same entry
+
+
+def _select_blocked(q, k, chunk_size_q, chunk_size_k, sparsity, cdf_threshold):
+    """Gating of the blocked-order operator (bsa_interface.py:546-549): lists in ascending block order."""
     D = q.shape[-1]
-    assert D == k.shape[-1] and D == v.shape[-1]
-    assert D in {16, 32, 64, 128, 256}
     q_cmp = mean_pooling_compression(q, chunk_size_q)
     k_cmp = mean_pooling_compression(k, chunk_size_k)
     if sparsity is None and cdf_threshold is None:
@@ -331,6 +354,46 @@ def flash_attn_bsa(q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold,
         idx, lens, _ = _select_cdf(None, q_cmp, k_cmp, cdf_threshold, 1 / D ** 0.5, k_min, order="block")   # bsa:229, 248
     else:
         idx, lens, _ = _score_topk(q_cmp, k_cmp, num_selected(sparsity, k_cmp.shape[2]), order="block")
+    return idx, lens
+
+
+class _AttentionBsa(torch.autograd.Function):
+    """bsa_interface.py:535-596 (``_attention_bsa``): the blocked-order operator with its backward.  The gating
+    (pooling, scores, selection) gets no gradient, as in the reference."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold, sm_scale, tile_valid):
+        idx, lens = _select_blocked(q, k, chunk_size_q, chunk_size_k, sparsity, cdf_threshold)
+        o, lse = attn_fwd_bsa_varlen(q, k, v, sm_scale, idx, lens, chunk_size_q, chunk_size_k, sparsity, tile_valid)
+        ctx.save_for_backward(q, k, v, o, lse, idx, lens)
+        ctx.args = (sm_scale, chunk_size_q, chunk_size_k, sparsity, tile_valid)
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, o, lse, idx, lens = ctx.saved_tensors
+        sm_scale, chunk_size_q, chunk_size_k, sparsity, tile_valid = ctx.args
+        dq, dk, dv = (torch.empty(t.shape, dtype=t.dtype, device=t.device) for t in (q, k, v))
+        attn_bwd_bsa_varlen(do, q, k, v, o, dq, dk, dv, sm_scale, lse, idx, lens, chunk_size_q, chunk_size_k, sparsity,
+                            tile_valid)
+        return dq, dk, dv, None, None, None, None, None, None
+
+
+def _wants_grad(*tensors: torch.Tensor) -> bool:
+    return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+
+
+def flash_attn_bsa(q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold, sm_scale,
+                   tile_valid: Optional[torch.Tensor] = None):
+    """bsa_interface.py:535-568, 598 (``_attention_bsa.apply``) on blocked-order
+    tensors: pool, score, top-k, attention.  Returns ``o`` only, like the reference.  With inputs that
+    require a gradient (bf16 / fp16) the call is recorded for autograd."""
+    if _wants_grad(q, k, v):
+        return _AttentionBsa.apply(q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold, sm_scale, tile_valid)
+    D = q.shape[-1]
+    assert D == k.shape[-1] and D == v.shape[-1]
+    assert D in {16, 32, 64, 128, 256}
+    idx, lens = _select_blocked(q, k, chunk_size_q, chunk_size_k, sparsity, cdf_threshold)
     o, _ = attn_fwd_bsa_varlen(q, k, v, sm_scale, idx, lens, chunk_size_q, chunk_size_k, sparsity, tile_valid)
     return o
 
@@ -452,6 +515,44 @@ def attn_fwd_bsa_thw(q, k, v, latent_shape_q, latent_shape_k, chunk_3d_shape_q, 
         q, block_indices, block_indices_lens, return_lse, out)
 
 
+class _Bsa3dWithGrad(torch.autograd.Function):
+    """The operator for inputs that require a gradient: bsa_interface.py:646-660 as written there - permute,
+    ``_attention_bsa`` on blocked-order tensors, unpermute - with the permutes' own gradients (each is the other's)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, latent_shape_q, latent_shape_k, sparsity, cdf_threshold, chunk_q, chunk_k):
+        D = q.shape[-1]
+        bs_q, bs_k = int(math.prod(chunk_q)), int(math.prod(chunk_k))
+        qp, _, _ = _permute(q, latent_shape_q, chunk_q)
+        kp, _, valid = _permute(k, latent_shape_k, chunk_k, want_valid=True)
+        vp, _, _ = _permute(v, latent_shape_k, chunk_k)
+        padded_k = kp.shape[2] != k.shape[2]
+        idx, lens = _select_blocked(qp, kp, bs_q, bs_k, sparsity, cdf_threshold)
+        sm_scale = 1 / D ** 0.5
+        op, lse = attn_fwd_bsa_varlen(qp, kp, vp, sm_scale, idx, lens, bs_q, bs_k, sparsity, valid if padded_k else None)
+        ctx.save_for_backward(qp, kp, vp, op, lse, idx, lens, valid)
+        ctx.args = (tuple(latent_shape_q), tuple(latent_shape_k), tuple(chunk_q), tuple(chunk_k), sm_scale, padded_k)
+        return _unpermute(op, latent_shape_q, chunk_q)
+
+    @staticmethod
+    def backward(ctx, do):
+        qp, kp, vp, op, lse, idx, lens, valid = ctx.saved_tensors
+        latent_q, latent_k, chunk_q, chunk_k, sm_scale, padded_k = ctx.args
+        bs_q, bs_k = int(math.prod(chunk_q)), int(math.prod(chunk_k))
+        dop, _, _ = _permute(do, latent_q, chunk_q)                      # padded slots get a zero gradient
+        dqp, dkp, dvp = (torch.empty_like(t) for t in (qp, kp, vp))
+        attn_bwd_bsa_varlen(dop, qp, kp, vp, op, dqp, dkp, dvp, sm_scale, lse, idx, lens, bs_q, bs_k, None,
+                            valid if padded_k else None)
+        return (_unpermute(dqp, latent_q, chunk_q), _unpermute(dkp, latent_k, chunk_k), _unpermute(dvp, latent_k, chunk_k),
+                None, None, None, None, None, None)
+
+
+def _unpermute(xp, latent_shape, chunk):
+    T, Hh, W = (int(x) for x in latent_shape)
+    t, h, w = (int(x) for x in chunk)
+    return rearrange_3d_block_to_THW(xp, -(-T // t), -(-Hh // h), -(-W // w), t, h, w, xp.shape[-1], latent_shape=latent_shape)
+
+
 @torch.library.custom_op("longcat_video_amd::flash_attn_bsa_3d", mutates_args=())
 def _bsa_3d_op(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, latent_shape_q: Sequence[int],
                latent_shape_k: Sequence[int], sparsity: float, cdf_threshold: float, chunk_3d_shape_q: Sequence[int],
@@ -498,7 +599,11 @@ def flash_attn_bsa_3d(
     assert head_dim_q in {16, 32, 64, 128, 256}
     if sparsity is None and cdf_threshold is None:
         raise ValueError
-    _no_grad(q, k, v)
+    if _wants_grad(q, k, v):
+        if q.dtype == torch.float32:
+            raise NotImplementedError("the backward is built for bf16 and fp16")
+        return _Bsa3dWithGrad.apply(q, k, v, [int(x) for x in latent_shape_q], [int(x) for x in latent_shape_k], sparsity,
+                                    cdf_threshold, [int(x) for x in chunk_3d_shape_q], [int(x) for x in chunk_3d_shape_k])
     return _bsa_3d_op(q, k, v, [int(x) for x in latent_shape_q], [int(x) for x in latent_shape_k],
                       -1.0 if sparsity is None else float(sparsity), -1.0 if cdf_threshold is None else float(cdf_threshold),
                       [int(x) for x in chunk_3d_shape_q], [int(x) for x in chunk_3d_shape_k])

@@ -369,7 +369,8 @@ def blockwise_attention_backward(q, k, v, o, do, lse, idx, lens, bs_q: int, bs_k
       ds = p * (dp - delta) rounded to the storage type, p rounded to the storage type for dV;
       dV = sum p^T do, dK = (sum ds^T q) * sm_scale, dQ = (sum ds k_s) * LN2, fp32 accumulators, one final rounding.
     dQ walks a row's blocks in list order, dK / dV walk the query blocks of a KV block in ascending order
-    (bsa:389-392); fp32 summation order inside a product is free.  Padded keys (extension) have p = 0.
+    (bsa:389-392); fp32 summation order inside a product is free.  Padded keys (extension) have p = 0.  Lists name
+    a block at most once (a selection does); the reference gives a repeated block no consistent meaning.
     Returns (dq, dk, dv) in the input dtype."""
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
@@ -400,12 +401,8 @@ def blockwise_attention_backward(q, k, v, o, do, lse, idx, lens, bs_q: int, bs_k
     for b in range(B):
         for h in range(H):
             for m in range(nbq):                                            # dQ: list order (vmask:469-499)
-                seen = set()
                 for i in range(int(lens[b, h, m])):
                     j = int(idx[b, h, m, i])
-                    if j in seen:                                           # a mask has no duplicates
-                        continue
-                    seen.add(j)
                     qs, ks, dos, p, ds = pair(b, h, m, j)
                     dq[b, h, m * bs_q:(m + 1) * bs_q] += ds.float() @ ks.float()
             for j in range(nbk):                                            # dK, dV: ascending query blocks (vmask:327-356)

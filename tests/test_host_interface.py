@@ -57,15 +57,18 @@ def test_selection_mode_errors():
         I.get_select_indices_from_score(q, None, None)
 
 
-def test_no_cpu_fallback_and_forward_only():
+def test_no_cpu_fallback_with_or_without_gradients():
     q, k, v = qkv()
     with pytest.raises(RuntimeError, match="GPU only"):
         I.flash_attn_bsa_3d(q, k, v, (4, 8, 8), (4, 8, 8), chunk_3d_shape_q=[4, 4, 4], chunk_3d_shape_k=[4, 4, 4])
     with pytest.raises(RuntimeError, match="GPU only"):
         I.mean_pooling_compression(q, 64)
-    q.requires_grad_(True)
-    with pytest.raises(RuntimeError, match="forward-only"):
+    q.requires_grad_(True)                       # the differentiable route runs on the GPU only as well
+    with pytest.raises(RuntimeError, match="GPU only"):
         I.flash_attn_bsa_3d(q, k, v, (4, 8, 8), (4, 8, 8), chunk_3d_shape_q=[4, 4, 4], chunk_3d_shape_k=[4, 4, 4])
+    with pytest.raises(NotImplementedError, match="bf16 and fp16"):
+        I.flash_attn_bsa_3d(q.float().requires_grad_(True), k.float(), v.float(), (4, 8, 8), (4, 8, 8),
+                            chunk_3d_shape_q=[4, 4, 4], chunk_3d_shape_k=[4, 4, 4])
 
 
 def test_num_selected():

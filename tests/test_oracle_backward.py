@@ -99,16 +99,3 @@ def test_finite_differences_on_a_tiny_case():
             args_m = {"q": (tm, k, v), "k": (q, tm, v), "v": (q, k, tm)}[which]
             fd = float((loss(*args_p) - loss(*args_m)) / (2 * eps))
             assert abs(float(grad[pos]) - fd) <= 2e-4 * max(1.0, abs(fd)), (which, pos, float(grad[pos]), fd)
-
-
-def test_duplicate_list_entries_count_once():
-    sm = 1 / math.sqrt(128)
-    q, k, v, do, idx, lens = case(6, 1, 2, 4, 3, torch.float32)
-    idx[0, 0, 1] = torch.tensor([2, 2, 1])
-    lens[0, 0, 1] = 3
-    mask = O.block_mask_from_indices(idx, lens, 4)
-    o, lse = O.masked_dense_attention(q, k, v, mask, 64, 64, sm)
-    got = O.blockwise_attention_backward(q, k, v, o, do, lse, idx, lens, 64, 64, sm)
-    want = O.masked_dense_attention_autograd(q, k, v, do, mask, 64, 64, sm)
-    for a, b in zip(got, want):
-        assert torch.allclose(a, b, rtol=2e-4, atol=2e-5)
