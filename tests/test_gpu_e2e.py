@@ -223,6 +223,31 @@ def test_operator_with_cdf_selection(sparsity):
     assert torch.equal(pub, o)
 
 
+def test_operator_with_cdf_rows_of_more_than_1024_blocks():
+    """A grid of 1 152 blocks and a threshold that keeps nearly all of them: rows of more than 1 024 blocks go
+    through selection, visiting order and the attention kernel at their full length (the reference keeps however
+    many blocks fall under the threshold, bsa_interface.py:233-243)."""
+    latent = (36, 32, 64)
+    S = int(np.prod(latent))
+    q, k, v = seeded_qkv(53, 1, 1, S, S, 128, torch.bfloat16)
+    o, idx, lens, score = I()._bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, None, (4, 4, 4), (4, 4, 4), True,
+                                      cdf_threshold=0.97)
+    nb = 1152
+    assert idx.shape == (1, 1, nb, nb) and int(lens.max()) > 1024
+    want_idx, want_lens, cdf = O.select_cdf(score.cpu(), 0.97, 1 / math.sqrt(128))
+    near = (cdf - float(np.float32(0.97))).abs().min(-1).values < 1e-5
+    assert torch.equal(lens.cpu().long()[~near], want_lens.long()[~near])
+    long_rows = torch.nonzero(lens[0, 0].cpu() > 1024).flatten().tolist()
+    sample = long_rows[:2] + [long_rows[-1], 0]
+    qp, kp, vp = (O.rearrange_thw_to_3d_block(t, latent, (4, 4, 4)) for t in (q, k, v))
+    want_o, _ = O.gathered_attention(qp, kp, vp, idx.cpu().long().clamp(min=0), lens.cpu(), 64, 64, 1 / math.sqrt(128),
+                                     q_blocks=sample)
+    got_p = O.rearrange_thw_to_3d_block(o.cpu(), latent, (4, 4, 4))
+    for m in sample:
+        d = (got_p[:, :, m * 64:(m + 1) * 64].float() - want_o[:, :, m * 64:(m + 1) * 64]).abs()
+        assert d.max() <= MAX_ABS and d.mean() <= MEAN_ABS, (m, float(d.max()))
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_two_batches_on_a_ragged_grid(dtype):
     """Batch and head strides of the direct (T,H,W)-order path: B = 2, three heads, every axis ragged."""
