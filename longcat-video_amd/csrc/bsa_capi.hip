@@ -387,11 +387,16 @@ hipError_t prepare_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, cons
                        hipStream_t st) {
     hipError_t e;
     const bool padded_k = kv_padded(p);
-    if (pool)
+    if (pool && !(pl.frag && pl.gq.chunk() == 64))
         e = launch_permute(q, q_strides, nullptr, w.qc, nullptr, p->B, p->Hn, pl.gq, p->D, p->dtype, st, false, w.qrows, nullptr);
     else    // tables only: one (batch, head) slice of workgroups, no row is read
         e = launch_permute(q, q_strides, nullptr, nullptr, nullptr, 1, 1, pl.gq, p->D, p->dtype, st, false, w.qrows, nullptr);
     if (e != hipSuccess) return e;
+    if (pool && pl.frag && pl.gq.chunk() == 64) {
+        // chunk means of q from the fragment pass run without a destination: the same sums, a faster read
+        e = launch_frag(q, q_strides, nullptr, p->B, p->Hn, pl.gq, p->dtype, false, st, w.qc, nullptr);
+        if (e != hipSuccess) return e;
+    }
     if (pl.frag) {
         // 64-slot chunks: one pass over k gives its fragment order, its chunk means and the validity words
         if (pl.gk.chunk() == 64) {

@@ -143,7 +143,8 @@ void launch_schedule_choice(const int32_t* lens, int nbq, int tiles_per_block, i
 // K or V of a (T, H, W)-ordered tensor in fragment order (bsa_fwd_frag.hip): dst [B*Hn][padded slots / 64][16 KB],
 // padded slots zero; transpose = false for K, true for V.  bf16 / fp16.
 // For K (transpose = false) of 64-slot chunks the pass can also write the chunk means (pooled, [B*Hn][blocks][128],
-// the bits launch_permute's pooling gives) and the tile validity words; both optional.
+// the bits launch_permute's pooling gives) and the tile validity words; both optional.  dst may be null: the pass
+// then only reads (chunk means of q).
 hipError_t launch_frag(const void* src, const int64_t strides[3], void* dst, int B, int Hn, const Grid3& g, int dtype,
                        bool transpose, hipStream_t st, void* pooled = nullptr, uint64_t* tile_valid = nullptr);
 // The attention kernel on fragment-order K and V.  q_rows (optional): token row of every blocked-order query

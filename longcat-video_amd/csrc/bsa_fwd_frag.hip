@@ -114,6 +114,7 @@ __global__ __launch_bounds__(256) void frag_kernel(const T* __restrict__ src, in
             reinterpret_cast<uint16_t*>(pooled)[((int64_t)bh * gridDim.x + blockIdx.x) * kD + threadIdx.x] = bits;
         }
     }
+    if (dst == nullptr) return;                                    // chunk means (and validity words) only
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         T* row = tile + (rg + 16 * i) * kPitch + c16 * 8;          // 8-byte aligned (pitch 264 B)
