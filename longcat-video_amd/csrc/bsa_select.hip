@@ -23,43 +23,59 @@ using mfma::mfma32;
 using mfma::Vec8;
 
 // ---------------------------------------------------------------- score GEMM
-// Workgroup = 4 wavefronts = 128 score rows x up to kScoreCols columns; each wavefront keeps its 32
-// query rows (all 128 d, the A operand) in registers and walks the column tiles, fetching the B
-// fragments of the next tile while the 8 MFMAs of the current one run.  Operands come straight from
-// global memory (the pooled tensors are a few MB and stay in L2; the four wavefronts ask for the same
-// k rows): lane l supplies row l%32 and the 8 consecutive d values 16*s + 8*(l/32) .. +8 of k-step s.
-// A finished 32x32 tile goes through a wavefront-private LDS patch so that it leaves as 16-byte
-// stores (half a row per lane) instead of 2-byte ones.
+// Workgroup = 4 wavefronts = 128 score rows x up to kScoreCols columns.  The pooled key rows of the workgroup's
+// columns (64 KB) are staged in LDS once, with fully coalesced loads; each wavefront keeps its 32 pooled query rows
+// (all 128 d, the A operand) in registers and walks the 32-column tiles, reading the B fragments from LDS (lane l:
+// row l%32 of the tile, the 8 consecutive d values 16*s + 8*(l/32) .. +8 of k-step s).  Read from global memory
+// fragment by fragment instead, every load instruction touches 32 rows for 32 bytes each and the four wavefronts
+// ask for the same rows again: the L1 path, not the 17 GFLOP of arithmetic, then sets the time (0.107 ms at
+// 1440 x 1440 x 32 heads).  A finished 32x32 tile goes through a wavefront-private LDS patch so that it leaves
+// as 16-byte stores (half a row per lane) instead of 2-byte ones.
 constexpr int kScoreCols = 256;
+constexpr int kScorePitch = 128 + 8;     // elements: 272-byte rows keep 16-byte alignment and spread the banks
 template <typename T>
 __global__ __launch_bounds__(256) void score_mfma_kernel(const T* __restrict__ qc,
                                                          const T* __restrict__ kc,
                                                          T* __restrict__ score, int nbq, int nbk) {
     typedef typename Vec8<T>::type V8;
     constexpr int D = 128;
+    __shared__ __attribute__((aligned(16))) T keys[kScoreCols * kScorePitch];
     __shared__ __attribute__((aligned(16))) T patch[4][32][40];      // 80-byte rows: 16-byte aligned, bank-spread
     const int bh = blockIdx.z;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int m0 = blockIdx.y * 128 + wave * 32;
     const int n_begin = blockIdx.x * kScoreCols;
     const int n_end = min(n_begin + kScoreCols, nbk);
-    if (m0 >= nbq) return;                    // whole wavefront out of range (no workgroup barrier below)
     const int lr = lane & 31, lh = lane >> 5;
+    // the key rows of this workgroup's columns: 16 pieces of 16 bytes per row, consecutive threads on consecutive pieces
+    {
+        const T* kb = kc + ((int64_t)bh * nbk) * D;
+        uint4 piece[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int e = threadIdx.x + 256 * i, r = e >> 4, c = e & 15;
+            piece[i] = *reinterpret_cast<const uint4*>(kb + (int64_t)min(n_begin + r, nbk - 1) * D + c * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int e = threadIdx.x + 256 * i, r = e >> 4, c = e & 15;
+            *reinterpret_cast<uint4*>(keys + r * kScorePitch + c * 8) = piece[i];
+        }
+    }
     const int mrow = min(m0 + lr, nbq - 1);   // clamp: rows past the end are computed, not stored
     const T* qa = qc + ((int64_t)bh * nbq + mrow) * D + lh * 8;
-    V8 a[8], b[8], bn[8];
+    V8 a[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) a[s] = *reinterpret_cast<const V8*>(qa + s * 16);
-    auto load_b = [&](V8* dst, int n0) {
-        const T* kb = kc + ((int64_t)bh * nbk + min(n0 + lr, nbk - 1)) * D + lh * 8;
-#pragma unroll
-        for (int s = 0; s < 8; ++s) dst[s] = *reinterpret_cast<const V8*>(kb + s * 16);
-    };
-    load_b(b, n_begin);
+    __syncthreads();
+    if (m0 >= nbq) return;                    // whole wavefront out of range (no workgroup barrier below)
     T (*mine)[40] = patch[wave];
     const bool vec_ok = (nbk % 8) == 0;       // rows of the score matrix stay 16-byte aligned
     for (int n0 = n_begin; n0 < n_end; n0 += 32) {
-        if (n0 + 32 < n_end) load_b(bn, n0 + 32);
+        const T* kt = keys + (n0 - n_begin + lr) * kScorePitch + lh * 8;
+        V8 b[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) b[s] = *reinterpret_cast<const V8*>(kt + s * 16);
         f32x16 acc;
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.f;
@@ -83,8 +99,6 @@ __global__ __launch_bounds__(256) void score_mfma_kernel(const T* __restrict__ q
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);   // the patch is read before the next tile overwrites it
         __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int s = 0; s < 8; ++s) b[s] = bn[s];
     }
 }
 
