@@ -242,6 +242,18 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
     const int nent = min(min(max(lens[(int64_t)bh * nbq + qblock], 0), idx_stride), kListEntries);
     const int ntiles = nent * nsub;
     const int nsteps = 2 * ntiles;
+    // Q as the B operand of S^T: lane holds rows lr and 32 + lr, d = 16 c + 8 lh .. +8.  Requested before the list
+    // is staged, so that the two chains of dependent loads (row table -> Q rows, list length -> list -> LDS) run
+    // side by side.
+    V8 qreg[2][8];
+#pragma unroll
+    for (int qq = 0; qq < 2; ++qq) {
+        int64_t row = qrow0 + 32 * qq + lr;
+        if (L.q_rows != nullptr) row = max(L.q_rows[row], 0);          // padded slots read token 0, never stored
+        const T* qp = q + q_bh + row * L.q_st[2] + 8 * lh;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) qreg[qq][c] = *reinterpret_cast<const V8*>(qp + 16 * c);
+    }
     // the list goes to LDS: clamped block index (a malformed list gives wrong numbers, never a fault) and the flag
     for (int e = lane; e < nent; e += 64) {
         const int blk = min(max(list[e], 0), nbk - 1);
@@ -253,17 +265,6 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
     __syncthreads();
     const char* kbase = kf + (int64_t)bh * kv_bh_bytes;
     const char* vbase = vf + (int64_t)bh * kv_bh_bytes;
-
-    // Q as the B operand of S^T: lane holds rows lr and 32 + lr, d = 16 c + 8 lh .. +8
-    V8 qreg[2][8];
-#pragma unroll
-    for (int qq = 0; qq < 2; ++qq) {
-        int64_t row = qrow0 + 32 * qq + lr;
-        if (L.q_rows != nullptr) row = max(L.q_rows[row], 0);          // padded slots read token 0, never stored
-        const T* qp = q + q_bh + row * L.q_st[2] + 8 * lh;
-#pragma unroll
-        for (int c = 0; c < 8; ++c) qreg[qq][c] = *reinterpret_cast<const V8*>(qp + 16 * c);
-    }
 
     f32x16 oacc[4][2];
 #pragma unroll
