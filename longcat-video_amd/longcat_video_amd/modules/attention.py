@@ -11,10 +11,12 @@ C-ABI of the engine:
     block-sparse attention               bsa_fwd_3d        (attention.py:58-67, :124-137)
     x = Linear(o)                        bsa_linear_bf16   (attention.py:139-142)
 
-q, k and v are moved from the token-major projection output into per-head
-contiguous tensors by the same pass that normalises and rotates q and k (the
-attention kernel fetches K/V tiles faster from 256-byte-dense heads than from
-rows 24 KB apart), and the attention output is written token-major, so none of
+q is moved from the token-major projection output into a per-head contiguous
+tensor by the same pass that normalises and rotates it (the attention kernel
+fetches query rows tile by tile); k is normalised and rotated where it lies and
+v is used where it lies, since the operator reads both exactly once, to rewrite
+them in the attention kernel's fragment order.  The attention output is written
+token-major, so none of
 the reference's ``.contiguous()`` / ``cat`` / transpose copies (attention.py:127-135,
 :140-141, :166-171) exist here.  Only the block-sparse branch is built: dense back
 ends (flash-attn, xformers) raise ``NotImplementedError``.
@@ -269,13 +271,16 @@ class Attention(nn.Module):
         qs, ks, vs = self._project_qkv(x)
         new = lambda: torch.empty(B, Hn, N, D, dtype=x.dtype, device=x.device)
         eps = self.q_norm.eps
+        # q moves into a per-head tensor on the way (the attention kernel fetches its rows tile by tile); k is normed
+        # and rotated where it lies and v stays where it is: the operator reads both once, to rewrite them in its
+        # fragment order, and a strided read costs that pass less than a separate move costs
         q = norm_rope(qs, new(), self.q_norm.weight, shape, eps=eps)
-        v = norm_rope(vs, new())                                                  # plain move
+        v = vs
         if return_kv:
             k_cache = norm_rope(ks, new(), self.k_norm.weight, eps=eps)           # attention.py:118-119
             k = norm_rope(k_cache, new(), None, shape)
         else:
-            k = norm_rope(ks, new(), self.k_norm.weight, shape, eps=eps)
+            k = norm_rope(ks, ks, self.k_norm.weight, shape, eps=eps)
 
         o = torch.empty(B, N, Hn, D, dtype=x.dtype, device=x.device)             # token-major: reshape below is free
         ov = o.permute(0, 2, 1, 3)                                                # [B, H, N, D] view
@@ -287,7 +292,7 @@ class Attention(nn.Module):
             self._process_attn(q, k, v, shape, out=ov)
         y = self._linear(o.view(B, N, C), self.proj, self.proj_loras, residual=residual)
         if return_kv:
-            return y, (k_cache, v.clone())
+            return y, (k_cache, v.contiguous())
         return y
 
     @torch.no_grad()
