@@ -108,10 +108,21 @@ def make_coherent_inputs(torch, latent, seed):
     return q, q.clone(), v
 
 
-def time_events(torch, fn, steps, warmup):
-    for _ in range(warmup):
+def time_events(torch, fn, steps, warmup, settle_s=0.0):
+    """Average ms per call over `steps` calls between two events on the current stream, after `warmup` calls.
+    settle_s > 0: keep warming up until that much wall time has passed and time at least that long as well, so that
+    a kernel of a millisecond or two is measured at the clock it settles at, not on the ramp after an idle phase."""
+    t0 = time.perf_counter()
+    done = 0
+    while done < warmup or time.perf_counter() - t0 < settle_s:
         fn()
+        done += 1
+        if done % 8 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
+    if settle_s > 0 and done > 0:
+        per_call = (time.perf_counter() - t0) / done
+        steps = max(steps, int(settle_s / max(per_call, 1e-6)) + 1)
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(steps):
@@ -216,7 +227,7 @@ def run_c4(torch, args):
         _, idx, lens, _ = I._bsa_3d(a, b, c, lq, lk, 0.875, CHUNK, CHUNK, want_selection=True)
         idx = operator_lists(I, idx, lens, lk)
         attend = I.ThwAttention(b, c, lq, lk, CHUNK, CHUNK)
-        ms_attn += time_events(torch, lambda: attend(a, idx, lens, out=o), max(args.steps, 20), 5)
+        ms_attn += time_events(torch, lambda: attend(a, idx, lens, out=o), max(args.steps, 20), 5, settle_s=0.3)
         del attend
     assert torch.equal(out, want), "the separately timed attention kernel must reproduce the operator's output"
     pairs = HEADS * (312 * 39 + 936 * 156)
@@ -353,7 +364,7 @@ def run_c5(torch, args):
     idx = operator_lists(I, idx, lens, latent)
     attend = I.ThwAttention(kd, vd, latent, latent, CHUNK, CHUNK)
     o_buf = torch.empty(1, N, HEADS, D, dtype=x.dtype, device=x.device).permute(0, 2, 1, 3)
-    ms_attn = time_events(torch, lambda: attend(qd, idx, lens, out=o_buf), 20, 5)
+    ms_attn = time_events(torch, lambda: attend(qd, idx, lens, out=o_buf), 20, 5, settle_s=0.3)
     del attend
     qkv_tflops = 2 * N * C * 3 * C / ms_qkv / 1e9
     norm_rope_gbs = 2 * N * C * 2 / ms_norm_rope / 1e6          # one tensor: 708 MB read + 708 MB written
@@ -470,7 +481,7 @@ def main():
     ksteps, kwarm = max(args.steps, 20), max(args.warmup, 5)      # kernels alone: enough calls for a steady clock
     attend = I.ThwAttention(k, v, latent, latent, CHUNK, CHUNK)
     o_buf = torch.empty_like(q)
-    ms_attn = time_events(torch, lambda: attend(q, idx, lens, out=o_buf), ksteps, kwarm)
+    ms_attn = time_events(torch, lambda: attend(q, idx, lens, out=o_buf), ksteps, kwarm, settle_s=0.3)
     assert torch.equal(o_buf, o), "the separately timed attention kernel must reproduce the operator's output"
     del attend, o_buf
     # the other entry points on their own (the permutes are no longer part of the operator for bf16)
