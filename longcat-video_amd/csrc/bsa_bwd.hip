@@ -14,7 +14,7 @@
 // layout" = its V layout (A operand whose rows are head-dim columns, contraction over 16 tokens in accumulator
 // order).  Needed: k_s in both layouts and v in row layout (dQ); q and do in both layouts (dK, dV).
 //
-// dQ: one wavefront per 32 query rows.  S^T = K_s Q^T and dP^T = V dO^T (Q and dO rows in registers as B operands)
+// dQ: one wavefront per 64 query rows (two halves of 32, so that every K_s and V fragment feeds two MFMAs).  S^T = K_s Q^T and dP^T = V dO^T (Q and dO rows in registers as B operands)
 // put one query per lane, so M2 and delta are one scalar per lane and dS^T in the accumulator registers is already
 // the B operand of dQ^T += K_s^T dS^T.
 // dK, dV: one wavefront per 32 keys.  S = Q K_s^T and dP = dO V^T (K_s and V rows in registers as B operands) put
@@ -124,10 +124,10 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
     typedef typename Vec8<T>::type V8;
     const int lane = threadIdx.x, lr = lane & 31, lh = lane >> 5;
     const uint32_t lane_off = (uint32_t)lane * 16u;
-    const int64_t groups = Sq / 32;
+    const int64_t groups = Sq / kTile;
     const int64_t item = blockIdx.x;
     const int64_t bh = item / groups;
-    const int64_t qrow0 = (item % groups) * 32;
+    const int64_t qrow0 = (item % groups) * kTile;
     const int nbq = (int)(Sq / bs_q), nbk = (int)(Sk / bs_k), nsub = bs_k / kTile;
     const int64_t lrow = bh * nbq + qrow0 / bs_q;
     const int n = min(max(lens[lrow], 0), stride);
@@ -137,53 +137,71 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
     const char* kst = ks_tr + bh * kv_tiles * kTileBytes;
     const char* vr = v_row + bh * kv_tiles * kTileBytes;
 
-    const int64_t row = bh * Sq + qrow0 + lr;
-    V8 qreg[8], doreg[8];
+    // two query halves of 32 rows: every K_s / V fragment feeds two MFMAs
+    V8 qreg[2][8], doreg[2][8];
+    float m_row[2], d_row[2];
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-        qreg[c] = *reinterpret_cast<const V8*>(q + row * kD + 16 * c + 8 * lh);
-        doreg[c] = *reinterpret_cast<const V8*>(dout + row * kD + 16 * c + 8 * lh);
+    for (int qq = 0; qq < 2; ++qq) {
+        const int64_t row = bh * Sq + qrow0 + 32 * qq + lr;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            qreg[qq][c] = *reinterpret_cast<const V8*>(q + row * kD + 16 * c + 8 * lh);
+            doreg[qq][c] = *reinterpret_cast<const V8*>(dout + row * kD + 16 * c + 8 * lh);
+        }
+        m_row[qq] = m2[row];
+        d_row[qq] = delta[row];
     }
-    const float m_row = m2[row], d_row = delta[row];
-    f32x16 acc[4];
+    f32x16 acc[4][2];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+        for (int qq = 0; qq < 2; ++qq)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[t][qq][i] = 0.f;
 
-    // The fragments of a half tile (K_s rows, V rows, K_s transposed: 24 KB) are requested one half ahead of their
-    // use, into two register buffers that take turns.
-    struct Frags { V8 k[8], v[8], t[8]; };
+    // The row fragments of a half tile (K_s rows, V rows: 16 KB) are requested one half ahead of their use, into two
+    // register buffers that take turns; the transposed K_s fragments at the start of the half that uses them.
+    struct Frags { V8 k[8], v[8]; };
     auto load = [&](Frags& f, int64_t tile, int h) {
 #pragma unroll
         for (int c = 0; c < 8; ++c) f.k[c] = frag_row<V8>(ksr, tile, h, c, lane_off);
 #pragma unroll
         for (int c = 0; c < 8; ++c) f.v[c] = frag_row<V8>(vr, tile, h, c, lane_off);
-#pragma unroll
-        for (int x = 0; x < 8; ++x) f.t[x] = frag_tr<V8>(kst, tile, h, x >> 2, x & 3, lane_off);
     };
-    auto compute = [&](const Frags& f, uint32_t hv) {
-        f32x16 s, dp;
+    auto compute = [&](const Frags& f, int64_t tile, int h, uint32_t hv) {
+        V8 kt[8];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { s[i] = 0.f; dp[i] = 0.f; }
+        for (int x = 0; x < 8; ++x) kt[x] = frag_tr<V8>(kst, tile, h, x >> 2, x & 3, lane_off);
+        f32x16 s[2], dp[2];
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            s = mfma32(f.k[c], qreg[c], s);
-            dp = mfma32(f.v[c], doreg[c], dp);
-        }
-        // accumulator i <-> key 8 (i / 4) + 4 lh + i % 4 of the half, query lr
+        for (int qq = 0; qq < 2; ++qq)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int key = 8 * (i / 4) + 4 * lh + (i % 4);
-            float p = __builtin_amdgcn_exp2f(s[i] - m_row);
-            if (!((hv >> key) & 1u)) p = 0.f;
-            s[i] = p * (dp[i] - d_row);
-        }
+            for (int i = 0; i < 16; ++i) { s[qq][i] = 0.f; dp[qq][i] = 0.f; }
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+#pragma unroll
+            for (int qq = 0; qq < 2; ++qq) {
+                s[qq] = mfma32(f.k[c], qreg[qq][c], s[qq]);
+                dp[qq] = mfma32(f.v[c], doreg[qq][c], dp[qq]);
+            }
+        // accumulator i <-> key 8 (i / 4) + 4 lh + i % 4 of the half, query lr (+ 32)
+#pragma unroll
+        for (int qq = 0; qq < 2; ++qq)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int key = 8 * (i / 4) + 4 * lh + (i % 4);
+                float p = __builtin_amdgcn_exp2f(s[qq][i] - m_row[qq]);
+                if (!((hv >> key) & 1u)) p = 0.f;
+                s[qq][i] = p * (dp[qq][i] - d_row[qq]);
+            }
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
-            const V8 ds = pack8<T, V8>(s, st);
+            const V8 ds0 = pack8<T, V8>(s[0], st), ds1 = pack8<T, V8>(s[1], st);
 #pragma unroll
-            for (int t = 0; t < 4; ++t) acc[t] = mfma32(f.t[4 * st + t], ds, acc[t]);
+            for (int t = 0; t < 4; ++t) {
+                acc[t][0] = mfma32(kt[4 * st + t], ds0, acc[t][0]);
+                acc[t][1] = mfma32(kt[4 * st + t], ds1, acc[t][1]);
+            }
         }
     };
     const int ntiles = n * nsub;
@@ -198,24 +216,27 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
         for (int tp = 0; tp < ntiles; ++tp) {
             const uint64_t valid = tile_valid != nullptr ? tile_valid[tile] : ~0ull;
             load(fb, tile, 1);
-            compute(fa, (uint32_t)valid);
+            compute(fa, tile, 0, (uint32_t)valid);
             const int64_t next = tile_at(tp + 1);
             load(fa, next, 0);                            // behind the last tile: loaded again, not used
-            compute(fb, (uint32_t)(valid >> 32));
+            compute(fb, tile, 1, (uint32_t)(valid >> 32));
             tile = next;
         }
     }
-    // accumulator i of d tile t <-> d = 32 t + 8 (i / 4) + 4 lh + i % 4, query lr
-    T* out = dq + row * kD;
+    // accumulator i of d tile t <-> d = 32 t + 8 (i / 4) + 4 lh + i % 4, query lr (+ 32)
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int qq = 0; qq < 2; ++qq) {
+        T* out = dq + (bh * Sq + qrow0 + 32 * qq + lr) * kD;
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-            T x[4];
+        for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) x[j] = (T)(acc[t][4 * g4 + j] * kLn2);
-            *reinterpret_cast<uint2*>(out + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(x);
-        }
+            for (int g4 = 0; g4 < 4; ++g4) {
+                T x[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) x[j] = (T)(acc[t][qq][4 * g4 + j] * kLn2);
+                *reinterpret_cast<uint2*>(out + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(x);
+            }
+    }
 }
 
 // ------------------------------------------------------------------ dK, dV
@@ -432,7 +453,7 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
 
     const dim3 block(64);
     const size_t lds = (size_t)nbq * sizeof(int32_t);         // a KV block's query blocks (bwd_dkdv_kernel)
-    const dim3 grid_q((unsigned)(bh * (Sq / 32))), grid_k((unsigned)(bh * (Sk / 32)));
+    const dim3 grid_q((unsigned)(bh * (Sq / kTile))), grid_k((unsigned)(bh * (Sk / 32)));
     if (dtype == BSA_BF16) {
         hipLaunchKernelGGL((bwd_dq_kernel<__bf16>), grid_q, block, 0, st, (const __bf16*)q, (const __bf16*)dout, ks_row, ks_tr, v_row,
                            m2, delta, idx, lens, tile_valid, (__bf16*)dq, Sq, Sk, bs_q, bs_k, idx_stride);
