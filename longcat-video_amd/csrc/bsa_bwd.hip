@@ -14,11 +14,12 @@
 // layout" = its V layout (A operand whose rows are head-dim columns, contraction over 16 tokens in accumulator
 // order).  Needed: k_s in both layouts and v in row layout (dQ); q and do in both layouts (dK, dV).
 //
-// dQ: one wavefront per 64 query rows (two halves of 32, so that every K_s and V fragment feeds two MFMAs).  S^T = K_s Q^T and dP^T = V dO^T (Q and dO rows in registers as B operands)
-// put one query per lane, so M2 and delta are one scalar per lane and dS^T in the accumulator registers is already
+// dQ: one wavefront per 64 query rows (two halves of 32, so that every K_s and V fragment feeds two MFMAs).
+// S^T = K_s Q^T and dP^T = V dO^T (Q and dO rows in registers as B operands) put one query per lane, so M2 and delta are one scalar per lane and dS^T in the accumulator registers is already
 // the B operand of dQ^T += K_s^T dS^T.
-// dK, dV: one wavefront per 32 keys.  S = Q K_s^T and dP = dO V^T (K_s and V rows in registers as B operands) put
-// one key per lane; P and dS in the accumulator registers are the B operands of dV^T += dO^T P and dK^T += Q^T dS.
+// dK, dV: one wavefront per 64 keys and one kernel per gradient.  S = Q K_s^T and dP = dO V^T (K_s and V rows in
+// registers as B operands) put one key per lane; P and dS in the accumulator registers are the B operands of
+// dV^T += dO^T P and dK^T += Q^T dS.
 // The query blocks of a KV block come from a bit matrix [KV block][query block] that a small kernel fills from
 // the forward's lists (ascending order for free).  Lists are expected to name a block at most once, as a
 // selection does; for a repeated block dQ follows the list (as the forward does) and dK / dV the bit matrix, like
@@ -240,45 +241,53 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
 }
 
 // ------------------------------------------------------------------ dK, dV
-template <typename T>
-__global__ __launch_bounds__(64) void bwd_dkdv_kernel(const T* __restrict__ ks, const T* __restrict__ v,
-                                                      const char* __restrict__ q_row, const char* __restrict__ q_tr,
-                                                      const char* __restrict__ do_row, const char* __restrict__ do_tr,
-                                                      const float* __restrict__ m2, const float* __restrict__ delta,
-                                                      const uint32_t* __restrict__ bits,
-                                                      const uint64_t* __restrict__ tile_valid, T* __restrict__ dk,
-                                                      T* __restrict__ dv, int64_t Sq, int64_t Sk, int bs_q, int bs_k,
-                                                      int words, float sm_scale) {
+// One wavefront per 64 keys (one tile), as two halves of 32 so that every streamed Q / dO fragment feeds two MFMAs,
+// and one kernel per gradient - 64 keys of both accumulators (256 registers) plus the resident K_s and V rows and
+// the streamed fragments do not fit one wavefront's 512 registers.  kDK = false: dV (S from Q rows and K_s, P, then
+// dV^T += dO^T P).  kDK = true: dK (S again, dP from dO rows and V, dS, then dK^T += Q^T dS).  S is computed in
+// both: 80 MFMAs per tile pair instead of 64, at half the fragment bytes per MFMA.
+template <typename T, bool kDK>
+__global__ __launch_bounds__(64) void bwd_dkv_kernel(const T* __restrict__ ks, const T* __restrict__ v,
+                                                     const char* __restrict__ q_row, const char* __restrict__ q_tr,
+                                                     const char* __restrict__ do_row, const char* __restrict__ do_tr,
+                                                     const float* __restrict__ m2, const float* __restrict__ delta,
+                                                     const uint32_t* __restrict__ bits,
+                                                     const uint64_t* __restrict__ tile_valid, T* __restrict__ out,
+                                                     int64_t Sq, int64_t Sk, int bs_q, int bs_k, int words, float out_scale) {
     typedef typename Vec8<T>::type V8;
     const int lane = threadIdx.x, lr = lane & 31, lh = lane >> 5;
     const uint32_t lane_off = (uint32_t)lane * 16u;
-    const int64_t groups = Sk / 32;
+    const int64_t groups = Sk / kTile;
     const int64_t item = blockIdx.x;
     const int64_t bh = item / groups;
-    const int64_t krow0 = (item % groups) * 32;
+    const int64_t krow0 = (item % groups) * kTile;
     const int nbq = (int)(Sq / bs_q), nbk = (int)(Sk / bs_k), qsub = bs_q / kTile;
     const int kblk = (int)(krow0 / bs_k);
     const uint32_t* mask_row = bits + (bh * nbk + kblk) * words;
     const int64_t q_tiles = Sq / kTile;
     const char* qr = q_row + bh * q_tiles * kTileBytes;
-    const char* qt = q_tr + bh * q_tiles * kTileBytes;
+    const char* trp = (kDK ? q_tr : do_tr) + bh * q_tiles * kTileBytes;     // transposed operand of the last product
     const char* dor = do_row + bh * q_tiles * kTileBytes;
-    const char* dot = do_tr + bh * q_tiles * kTileBytes;
 
-    const int64_t row = bh * Sk + krow0 + lr;
-    V8 kreg[8], vreg[8];
+    V8 kreg[2][8], vreg[kDK ? 2 : 1][8];
+    bool key_ok[2] = {true, true};
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-        kreg[c] = *reinterpret_cast<const V8*>(ks + row * kD + 16 * c + 8 * lh);
-        vreg[c] = *reinterpret_cast<const V8*>(v + row * kD + 16 * c + 8 * lh);
+    for (int kk = 0; kk < 2; ++kk) {
+        const int64_t row = bh * Sk + krow0 + 32 * kk + lr;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            kreg[kk][c] = *reinterpret_cast<const V8*>(ks + row * kD + 16 * c + 8 * lh);
+            if constexpr (kDK) vreg[kk][c] = *reinterpret_cast<const V8*>(v + row * kD + 16 * c + 8 * lh);
+        }
+        if (tile_valid != nullptr) key_ok[kk] = (tile_valid[krow0 / kTile] >> (32 * kk + lr)) & 1ull;
     }
-    bool key_ok = true;
-    if (tile_valid != nullptr) key_ok = (tile_valid[krow0 / kTile] >> ((krow0 % kTile) + lr)) & 1ull;
-    f32x16 adv[4], adk[4];
+    f32x16 acc[4][2];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { adv[t][i] = 0.f; adk[t][i] = 0.f; }
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[t][kk][i] = 0.f;
 
     // the query blocks of this KV block, ascending, from the bit matrix into LDS
     extern __shared__ int32_t qlist[];
@@ -301,57 +310,67 @@ __global__ __launch_bounds__(64) void bwd_dkdv_kernel(const T* __restrict__ ks, 
         count += __shfl(upto, 63);
     }
     __syncthreads();
-    // Row fragments of a half tile of queries (Q rows, dO rows: 16 KB) are requested one half ahead of their use,
-    // into two register buffers that take turns; the transposed fragments at the start of the half that uses them.
-    struct Rows { V8 q[8], d[8]; };
+    // The Q row fragments of a half tile of queries are requested one half ahead of their use, into two register
+    // buffers that take turns; the dO rows (dK) and the transposed fragments at the start of the half that uses them.
+    struct Rows { V8 q[8]; };
     auto load = [&](Rows& f, int64_t tile, int h) {
 #pragma unroll
         for (int c = 0; c < 8; ++c) f.q[c] = frag_row<V8>(qr, tile, h, c, lane_off);
-#pragma unroll
-        for (int c = 0; c < 8; ++c) f.d[c] = frag_row<V8>(dor, tile, h, c, lane_off);
     };
     auto compute = [&](const Rows& f, int64_t tile, int h) {
-        V8 tq[8], td[8];
+        V8 drow[kDK ? 8 : 1], tr[8];
+        if constexpr (kDK) {
 #pragma unroll
-        for (int x = 0; x < 8; ++x) td[x] = frag_tr<V8>(dot, tile, h, x >> 2, x & 3, lane_off);
+            for (int c = 0; c < 8; ++c) drow[c] = frag_row<V8>(dor, tile, h, c, lane_off);
+        }
 #pragma unroll
-        for (int x = 0; x < 8; ++x) tq[x] = frag_tr<V8>(qt, tile, h, x >> 2, x & 3, lane_off);
-        // accumulator i <-> query 8 (i / 4) + 4 lh + i % 4 of the half, key lr
+        for (int x = 0; x < 8; ++x) tr[x] = frag_tr<V8>(trp, tile, h, x >> 2, x & 3, lane_off);
+        // accumulator i <-> query 8 (i / 4) + 4 lh + i % 4 of the half, key lr (+ 32)
         const int64_t qrow = bh * Sq + tile * kTile + 32 * h + 4 * lh;
-        float4 mm[4], dd[4];
+        f32x16 s[2], dp[kDK ? 2 : 1];
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-            mm[g4] = *reinterpret_cast<const float4*>(m2 + qrow + 8 * g4);
-            dd[g4] = *reinterpret_cast<const float4*>(delta + qrow + 8 * g4);
-        }
-        f32x16 s, dp;
+        for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { s[i] = 0.f; dp[i] = 0.f; }
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            s = mfma32(f.q[c], kreg[c], s);
-            dp = mfma32(f.d[c], vreg[c], dp);
-        }
-        f32x16 p;
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-            const float mv[4] = {mm[g4].x, mm[g4].y, mm[g4].z, mm[g4].w}, dl[4] = {dd[g4].x, dd[g4].y, dd[g4].z, dd[g4].w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int i = 4 * g4 + j;
-                float pi = __builtin_amdgcn_exp2f(s[i] - mv[j]);
-                if (!key_ok) pi = 0.f;
-                p[i] = pi;
-                s[i] = pi * (dp[i] - dl[j]);
+            for (int i = 0; i < 16; ++i) {
+                s[kk][i] = 0.f;
+                if constexpr (kDK) dp[kk][i] = 0.f;
             }
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+                s[kk] = mfma32(f.q[c], kreg[kk][c], s[kk]);
+                if constexpr (kDK) dp[kk] = mfma32(drow[c], vreg[kk][c], dp[kk]);
+            }
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            // M2 and delta of the four queries of this accumulator group, fetched where they are used (L1 hits) so
+            // that they do not sit in registers through the products above
+            const float4 mm = *reinterpret_cast<const float4*>(m2 + qrow + 8 * g4);
+            const float mv[4] = {mm.x, mm.y, mm.z, mm.w};
+            float dl[4] = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (kDK) {
+                const float4 dd = *reinterpret_cast<const float4*>(delta + qrow + 8 * g4);
+                dl[0] = dd.x; dl[1] = dd.y; dl[2] = dd.z; dl[3] = dd.w;
+            }
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int i = 4 * g4 + j;
+                    float pi = __builtin_amdgcn_exp2f(s[kk][i] - mv[j]);
+                    if (!key_ok[kk]) pi = 0.f;
+                    if constexpr (kDK) pi = pi * (dp[kk][i] - dl[j]);
+                    s[kk][i] = pi;                               // P for dV, dS for dK
+                }
         }
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
-            const V8 pb = pack8<T, V8>(p, st), dsb = pack8<T, V8>(s, st);
+            const V8 b0 = pack8<T, V8>(s[0], st), b1 = pack8<T, V8>(s[1], st);
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                adv[t] = mfma32(td[4 * st + t], pb, adv[t]);
-                adk[t] = mfma32(tq[4 * st + t], dsb, adk[t]);
+                acc[t][0] = mfma32(tr[4 * st + t], b0, acc[t][0]);
+                acc[t][1] = mfma32(tr[4 * st + t], b1, acc[t][1]);
             }
         }
     };
@@ -373,19 +392,23 @@ __global__ __launch_bounds__(64) void bwd_dkdv_kernel(const T* __restrict__ ks, 
             tile = next;
         }
     }
-    // accumulator i of d tile t <-> d = 32 t + 8 (i / 4) + 4 lh + i % 4, key lr
-    T* okk = dk + row * kD;
-    T* ovv = dv + row * kD;
+    // accumulator i of d tile t <-> d = 32 t + 8 (i / 4) + 4 lh + i % 4, key lr (+ 32)
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int kk = 0; kk < 2; ++kk) {
+        T* orow = out + (bh * Sk + krow0 + 32 * kk + lr) * kD;
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-            T x[4], y[4];
+        for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) { x[j] = (T)(adk[t][4 * g4 + j] * sm_scale); y[j] = (T)adv[t][4 * g4 + j]; }
-            *reinterpret_cast<uint2*>(okk + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(x);
-            *reinterpret_cast<uint2*>(ovv + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(y);
-        }
+            for (int g4 = 0; g4 < 4; ++g4) {
+                T x[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float a = acc[t][kk][4 * g4 + j];
+                    x[j] = kDK ? (T)(a * out_scale) : (T)a;
+                }
+                *reinterpret_cast<uint2*>(orow + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(x);
+            }
+    }
 }
 
 }  // namespace
@@ -452,19 +475,22 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     if ((e = launch_frag(v, stk, v_row, B, Hn, gk, dtype, false, st)) != hipSuccess) return e;
 
     const dim3 block(64);
-    const size_t lds = (size_t)nbq * sizeof(int32_t);         // a KV block's query blocks (bwd_dkdv_kernel)
-    const dim3 grid_q((unsigned)(bh * (Sq / kTile))), grid_k((unsigned)(bh * (Sk / 32)));
+    const size_t lds = (size_t)nbq * sizeof(int32_t);         // a KV block's query blocks (bwd_dkv_kernel)
+    const dim3 grid_q((unsigned)(bh * (Sq / kTile))), grid_k((unsigned)(bh * (Sk / kTile)));
     if (dtype == BSA_BF16) {
         hipLaunchKernelGGL((bwd_dq_kernel<__bf16>), grid_q, block, 0, st, (const __bf16*)q, (const __bf16*)dout, ks_row, ks_tr, v_row,
                            m2, delta, idx, lens, tile_valid, (__bf16*)dq, Sq, Sk, bs_q, bs_k, idx_stride);
-        hipLaunchKernelGGL((bwd_dkdv_kernel<__bf16>), grid_k, block, lds, st, (const __bf16*)ks, (const __bf16*)v, q_row, q_tr, do_row,
-                           do_tr, m2, delta, bits, tile_valid, (__bf16*)dk, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words, sm_scale);
+        hipLaunchKernelGGL((bwd_dkv_kernel<__bf16, false>), grid_k, block, lds, st, (const __bf16*)ks, (const __bf16*)v, q_row, q_tr,
+                           do_row, do_tr, m2, delta, bits, tile_valid, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words, 1.0f);
+        hipLaunchKernelGGL((bwd_dkv_kernel<__bf16, true>), grid_k, block, lds, st, (const __bf16*)ks, (const __bf16*)v, q_row, q_tr,
+                           do_row, do_tr, m2, delta, bits, tile_valid, (__bf16*)dk, Sq, Sk, bs_q, bs_k, words, sm_scale);
     } else {
         hipLaunchKernelGGL((bwd_dq_kernel<_Float16>), grid_q, block, 0, st, (const _Float16*)q, (const _Float16*)dout, ks_row, ks_tr,
                            v_row, m2, delta, idx, lens, tile_valid, (_Float16*)dq, Sq, Sk, bs_q, bs_k, idx_stride);
-        hipLaunchKernelGGL((bwd_dkdv_kernel<_Float16>), grid_k, block, lds, st, (const _Float16*)ks, (const _Float16*)v, q_row, q_tr,
-                           do_row, do_tr, m2, delta, bits, tile_valid, (_Float16*)dk, (_Float16*)dv, Sq, Sk, bs_q, bs_k, words,
-                           sm_scale);
+        hipLaunchKernelGGL((bwd_dkv_kernel<_Float16, false>), grid_k, block, lds, st, (const _Float16*)ks, (const _Float16*)v, q_row,
+                           q_tr, do_row, do_tr, m2, delta, bits, tile_valid, (_Float16*)dv, Sq, Sk, bs_q, bs_k, words, 1.0f);
+        hipLaunchKernelGGL((bwd_dkv_kernel<_Float16, true>), grid_k, block, lds, st, (const _Float16*)ks, (const _Float16*)v, q_row,
+                           q_tr, do_row, do_tr, m2, delta, bits, tile_valid, (_Float16*)dk, Sq, Sk, bs_q, bs_k, words, sm_scale);
     }
     return hipGetLastError();
 }
