@@ -121,12 +121,21 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
                                                     const float* __restrict__ delta, const int32_t* __restrict__ idx,
                                                     const int32_t* __restrict__ lens,
                                                     const uint64_t* __restrict__ tile_valid, T* __restrict__ dq,
-                                                    int64_t Sq, int64_t Sk, int bs_q, int bs_k, int stride) {
+                                                    int64_t Sq, int64_t Sk, int bs_q, int bs_k, int stride, int item_begin,
+                                                    int item_end, int round) {
     typedef typename Vec8<T>::type V8;
     const int lane = threadIdx.x, lr = lane & 31, lh = lane >> 5;
     const uint32_t lane_off = (uint32_t)lane * 16u;
     const int64_t groups = Sq / kTile;
-    const int64_t item = blockIdx.x;
+    // The launch's items are taken in rounds of `round` (a multiple of 8) in workgroup order; workgroup b runs on
+    // XCD b % 8 and within a round every XCD takes a contiguous run of the round's items, as in the forward kernel:
+    // the items of a round walk their lists together and share K_s / V tiles in L2.
+    int64_t item;
+    {
+        const int local = blockIdx.x, r0 = local / round * round;
+        const int n = min(round, item_end - item_begin - r0), w = local - r0, x = w & 7;
+        item = item_begin + r0 + x * (n >> 3) + min(x, n & 7) + (w >> 3);
+    }
     const int64_t bh = item / groups;
     const int64_t qrow0 = (item % groups) * kTile;
     const int nbq = (int)(Sq / bs_q), nbk = (int)(Sk / bs_k), nsub = bs_k / kTile;
@@ -414,12 +423,14 @@ __global__ __launch_bounds__(64) void bwd_dkv_kernel(const T* __restrict__ ks, c
 }  // namespace
 
 // Workspace of the backward, in bytes: seven fragment-order copies ([B*Hn][S/64][16 KB]: q and do in both
-// layouts, k_s in both, v in row layout), k_s in blocked order, delta and M2, the bit matrix.
-size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k) {
+// layouts, k_s in both, v in row layout), k_s in blocked order, delta and M2, the bit matrix, the lists in the dQ
+// kernel's visiting order.
+size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride) {
     const size_t bh = (size_t)B * Hn;
     auto up = [](size_t x) { return (x + 255) / 256 * 256; };
     const size_t words = (size_t)((Sq / bs_q + 31) / 32);
-    return 4 * up(bh * Sq * kD * 2) + 4 * up(bh * Sk * kD * 2) + 2 * up(bh * Sq * 4) + up(bh * (Sk / bs_k) * words * 4);
+    return 4 * up(bh * Sq * kD * 2) + 4 * up(bh * Sk * kD * 2) + 2 * up(bh * Sq * 4) + up(bh * (Sk / bs_k) * words * 4) +
+           up(bh * (Sq / bs_q) * (size_t)idx_stride * 4);
 }
 
 hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
@@ -443,6 +454,7 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     const int nbq = (int)(Sq / bs_q), nbk = (int)(Sk / bs_k);
     const int words = (nbq + 31) / 32;
     uint32_t* bits = reinterpret_cast<uint32_t*>(take(bh * nbk * (size_t)words * 4));
+    int32_t* paced = reinterpret_cast<int32_t*>(take(bh * nbq * (size_t)idx_stride * 4));
 
     const int64_t qrows = (int64_t)bh * Sq, krows = (int64_t)bh * Sk;
     const float c = sm_scale * kRcpLn2;
@@ -466,6 +478,9 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     const Grid3 gq = make_grid((int)(Sq / kTile), 1, kTile, 1, 1, kTile), gk = make_grid((int)(Sk / kTile), 1, kTile, 1, 1, kTile);
     const int64_t stq[3] = {(int64_t)Hn * Sq * kD, Sq * kD, kD}, stk[3] = {(int64_t)Hn * Sk * kD, Sk * kD, kD};
     hipError_t e;
+    // dQ walks every list in the forward kernel's visiting order when the list is ascending (a selection in block
+    // order); any other order is walked as given.  The order only moves fp32 roundings of the dQ sum.
+    if ((e = launch_pace_order(idx, paced, lens, (int64_t)bh * nbq, nbk, idx_stride, st)) != hipSuccess) return e;
     if ((e = launch_frag(q, stq, q_row, B, Hn, gq, dtype, false, st)) != hipSuccess) return e;
     if ((e = launch_frag(q, stq, q_tr, B, Hn, gq, dtype, true, st)) != hipSuccess) return e;
     if ((e = launch_frag(dout, stq, do_row, B, Hn, gq, dtype, false, st)) != hipSuccess) return e;
@@ -476,17 +491,31 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
 
     const dim3 block(64);
     const size_t lds = (size_t)nbq * sizeof(int32_t);         // a KV block's query blocks (bwd_dkv_kernel)
-    const dim3 grid_q((unsigned)(bh * (Sq / kTile))), grid_k((unsigned)(bh * (Sk / kTile)));
+    const dim3 grid_k((unsigned)(bh * (Sk / kTile)));
+    // dQ: rounds of as many wavefronts as the device runs at once (one per SIMD), two rounds per launch.  The dK / dV
+    // kernels run as one grid: their lists (the query blocks of a KV block) differ in length, and rounds that wait
+    // for the longest list cost more than the shared L2 tiles bring (measured: 62 -> 70-75 ms).
+    int cus = 256, dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    const int round = 4 * (cus > 0 ? cus : 256), span = 2 * round;
+    const int total_q = (int)(bh * (Sq / kTile));
     if (dtype == BSA_BF16) {
-        hipLaunchKernelGGL((bwd_dq_kernel<__bf16>), grid_q, block, 0, st, (const __bf16*)q, (const __bf16*)dout, ks_row, ks_tr, v_row,
-                           m2, delta, idx, lens, tile_valid, (__bf16*)dq, Sq, Sk, bs_q, bs_k, idx_stride);
+        for (int first = 0; first < total_q; first += span) {
+            const int end = first + span < total_q ? first + span : total_q;
+            hipLaunchKernelGGL((bwd_dq_kernel<__bf16>), dim3(end - first), block, 0, st, (const __bf16*)q, (const __bf16*)dout, ks_row,
+                               ks_tr, v_row, m2, delta, paced, lens, tile_valid, (__bf16*)dq, Sq, Sk, bs_q, bs_k, idx_stride, first, end, round);
+        }
         hipLaunchKernelGGL((bwd_dkv_kernel<__bf16, false>), grid_k, block, lds, st, (const __bf16*)ks, (const __bf16*)v, q_row, q_tr,
                            do_row, do_tr, m2, delta, bits, tile_valid, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words, 1.0f);
         hipLaunchKernelGGL((bwd_dkv_kernel<__bf16, true>), grid_k, block, lds, st, (const __bf16*)ks, (const __bf16*)v, q_row, q_tr,
                            do_row, do_tr, m2, delta, bits, tile_valid, (__bf16*)dk, Sq, Sk, bs_q, bs_k, words, sm_scale);
     } else {
-        hipLaunchKernelGGL((bwd_dq_kernel<_Float16>), grid_q, block, 0, st, (const _Float16*)q, (const _Float16*)dout, ks_row, ks_tr,
-                           v_row, m2, delta, idx, lens, tile_valid, (_Float16*)dq, Sq, Sk, bs_q, bs_k, idx_stride);
+        for (int first = 0; first < total_q; first += span) {
+            const int end = first + span < total_q ? first + span : total_q;
+            hipLaunchKernelGGL((bwd_dq_kernel<_Float16>), dim3(end - first), block, 0, st, (const _Float16*)q, (const _Float16*)dout,
+                               ks_row, ks_tr, v_row, m2, delta, paced, lens, tile_valid, (_Float16*)dq, Sq, Sk, bs_q, bs_k, idx_stride, first,
+                               end, round);
+        }
         hipLaunchKernelGGL((bwd_dkv_kernel<_Float16, false>), grid_k, block, lds, st, (const _Float16*)ks, (const _Float16*)v, q_row,
                            q_tr, do_row, do_tr, m2, delta, bits, tile_valid, (_Float16*)dv, Sq, Sk, bs_q, bs_k, words, 1.0f);
         hipLaunchKernelGGL((bwd_dkv_kernel<_Float16, true>), grid_k, block, lds, st, (const _Float16*)ks, (const _Float16*)v, q_row,

@@ -243,9 +243,10 @@ static int check_bwd_shape(int B, int Hn, int64_t Sq, int64_t Sk, int D, int bs_
     return BSA_OK;
 }
 
-size_t bsa_bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int D, int bs_q, int bs_k, int dtype) {
+size_t bsa_bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int D, int bs_q, int bs_k, int idx_stride, int dtype) {
     if (check_bwd_shape(B, Hn, Sq, Sk, D, bs_q, bs_k, dtype) != BSA_OK) return 0;
-    return bwd_workspace_bytes(B, Hn, Sq, Sk, bs_q, bs_k);
+    if (idx_stride <= 0 || idx_stride > 4096) { set_error(BSA_ERR_BAD_ARG, "bwd: idx_stride=%d outside [1, 4096]", idx_stride); return 0; }
+    return bwd_workspace_bytes(B, Hn, Sq, Sk, bs_q, bs_k, idx_stride);
 }
 
 int bsa_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
@@ -260,7 +261,7 @@ int bsa_bwd(const void* q, const void* k, const void* v, const void* o, const vo
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) ||
         !aligned16(dv) || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return set_error(BSA_ERR_BAD_ARG, "bwd: tensors must be 16-byte aligned, the workspace 256-byte aligned");
-    const size_t need = bwd_workspace_bytes(B, Hn, Sq, Sk, bs_q, bs_k);
+    const size_t need = bwd_workspace_bytes(B, Hn, Sq, Sk, bs_q, bs_k, idx_stride);
     if (workspace_bytes < need) return set_error(BSA_ERR_WORKSPACE, "bwd: workspace of %zu bytes, %zu needed", workspace_bytes, need);
     const hipError_t e = launch_bwd(q, k, v, o, d_o, lse, idx, lens, tile_valid, dq, dk, dv, B, Hn, Sq, Sk, bs_q, bs_k, idx_stride,
                                     sm_scale, dtype, workspace, (hipStream_t)stream);

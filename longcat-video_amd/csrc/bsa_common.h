@@ -157,7 +157,7 @@ hipError_t launch_fwd_frag(const void* q, const void* kf, const void* vf, const 
 
 
 // Backward of the blocked-order attention (bsa_bwd.hip), bf16 / fp16.  workspace: bwd_workspace_bytes() bytes.
-size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k);
+size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride);
 hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
                       const int32_t* idx, const int32_t* lens, const uint64_t* tile_valid, void* dq, void* dk, void* dv,
                       int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride, float sm_scale, int dtype,

@@ -328,7 +328,7 @@ def attn_bwd_bsa_varlen(do, q, k, v, o, dq, dk, dv, sm_scale, M, block_indices, 
     lens = block_indices_lens.to(torch.int32).contiguous()
     assert idx.shape[:3] == (B, H, Sq // chunk_size_q) and lens.shape == idx.shape[:3] and lse.shape == (B, H, Sq)
     lib = _capi.load()
-    need = lib.bsa_bwd_workspace_bytes(B, H, Sq, Sk, D, int(chunk_size_q), int(chunk_size_k), _code(q))
+    need = lib.bsa_bwd_workspace_bytes(B, H, Sq, Sk, D, int(chunk_size_q), int(chunk_size_k), idx.shape[3], _code(q))
     if need == 0:
         raise RuntimeError("bsa_bwd: " + lib.bsa_last_error().decode())
     ws = torch.empty(need, dtype=torch.uint8, device=q.device)
