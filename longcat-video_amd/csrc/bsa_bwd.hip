@@ -94,6 +94,16 @@ __global__ __launch_bounds__(256) void bwd_mask_kernel(const int32_t* __restrict
     }
 }
 
+// counts[bh * nbk + j] = number of query blocks that selected KV block j (bits set in its row of the bit matrix)
+__global__ __launch_bounds__(256) void bwd_count_kernel(const uint32_t* __restrict__ bits, int32_t* __restrict__ counts,
+                                                        int words, int64_t rows) {
+    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (row >= rows) return;
+    int c = 0;
+    for (int w = 0; w < words; ++w) c += __popc(bits[row * words + w]);
+    counts[row] = c;
+}
+
 // ------------------------------------------------------------------ fragment access
 // row layout: [tile][half h][d step c][lane][8];  transposed layout: [tile][half h][16-row step s][d tile t][lane][8]
 template <typename V8>
@@ -262,12 +272,22 @@ __global__ __launch_bounds__(64) void bwd_dkv_kernel(const T* __restrict__ ks, c
                                                      const float* __restrict__ m2, const float* __restrict__ delta,
                                                      const uint32_t* __restrict__ bits,
                                                      const uint64_t* __restrict__ tile_valid, T* __restrict__ out,
-                                                     int64_t Sq, int64_t Sk, int bs_q, int bs_k, int words, float out_scale) {
+                                                     int64_t Sq, int64_t Sk, int bs_q, int bs_k, int words, float out_scale,
+                                                     const int32_t* __restrict__ order, int item_begin, int item_end, int round) {
     typedef typename Vec8<T>::type V8;
     const int lane = threadIdx.x, lr = lane & 31, lh = lane >> 5;
     const uint32_t lane_off = (uint32_t)lane * 16u;
     const int64_t groups = Sk / kTile;
-    const int64_t item = blockIdx.x;
+    // Items are taken longest list first (order: the tiles of every (batch, head) by descending number of query
+    // blocks), in groups of `round` workgroups of which every XCD (workgroup b runs on XCD b % 8) takes a contiguous
+    // run: the wavefronts that run side by side have lists of similar length, so they walk the query blocks at a
+    // similar pace and share Q / dO tiles in L2, and the long lists do not end up alone at the tail.
+    int64_t item;
+    {
+        const int local = blockIdx.x, r0 = local / round * round;
+        const int n = min(round, item_end - item_begin - r0), w = local - r0, x = w & 7;
+        item = order[item_begin + r0 + x * (n >> 3) + min(x, n & 7) + (w >> 3)];
+    }
     const int64_t bh = item / groups;
     const int64_t krow0 = (item % groups) * kTile;
     const int nbq = (int)(Sq / bs_q), nbk = (int)(Sk / bs_k), qsub = bs_q / kTile;
@@ -424,13 +444,13 @@ __global__ __launch_bounds__(64) void bwd_dkv_kernel(const T* __restrict__ ks, c
 
 // Workspace of the backward, in bytes: seven fragment-order copies ([B*Hn][S/64][16 KB]: q and do in both
 // layouts, k_s in both, v in row layout), k_s in blocked order, delta and M2, the bit matrix, the lists in the dQ
-// kernel's visiting order.
+// kernel's visiting order, per KV block its number of query blocks, the KV tiles of every head by that number.
 size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride) {
     const size_t bh = (size_t)B * Hn;
     auto up = [](size_t x) { return (x + 255) / 256 * 256; };
     const size_t words = (size_t)((Sq / bs_q + 31) / 32);
     return 4 * up(bh * Sq * kD * 2) + 4 * up(bh * Sk * kD * 2) + 2 * up(bh * Sq * 4) + up(bh * (Sk / bs_k) * words * 4) +
-           up(bh * (Sq / bs_q) * (size_t)idx_stride * 4);
+           up(bh * (Sq / bs_q) * (size_t)idx_stride * 4) + up(bh * (Sk / bs_k) * 4) + up(bh * (Sk / kTile) * 4);
 }
 
 hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
@@ -455,6 +475,8 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     const int words = (nbq + 31) / 32;
     uint32_t* bits = reinterpret_cast<uint32_t*>(take(bh * nbk * (size_t)words * 4));
     int32_t* paced = reinterpret_cast<int32_t*>(take(bh * nbq * (size_t)idx_stride * 4));
+    int32_t* counts = reinterpret_cast<int32_t*>(take(bh * nbk * 4));
+    int32_t* order = reinterpret_cast<int32_t*>(take(bh * (size_t)(Sk / kTile) * 4));
 
     const int64_t qrows = (int64_t)bh * Sq, krows = (int64_t)bh * Sk;
     const float c = sm_scale * kRcpLn2;
@@ -478,6 +500,8 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     const Grid3 gq = make_grid((int)(Sq / kTile), 1, kTile, 1, 1, kTile), gk = make_grid((int)(Sk / kTile), 1, kTile, 1, 1, kTile);
     const int64_t stq[3] = {(int64_t)Hn * Sq * kD, Sq * kD, kD}, stk[3] = {(int64_t)Hn * Sk * kD, Sk * kD, kD};
     hipError_t e;
+    hipLaunchKernelGGL(bwd_count_kernel, dim3((unsigned)((bh * nbk + 255) / 256)), dim3(256), 0, st, bits, counts, words, (int64_t)(bh * nbk));
+    if ((e = launch_order_by_length(counts, order, (int)bh, nbk, bs_k / kTile, nbq, st)) != hipSuccess) return e;
     // dQ walks every list in the forward kernel's visiting order when the list is ascending (a selection in block
     // order); any other order is walked as given.  The order only moves fp32 roundings of the dQ sum.
     if ((e = launch_pace_order(idx, paced, lens, (int64_t)bh * nbq, nbk, idx_stride, st)) != hipSuccess) return e;
@@ -493,12 +517,13 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     const size_t lds = (size_t)nbq * sizeof(int32_t);         // a KV block's query blocks (bwd_dkv_kernel)
     const dim3 grid_k((unsigned)(bh * (Sk / kTile)));
     // dQ: rounds of as many wavefronts as the device runs at once (one per SIMD), two rounds per launch.  The dK / dV
-    // kernels run as one grid: their lists (the query blocks of a KV block) differ in length, and rounds that wait
-    // for the longest list cost more than the shared L2 tiles bring (measured: 62 -> 70-75 ms).
+    // kernels run as one grid each, longest list first: their lists (the query blocks of a KV block) differ in
+    // length, and rounds that wait for the longest list cost more than they bring (measured at the 720p geometry:
+    // one grid in tile order 60.6 ms for the whole backward, rounds 62-75 ms, one grid longest first 54.1 ms).
     int cus = 256, dev = 0;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     const int round = 4 * (cus > 0 ? cus : 256), span = 2 * round;
-    const int total_q = (int)(bh * (Sq / kTile));
+    const int total_q = (int)(bh * (Sq / kTile)), total_k = (int)(bh * (Sk / kTile));
     if (dtype == BSA_BF16) {
         for (int first = 0; first < total_q; first += span) {
             const int end = first + span < total_q ? first + span : total_q;
@@ -506,9 +531,9 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
                                ks_tr, v_row, m2, delta, paced, lens, tile_valid, (__bf16*)dq, Sq, Sk, bs_q, bs_k, idx_stride, first, end, round);
         }
         hipLaunchKernelGGL((bwd_dkv_kernel<__bf16, false>), grid_k, block, lds, st, (const __bf16*)ks, (const __bf16*)v, q_row, q_tr,
-                           do_row, do_tr, m2, delta, bits, tile_valid, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words, 1.0f);
+                           do_row, do_tr, m2, delta, bits, tile_valid, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words, 1.0f, order, 0, total_k, round);
         hipLaunchKernelGGL((bwd_dkv_kernel<__bf16, true>), grid_k, block, lds, st, (const __bf16*)ks, (const __bf16*)v, q_row, q_tr,
-                           do_row, do_tr, m2, delta, bits, tile_valid, (__bf16*)dk, Sq, Sk, bs_q, bs_k, words, sm_scale);
+                           do_row, do_tr, m2, delta, bits, tile_valid, (__bf16*)dk, Sq, Sk, bs_q, bs_k, words, sm_scale, order, 0, total_k, round);
     } else {
         for (int first = 0; first < total_q; first += span) {
             const int end = first + span < total_q ? first + span : total_q;
@@ -517,9 +542,9 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
                                end, round);
         }
         hipLaunchKernelGGL((bwd_dkv_kernel<_Float16, false>), grid_k, block, lds, st, (const _Float16*)ks, (const _Float16*)v, q_row,
-                           q_tr, do_row, do_tr, m2, delta, bits, tile_valid, (_Float16*)dv, Sq, Sk, bs_q, bs_k, words, 1.0f);
+                           q_tr, do_row, do_tr, m2, delta, bits, tile_valid, (_Float16*)dv, Sq, Sk, bs_q, bs_k, words, 1.0f, order, 0, total_k, round);
         hipLaunchKernelGGL((bwd_dkv_kernel<_Float16, true>), grid_k, block, lds, st, (const _Float16*)ks, (const _Float16*)v, q_row,
-                           q_tr, do_row, do_tr, m2, delta, bits, tile_valid, (_Float16*)dk, Sq, Sk, bs_q, bs_k, words, sm_scale);
+                           q_tr, do_row, do_tr, m2, delta, bits, tile_valid, (_Float16*)dk, Sq, Sk, bs_q, bs_k, words, sm_scale, order, 0, total_k, round);
     }
     return hipGetLastError();
 }
