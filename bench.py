@@ -227,7 +227,7 @@ def run_c4(torch, args):
         _, idx, lens, _ = I._bsa_3d(a, b, c, lq, lk, 0.875, CHUNK, CHUNK, want_selection=True)
         idx = operator_lists(I, idx, lens, lk)
         attend = I.ThwAttention(b, c, lq, lk, CHUNK, CHUNK)
-        ms_attn += time_events(torch, lambda: attend(a, idx, lens, out=o), max(args.steps, 20), 5, settle_s=0.3)
+        ms_attn += time_events(torch, lambda: attend(a, idx, lens, out=o), max(args.steps, 20), 5, settle_s=args.settle)
         del attend
     assert torch.equal(out, want), "the separately timed attention kernel must reproduce the operator's output"
     pairs = HEADS * (312 * 39 + 936 * 156)
@@ -364,7 +364,7 @@ def run_c5(torch, args):
     idx = operator_lists(I, idx, lens, latent)
     attend = I.ThwAttention(kd, vd, latent, latent, CHUNK, CHUNK)
     o_buf = torch.empty(1, N, HEADS, D, dtype=x.dtype, device=x.device).permute(0, 2, 1, 3)
-    ms_attn = time_events(torch, lambda: attend(qd, idx, lens, out=o_buf), 20, 5, settle_s=0.3)
+    ms_attn = time_events(torch, lambda: attend(qd, idx, lens, out=o_buf), 20, 5, settle_s=args.settle)
     del attend
     qkv_tflops = 2 * N * C * 3 * C / ms_qkv / 1e9
     norm_rope_gbs = 2 * N * C * 2 / ms_norm_rope / 1e6          # one tensor: 708 MB read + 708 MB written
@@ -436,6 +436,9 @@ def main():
                          "video; c5 the attention module around the operator; bwd the backward of the c3 layer")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the CPU baseline's attention sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--settle", type=float, default=0.3,
+                    help="seconds of warm-up, and at least as many of timing, for the kernel-alone measurements (0: fixed "
+                         "call counts, for runs under a profiler whose per-dispatch averages must weigh every call alike)")
     ap.add_argument("--no-gemm-tuning", action="store_true", help="c5: leave the GEMM algorithm choice to hipBLASLt's first proposal")
     ap.add_argument("--data", default="random", choices=["random", "coherent"],
                     help="random (the benchmark's definition) or spatially coherent q/k (c2, c3 only; no CPU baseline)")
@@ -481,7 +484,7 @@ def main():
     ksteps, kwarm = max(args.steps, 20), max(args.warmup, 5)      # kernels alone: enough calls for a steady clock
     attend = I.ThwAttention(k, v, latent, latent, CHUNK, CHUNK)
     o_buf = torch.empty_like(q)
-    ms_attn = time_events(torch, lambda: attend(q, idx, lens, out=o_buf), ksteps, kwarm, settle_s=0.3)
+    ms_attn = time_events(torch, lambda: attend(q, idx, lens, out=o_buf), ksteps, kwarm, settle_s=args.settle)
     assert torch.equal(o_buf, o), "the separately timed attention kernel must reproduce the operator's output"
     del attend, o_buf
     # the other entry points on their own (the permutes are no longer part of the operator for bf16)
