@@ -376,6 +376,25 @@ int bsa_linear_bf16_tune(const void* x, int64_t ldx, const void* w, int64_t ldw,
 int bsa_lora_add(const void* org, const void* const* up, const float* multiplier, const float* alpha_scale, int n_loras,
                  void* out, int64_t n, int dtype, void* stream);
 
+/* The engine's own GEMM for the two projections of the attention module (attention.py:111 and :142):
+ * out[M,N] = x[M,K] . w[N,K]^T (+ bias[N]) (+ residual[M,N]), bf16 in/out, fp32 accumulation on MFMA, one
+ * rounding at the end.  Row strides in elements (ldx, ldw >= K; ldo, ldr >= N; multiples of 8).  N must be a
+ * multiple of 128 and K of 32; x, w, out, residual 16-byte aligned.  Needs no workspace and allocates nothing. */
+int bsa_gemm_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, const void* bias, const void* residual,
+                  int64_t ldr, void* out, int64_t ldo, int64_t M, int N, int K, void* stream);
+
+/* attention.py:111-121 in one kernel: qkv = Linear(x) with w [3*Hn*128, K] (rows: q heads, k heads, v heads, as
+ * the view/permute of attention.py:112-113 splits them), the projection output rounded to bf16 as the reference's
+ * tensor is, q and k normalised per head (RMSNorm_FP32, blocks.py:42-53, weights q_weight / k_weight of 128
+ * elements) and rotated (rope_3d.py:100-120; rope_table as for bsa_norm_rope, frames t_offset.. of table_T), v
+ * as projected.  x holds M = B*T*H*W token rows.  q, k, v receive [B, Hn, T*H*W, 128] through
+ * dst_strides = {batch, head, token} (elements, multiples of 8): per-head contiguous tensors, or any other
+ * layout bsa_fwd_3d accepts.  Rounding points are those of bsa_norm_rope fed with the bf16 projection. */
+int bsa_qkv_projection(const void* x, int64_t ldx, const void* w, int64_t ldw, const void* bias, const void* q_weight,
+                       const void* k_weight, const float* rope_table, void* q, void* k, void* v,
+                       const int64_t dst_strides[3], int B, int Hn, int T, int H, int W, int t_offset, int table_T,
+                       int D, int K, float eps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

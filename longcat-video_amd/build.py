@@ -21,7 +21,7 @@ OUT_DIR = os.path.join(HERE, "longcat_video_amd", "lib")
 LIB = os.path.join(OUT_DIR, "libbsa_mi355x.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["bsa_capi.hip", "bsa_permute.hip", "bsa_select.hip", "bsa_fwd.hip", "bsa_fwd_frag.hip", "bsa_bwd.hip", "bsa_glue.hip"]
+SOURCES = ["bsa_capi.hip", "bsa_permute.hip", "bsa_select.hip", "bsa_fwd.hip", "bsa_fwd_frag.hip", "bsa_bwd.hip", "bsa_glue.hip", "bsa_gemm.hip"]
 # The attention kernel never produces a NaN by construction (the -inf cases are guarded), so its
 # maxima need no NaN-quieting extra instructions.  Infinities keep their IEEE meaning.
 # The glue kernels restate eager fp32 expressions (x * cos + rot * sin, x * (scale + 1) + shift, x + gate * y)

@@ -64,6 +64,8 @@ SIGNATURES = {
     "bsa_linear_bf16_ld": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i, _i, _p, C.c_size_t, _p]),
     "bsa_linear_bf16_tune": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i64, _i64, _i, _i, _p, C.c_size_t, _p, _p, _p]),
     "bsa_lora_add": (_i, [_p, _p, _p, _p, _i, _p, _i64, _i, _p]),
+    "bsa_gemm_bf16": (_i, [_p, _i64, _p, _i64, _p, _p, _i64, _p, _i64, _i64, _i, _i, _p]),
+    "bsa_qkv_projection": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _strides] + [_i] * 9 + [_f, _p]),
 }
 
 _lib = None

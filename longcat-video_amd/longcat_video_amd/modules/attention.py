@@ -127,6 +127,69 @@ def tune_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
     return n, d.value, best.value
 
 
+def gemm_bf16(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+              residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x @ weight.T + bias (+ residual)`` through the engine's own MFMA GEMM (no workspace, nothing allocated by
+    the library).  weight [N, K] with N a multiple of 128 and K of 64."""
+    if not x.is_cuda:
+        raise RuntimeError("the engine runs on the GPU only")
+    if x.dtype != torch.bfloat16:
+        raise NotImplementedError("gemm: only bf16 is built")
+    K, N = x.shape[-1], weight.shape[0]
+    assert weight.shape[1] == K
+    x2 = x.reshape(-1, K)
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    w = weight.to(torch.bfloat16)
+    if w.stride(1) != 1:
+        w = w.contiguous()
+    b = None if bias is None else bias.to(torch.bfloat16).contiguous()
+    if out is None:
+        out = torch.empty(x2.shape[0], N, dtype=torch.bfloat16, device=x.device)
+    assert out.shape == (x2.shape[0], N) and out.dtype == torch.bfloat16 and out.stride(1) == 1
+    r, ldr = None, 0
+    if residual is not None:
+        r = residual.reshape(-1, N)
+        assert r.shape == out.shape and r.dtype == torch.bfloat16 and r.stride(1) == 1
+        ldr = r.stride(0)
+    with torch.cuda.device(x.device):
+        _capi.check(_capi.load().bsa_gemm_bf16(_ptr(x2), x2.stride(0), _ptr(w), w.stride(0), _ptr(b), _ptr(r), ldr, _ptr(out),
+                                               out.stride(0), x2.shape[0], N, K, _stream(x)), "gemm")
+    return out.view(*x.shape[:-1], N)
+
+
+def qkv_projection(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], q_weight: torch.Tensor,
+                   k_weight: torch.Tensor, grid_size, num_heads: int, eps: float = 1e-6, t_offset: int = 0,
+                   table_grid=None):
+    """attention.py:111-121 in one kernel: the QKV Linear, the split into heads, RMSNorm of q and k per head and
+    the 3-D RoPE.  x [B, T*H*W, C]; returns q, k, v as contiguous [B, heads, T*H*W, 128] tensors."""
+    if not x.is_cuda:
+        raise RuntimeError("the engine runs on the GPU only")
+    if x.dtype != torch.bfloat16:
+        raise NotImplementedError("qkv_projection: only bf16 is built")
+    B, S, K = x.shape
+    T, Hg, Wg = (int(g) for g in grid_size)
+    assert S == T * Hg * Wg and weight.shape == (3 * num_heads * 128, K)
+    table_grid = tuple(int(g) for g in (table_grid if table_grid is not None else grid_size))
+    assert table_grid[1:] == (Hg, Wg)
+    tab = rope_table(table_grid, 128, x.device)
+    x2 = x.reshape(B * S, K)
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    w = weight.to(torch.bfloat16)
+    if w.stride(1) != 1:
+        w = w.contiguous()
+    b = None if bias is None else bias.to(torch.bfloat16).contiguous()
+    qw, kw = q_weight.to(torch.bfloat16).contiguous(), k_weight.to(torch.bfloat16).contiguous()
+    qkv = torch.empty(3, B, num_heads, S, 128, dtype=torch.bfloat16, device=x.device)
+    with torch.cuda.device(x.device):
+        _capi.check(_capi.load().bsa_qkv_projection(
+            _ptr(x2), x2.stride(0), _ptr(w), w.stride(0), _ptr(b), _ptr(qw), _ptr(kw), _ptr(tab), _ptr(qkv[0]), _ptr(qkv[1]),
+            _ptr(qkv[2]), _capi.strides3(qkv[0].stride()[:3]), B, num_heads, T, Hg, Wg, int(t_offset), table_grid[0], 128, K,
+            float(eps), _stream(x)), "qkv_projection")
+    return qkv[0], qkv[1], qkv[2]
+
+
 _ROPE_TABLES = {}
 
 
