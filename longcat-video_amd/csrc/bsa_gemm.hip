@@ -15,28 +15,31 @@
 // A workgroup of four wavefronts (one per SIMD, 512 registers each) computes a tile of 256 tokens x 256
 // features; every wavefront owns 128 x 128 of it (16 accumulator blocks = 256 registers), which for the QKV
 // projection is exactly one head of 128 tokens.  Per k block of 64 the workgroup brings 256 rows x 128 bytes of
-// either operand (a slab of 32 KB, whole cache lines) from global memory straight into LDS
-// (global_load_lds_dwordx4, no staging registers), two stages of 64 KB.  The LDS side of such a load is linear in
-// the lane index, so the XOR swizzle that keeps the fragment reads (ds_read_b128, rows 128 bytes apart) free of
-// bank conflicts is applied on the global side: the 16-byte slot p of row r receives k unit p ^ ((r >> 1) & 7).
+// either operand (a half-slab of 32 KB, whole cache lines) from global memory straight into LDS
+// (global_load_lds_dwordx4, no staging registers); five half-slab stages fill the 160 KB of LDS: two in use, up to
+// three on their way.  The LDS side of such a load is linear in the lane index, so the XOR swizzle that keeps the
+// fragment reads (ds_read_b128, rows 128 bytes apart; measured: bank-conflict cycles 4 % of the LDS-active ones)
+// free of bank conflicts is applied on the global side: the 16-byte slot p of row r receives k unit
+// p ^ ((r >> 1) & 7).
 //
 // One barrier per k block, after the third of its four k sub-steps: the fragments of a sub-step are read during
-// the MFMAs of the one before.  At the barrier every wavefront has awaited its own share of the next slab and
-// holds the last fragments of this one; right after it the slab two blocks ahead is requested into the stage
-// just drained.
+// the MFMAs of the one before.  At the barrier every wavefront has awaited its own share of the next block's two
+// half-slabs and holds the last fragments of this one; the two stages so drained take the half-slabs five further
+// on, requested one load per four MFMAs over the k block that follows.
 //
 // Tiles are handed out so that the workgroups resident on one XCD (32 CUs, one shared L2; workgroup b runs
 // on XCD b % 8) form a block of 8 token tiles x 4 feature tiles: they run in step, so each slab fetched from
 // HBM serves 4 (token slab) or 8 (weight slab) workgroups out of L2 (measured at the 720p QKV shape: 15 GB leave
 // L2 per call for 65 GB that enter LDS).
 //
-// What bounds it (measured at [86400, 4096] x [4096, 12288]^T, the kernel alone 8.0 ms): the MFMAs with the
-// fragment reads but without the loads take 5.0 ms, the loads and barriers without the MFMAs 5.9 ms (4.7 ms
-// when nothing waits for them: 14 TB/s from L2 into LDS, which is what this path delivers), and both together do
-// not overlap fully: a slab is requested one k block before it is needed, and under MFMA load it takes longer
-// than that to arrive.  Deeper variants were built and measured: five 32 KB half-slab stages (160 KB of LDS, 1.5
-// blocks in flight) 8.5 ms, ten 16 KB quarter-slab stages with paired loads 8.4 ms, register prefetch two blocks
-// ahead with compiler-placed waits 9.1 ms (the waits it places allow one block in flight).
+// What bounds it (measured at [86400, 4096] x [4096, 12288]^T on random data): the board's power limit.  Under this
+// kernel the clock settles near 1.83 GHz instead of 2.4 (under hipBLASLt's kernel for the same product near
+// 1.72 GHz), so a gain in work per clock is partly paid back in clock.  Per clock the k loop reaches about 0.61 of
+// the MFMA rate.  Variants measured on the way: all sixteen loads of a k block in one burst after the barrier
+// 8.5 ms (the wavefronts then wait for the address unit, not for data: with a software barrier instead of
+// s_barrier no better, without any barrier 5.3 ms but wrong); two stages of a whole k block 8.0 ms; ten 16 KB
+// stages with paired loads of the two halves of a cache line 8.4 ms; register prefetch two blocks ahead with
+// compiler-placed waits 9.1 ms (the waits it places allow only one block in flight).
 #include "bsa_mfma.h"
 
 namespace bsa {
@@ -48,8 +51,7 @@ constexpr int kTileM = 256;              // tokens per workgroup
 constexpr int kTileN = 256;              // features per workgroup
 constexpr int kBK = 64;                  // k per pipeline step
 constexpr int kPart = 256 * kBK * 2;     // bytes of one operand's slab
-constexpr int kStageBytes = 2 * kPart;   // weight slab, then token slab
-constexpr int kStages = 2;
+constexpr int kStages = 5;               // half-slabs resident in LDS: 160 KB
 constexpr int kEpiPitch = 272;           // bytes per token row of the output staging area (256 + 16)
 constexpr int kEpiBytes = 64 * kEpiPitch;
 constexpr int kSuperM = 8, kSuperN = 4;  // tiles of one XCD's block
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs a) {
     if (tile_f >= a.tiles_n || tile_m >= a.tiles_m) return;
     const int f_tile0 = tile_f * kTileN, m_tile0 = tile_m * kTileM;
 
-    // ---- global -> LDS: this wavefront brings rows [64 wave, 64 wave + 64) of either slab, 8 rows (of 128 bytes:
+    // ---- global -> LDS: this wavefront brings rows [64 wave, 64 wave + 64) of a half-slab, 8 rows (of 128 bytes:
     // one cache line each) per load
     uint32_t voff_w[8], voff_x[8];
 #pragma unroll
@@ -103,31 +105,31 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs a) {
     }
     const char* wbase = reinterpret_cast<const char*>(a.w + (int64_t)f_tile0 * a.ldw);
     const char* xbase = reinterpret_cast<const char*>(a.x + (int64_t)m_tile0 * a.ldx);
+    // Half-slab h (even: weight rows, odd: token rows, of k block h / 2) lives in stage h % kStages.
     const uint32_t lds0 = lds_address(smem) + wave * 8192;
-    const int nblocks = a.K / kBK;
-    auto issue = [&](int kb, int stage) __attribute__((always_inline)) {
-        const char* wb = wbase + (int64_t)kb * (kBK * 2);
-        const char* xb = xbase + (int64_t)kb * (kBK * 2);
-        const uint32_t l = lds0 + stage * kStageBytes;
-#pragma unroll
-        for (int r = 0; r < 8; ++r) load_to_lds_16(wb, voff_w[r], l + r * 1024);
-#pragma unroll
-        for (int r = 0; r < 8; ++r) load_to_lds_16(xb, voff_x[r], l + kPart + r * 1024);
+    const int nblocks = a.K / kBK, nhalf = 2 * nblocks;
+    // load r (of eight) of half-slab h; `odd` = h & 1, known at compile time
+    auto issue_one = [&](int h, int stage, auto odd_c, int r) __attribute__((always_inline)) {
+        constexpr int odd = decltype(odd_c)::value;
+        if (h >= nhalf) return;
+        const char* base = (odd ? xbase : wbase) + (int64_t)(h >> 1) * (kBK * 2);
+        load_to_lds_16(base, odd ? voff_x[r] : voff_w[r], lds0 + stage * kPart + r * 1024);
     };
 
     // ---- LDS -> fragments
     const uint32_t swz = ((lane & 31) >> 1) & 7, g = lane >> 5;
-    const uint32_t a_lane = (wm * 128 + (lane & 31)) * 128, b_lane = kPart + (wn * 128 + (lane & 31)) * 128;
+    const uint32_t a_lane = (wm * 128 + (lane & 31)) * 128, b_lane = (wn * 128 + (lane & 31)) * 128;
     uint32_t unit_of[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) unit_of[ks] = ((2 * ks + g) ^ swz) * 16;
     V8 af[2][4], bf[2][4];
-    auto read_frags = [&](int stage, int ks) __attribute__((always_inline)) {
-        const char* s = smem + stage * kStageBytes + unit_of[ks];
+    auto read_frags = [&](int stage_w, int stage_x, int ks) __attribute__((always_inline)) {
+        const char* sw = smem + stage_w * kPart + unit_of[ks] + a_lane;
+        const char* sx = smem + stage_x * kPart + unit_of[ks] + b_lane;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) af[ks & 1][i] = *reinterpret_cast<const V8*>(s + a_lane + i * 4096);
+        for (int i = 0; i < 4; ++i) af[ks & 1][i] = *reinterpret_cast<const V8*>(sw + i * 4096);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) bf[ks & 1][j] = *reinterpret_cast<const V8*>(s + b_lane + j * 4096);
+        for (int j = 0; j < 4; ++j) bf[ks & 1][j] = *reinterpret_cast<const V8*>(sx + j * 4096);
     };
     f32x16 acc[4][4];
 #pragma unroll
@@ -136,41 +138,77 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs a) {
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    auto products = [&](int ks) __attribute__((always_inline)) {
+    // The sixteen MFMAs of k sub-step ks, and between them four of the sixteen loads requested at the last barrier
+    // (token half-slab pend_h first, then weight half-slab pend_h + 1): one load per four MFMAs.  Issued in one
+    // burst right after the barrier, the four wavefronts' loads queue up in the CU's one address unit and the
+    // wavefronts, which issue in order, cannot start their MFMAs until their last load is taken.
+    int pend_h = nhalf, pend_sw = 0, pend_sx = 0;
+    auto products = [&](auto ks_c) __attribute__((always_inline)) {
+        constexpr int ks = decltype(ks_c)::value;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc[i][j] = mfma32(af[ks & 1][i], bf[ks & 1][j], acc[i][j]);
+            constexpr int quarter = (ks + 1) & 3;            // sub-step 3 is the first after the barrier
+            const int n = 4 * quarter + i;
+            __builtin_amdgcn_sched_barrier(0);
+            if (n < 8) issue_one(pend_h, pend_sx, IC<1>{}, n); else issue_one(pend_h + 1, pend_sw, IC<0>{}, n - 8);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     };
 
-    // ---- pipeline: the slab of k block b lives in stage b & 1
-    issue(0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // ---- pipeline
+#pragma unroll
+    for (int r = 0; r < 8; ++r) issue_one(0, 0, IC<0>{}, r);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) issue_one(1, 1, IC<1>{}, r);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) issue_one(2, 2, IC<0>{}, r);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) issue_one(3, 3, IC<1>{}, r);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) issue_one(4, 4, IC<0>{}, r);
+    if (nhalf >= kStages) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");    // half-slabs 0 and 1 of five
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
-    if (nblocks > 1) issue(1, 1);
-    read_frags(0, 0);
-    auto block = [&](int kb, auto stage_c) __attribute__((always_inline)) {
-        constexpr int st = decltype(stage_c)::value;
-        read_frags(st, 1);
-        products(0);
-        read_frags(st, 2);
-        products(1);
-        read_frags(st, 3);
-        products(2);
-        // Slab kb + 1: this wavefront's share has landed, then (barrier) everybody's; and everybody has the last
-        // fragments of slab kb in registers, so its stage can take slab kb + 2.
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    read_frags(0, 1, 0);
+    // k block kb, with c = kb % kStages known at compile time
+    auto block = [&](int kb, auto c_) __attribute__((always_inline)) {
+        constexpr int c = decltype(c_)::value;
+        constexpr int sw = (2 * c) % kStages, sx = (2 * c + 1) % kStages;              // stages of this block
+        constexpr int nw = (2 * c + 2) % kStages, nx = (2 * c + 3) % kStages;          // ... of the next one
+        read_frags(sw, sx, 1);
+        products(IC<0>{});
+        read_frags(sw, sx, 2);
+        products(IC<1>{});
+        read_frags(sw, sx, 3);
+        products(IC<2>{});
+        // The next block's two half-slabs: this wavefront's share has landed (the one requested after them may still
+        // be on its way), then (barrier) everybody's; and everybody holds the last fragments of this block in
+        // registers, so its two stages can take the half-slabs five further on (tokens of block kb + 2, needed at
+        // the next barrier, then weights of block kb + 3), requested piecemeal by products().
+        if (2 * kb + 4 < nhalf) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
-        if (kb + 2 < nblocks) issue(kb + 2, st);
-        if (kb + 1 < nblocks) read_frags(st ^ 1, 0);
-        products(3);
+        pend_h = 2 * kb + kStages;
+        pend_sx = sw;                    // half-slab 2 kb + 5 (tokens) takes the stage of half-slab 2 kb (weights)
+        pend_sw = sx;                    // half-slab 2 kb + 6 (weights) the stage of half-slab 2 kb + 1 (tokens)
+        if (kb + 1 < nblocks) read_frags(nw, nx, 0);
+        products(IC<3>{});
     };
     int kb = 0;
-    for (; kb + 2 <= nblocks; kb += 2) {
+    for (; kb + kStages <= nblocks; kb += kStages) {
         block(kb, IC<0>{});
         block(kb + 1, IC<1>{});
+        block(kb + 2, IC<2>{});
+        block(kb + 3, IC<3>{});
+        block(kb + 4, IC<4>{});
     }
-    if (kb < nblocks) block(kb, IC<0>{});
+    if (kb < nblocks) { block(kb, IC<0>{}); ++kb; }
+    if (kb < nblocks) { block(kb, IC<1>{}); ++kb; }
+    if (kb < nblocks) { block(kb, IC<2>{}); ++kb; }
+    if (kb < nblocks) { block(kb, IC<3>{}); ++kb; }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();        // every wavefront is done with the slabs: the staging area may overwrite them
 
     // ---- epilogue.  Feature of register r of block i: f0 + 32 i + 8 (r / 4) + 4 g + r % 4; token of block j: m0 + 32 j + lane % 32.
@@ -313,8 +351,8 @@ int launch_gemm(GemmArgs& a, hipStream_t stream) {
     a.super_m = (a.tiles_m + kSuperM - 1) / kSuperM;
     a.super_total = a.super_m * ((a.tiles_n + kSuperN - 1) / kSuperN);
     const unsigned grid = (unsigned)((a.super_total + 7) / 8) * 256u;
-    const size_t lds = (size_t)kStages * kStageBytes;
-    static_assert(kStages * kStageBytes >= 4 * kEpiBytes, "the staging area reuses the slabs");
+    const size_t lds = (size_t)kStages * kPart;
+    static_assert(kStages * kPart >= 4 * kEpiBytes, "the staging area reuses the slabs");
     auto kernel = gemm_nt_kernel<QKV>;
     // more than the 64 KB a kernel gets without asking; the attribute is per device, so it is set on every call
     const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
