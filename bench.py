@@ -366,6 +366,16 @@ def run_c5(torch, args):
     o_buf = torch.empty(1, N, HEADS, D, dtype=x.dtype, device=x.device).permute(0, 2, 1, 3)
     ms_attn = time_events(torch, lambda: attend(qd, idx, lens, out=o_buf), 20, 5, settle_s=args.settle)
     del attend
+    # ---- the engine's own GEMM: QKV projection with norm, rotation and head split in its epilogue, and the output
+    # projection; and the module with both (projection_backend = "engine")
+    xn = M.rms_norm(x, w_pre, 1e-6)
+    ms_eng_qkv = time_events(torch, lambda: M.qkv_projection(xn, attn.qkv.weight, attn.qkv.bias, attn.q_norm.weight,
+                                                             attn.k_norm.weight, latent, HEADS), 5, 2)
+    ms_eng_proj = time_events(torch, lambda: M.gemm_bf16(x, attn.proj.weight, attn.proj.bias, residual=x), 5, 2)
+    attn.projection_backend = "engine"
+    ms_eng_step = time_events(torch, lambda: M.attention_block_forward(x, w_pre, attn, latent), max(args.steps // 2, 3), 2)
+    attn.projection_backend = "hipblaslt"
+    eng_tflops = 2 * N * C * 3 * C / ms_eng_qkv / 1e9
     qkv_tflops = 2 * N * C * 3 * C / ms_qkv / 1e9
     norm_rope_gbs = 2 * N * C * 2 / ms_norm_rope / 1e6          # one tensor: 708 MB read + 708 MB written
     result = {
@@ -375,7 +385,10 @@ def run_c5(torch, args):
         "dtype": "bf16", "data": "synthetic N(0,1) activations, N(0,0.02) weights, zero biases, unit norm weights",
         "config": {"workload": "c5: x [1, 86400, 4096] bf16, 32 heads x 128, grid 24x45x80, density 1/16"},
         "kernels_ms": {"attention": round(ms_attn, 4), "qkv_gemm": round(ms_qkv, 4), "proj_gemm_with_residual": round(ms_proj, 4),
-                       "norm_rope_move_one_tensor": round(ms_norm_rope, 4)},
+                       "norm_rope_move_one_tensor": round(ms_norm_rope, 4),
+                       "engine_qkv_projection_with_norm_rope_epilogue": round(ms_eng_qkv, 4),
+                       "engine_proj_gemm_with_residual": round(ms_eng_proj, 4)},
+        "ms_per_step_with_engine_projections": round(ms_eng_step, 4),
         "qkv_gemm_ms": round(ms_qkv, 4), "qkv_gemm_tflops": round(qkv_tflops, 1),
         "gemm_tuning": {"qkv": {"algorithms_timed": tuned[0][0], "default_ms": round(tuned[0][1], 4), "chosen_ms": round(tuned[0][2], 4)},
                         "proj": {"algorithms_timed": tuned[1][0], "default_ms": round(tuned[1][1], 4), "chosen_ms": round(tuned[1][2], 4)}},
@@ -385,6 +398,9 @@ def run_c5(torch, args):
         "roofline_qkv_gemm": {"kernel": "hipBLASLt bf16 GEMM [86400,4096]x[4096,12288]^T + bias (library kernel)", "bound": "mfma",
                               "achieved": round(qkv_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                               "frac": round(qkv_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None, "ms": round(ms_qkv, 4)},
+        "roofline_engine_gemm": {"kernel": "gemm_nt_kernel<qkv epilogue> [86400,4096]x[4096,12288]^T + bias, per-head RMSNorm, RoPE, head split",
+                                 "bound": "mfma", "achieved": round(eng_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                                 "frac": round(eng_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None, "ms": round(ms_eng_qkv, 4)},
         "roofline_norm_rope": {"kernel": "norm_rope_kernel<bf16> (per-head RMSNorm + 3-D RoPE + move of one tensor)", "bound": "hbm",
                                "achieved": round(norm_rope_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                "frac": round(norm_rope_gbs / PEAK_HBM_GBS, 4), "traffic": None, "ms": round(ms_norm_rope, 4)},

@@ -287,13 +287,25 @@ class Attention(nn.Module):
         # `attn.qkv` and `attn.proj` (longcat_video_dit.py:211-232); empty = the plain Linear
         self.qkv_loras = []
         self.proj_loras = []
+        # "hipblaslt": the projections through bsa_linear_bf16, norm and rotation as separate passes (the faster
+        # route at the 720p shapes); "engine": bsa_qkv_projection (GEMM with norm, rotation and head split in its
+        # epilogue) and bsa_gemm_bf16.  Both round at the same points.
+        self.projection_backend = "hipblaslt"
 
     def _linear(self, x, layer, loras, residual=None):
         if any(b.use_lora for b in loras):
             from .lora import lora_linear
             y = lora_linear(x, layer.weight, layer.bias, loras)
             return y if residual is None else y + residual
+        if self.projection_backend == "engine" and layer.weight.shape[0] % 128 == 0 and layer.weight.shape[1] % 64 == 0:
+            return gemm_bf16(x, layer.weight, layer.bias, residual=residual)
         return linear_bf16(x, layer.weight, layer.bias, residual=residual)
+
+    def _fused_projection(self, x, shape, return_kv):
+        """True when the QKV GEMM with the fused epilogue applies: engine backend, no LoRA branch on qkv, no
+        k cache wanted (the cache holds k before the rotation, which the fused epilogue does not keep)."""
+        return (self.projection_backend == "engine" and not return_kv and self.head_dim == 128 and x.shape[-1] % 64 == 0
+                and not any(b.use_lora for b in self.qkv_loras))
 
     @torch.no_grad()
     def tune(self, x: torch.Tensor, residual: bool = False):
@@ -331,19 +343,22 @@ class Attention(nn.Module):
         """attention.py:107-147.  `residual` (extension): added to the projection output inside the GEMM."""
         B, N, C = x.shape
         Hn, D = self.num_heads, self.head_dim
-        qs, ks, vs = self._project_qkv(x)
-        new = lambda: torch.empty(B, Hn, N, D, dtype=x.dtype, device=x.device)
         eps = self.q_norm.eps
-        # q moves into a per-head tensor on the way (the attention kernel fetches its rows tile by tile); k is normed
-        # and rotated where it lies and v stays where it is: the operator reads both once, to rewrite them in its
-        # fragment order, and a strided read costs that pass less than a separate move costs
-        q = norm_rope(qs, new(), self.q_norm.weight, shape, eps=eps)
-        v = vs
-        if return_kv:
-            k_cache = norm_rope(ks, new(), self.k_norm.weight, eps=eps)           # attention.py:118-119
-            k = norm_rope(k_cache, new(), None, shape)
+        new = lambda: torch.empty(B, Hn, N, D, dtype=x.dtype, device=x.device)
+        if self._fused_projection(x, shape, return_kv):
+            q, k, v = qkv_projection(x, self.qkv.weight, self.qkv.bias, self.q_norm.weight, self.k_norm.weight, shape,
+                                     Hn, eps=eps)
         else:
-            k = norm_rope(ks, ks, self.k_norm.weight, shape, eps=eps)
+            # q moves into a per-head tensor on the way (the attention kernel fetches its rows tile by tile); k is
+            # normed and rotated where it lies and v stays where it is: the operator reads both once, to rewrite
+            # them in its fragment order, and a strided read costs that pass less than a separate move costs
+            qs, ks, v = self._project_qkv(x)
+            q = norm_rope(qs, new(), self.q_norm.weight, shape, eps=eps)
+            if return_kv:
+                k_cache = norm_rope(ks, new(), self.k_norm.weight, eps=eps)       # attention.py:118-119
+                k = norm_rope(k_cache, new(), None, shape)
+            else:
+                k = norm_rope(ks, ks, self.k_norm.weight, shape, eps=eps)
 
         o = torch.empty(B, N, Hn, D, dtype=x.dtype, device=x.device)             # token-major: reshape below is free
         ov = o.permute(0, 2, 1, 3)                                                # [B, H, N, D] view

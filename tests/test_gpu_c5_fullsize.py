@@ -146,6 +146,46 @@ def test_module_stages_at_720p_size(c5):
     assert torch.equal(y_mod, y)
 
 
+def test_engine_projections_at_720p_size(c5):
+    """The engine's own GEMM at the two projection shapes of the module: the fused QKV projection (norm, rotation,
+    head split in the epilogue) against the hipBLASLt route's q, k, v on sampled tokens and against the oracle's
+    chain on fp32 products of sampled rows; the output projection with bias and residual against fp32."""
+    x, m = c5
+    att = M()
+    B, N, C, Hn, D = 1, N_TOK, DIM, HEADS, 128
+    q, k, v = att.qkv_projection(x, m.qkv.weight, m.qkv.bias, m.q_norm.weight, m.k_norm.weight, SHAPE, Hn, eps=m.q_norm.eps)
+    torch.cuda.synchronize()
+    assert q.shape == (B, Hn, N, D) and torch.isfinite(q.float()).all() and torch.isfinite(k.float()).all()
+    toks = torch.cat([sampled_rows(N, 64, 12), torch.tensor([255, 256, N - 129, N - 128])])   # tile edges and the half tile at the end
+    rows = x[0, toks].float().cpu() @ m.qkv.weight.float().cpu().t() + m.qkv.bias.float().cpu()      # [n, 3C] in fp32
+    qkv = rows.bfloat16().view(len(toks), 3, Hn, D).permute(1, 2, 0, 3)[:, None]                    # [3, 1, H, n, D]
+    ang = O.rope_3d_angles(SHAPE, D)[toks]
+    assert torch.all((v[:, :, toks].cpu().float() - qkv[2].float()).abs() <= qkv[2].float().abs() * BF16_ULP + 4e-3)
+    for got, src, w in ((q, qkv[0], m.q_norm.weight), (k, qkv[1], m.k_norm.weight)):
+        want = O.rope_3d_apply(O.rms_norm_fp32(src, w.cpu()), ang)
+        d = (got[:, :, toks].cpu().float() - want.float()).abs()
+        # the projection feeding the norm may differ by one rounding from the fp32 one: a few ulps after the norm
+        assert torch.all(d <= want.float().abs() * 4 * BF16_ULP + 0.03), float(d.max())
+        assert (d > want.float().abs() * BF16_ULP + 1e-3).float().mean() < 0.02
+    # the module's two routes agree closely (different summation orders inside the GEMMs)
+    y_lt = m(x, shape=SHAPE, residual=x)
+    m.projection_backend = "engine"
+    try:
+        y_en = m(x, shape=SHAPE, residual=x)
+    finally:
+        m.projection_backend = "hipblaslt"
+    torch.cuda.synchronize()
+    assert torch.isfinite(y_en.float()).all()
+    d = (y_en.float() - y_lt.float()).abs()
+    assert d.mean() <= 4e-3 and (d > 0.25).float().mean() < 1e-3, (float(d.mean()), float(d.max()))
+    # output projection
+    o = torch.randn(N, C, generator=torch.Generator(device="cuda").manual_seed(13), device="cuda").bfloat16()
+    y = att.gemm_bf16(o, m.proj.weight, m.proj.bias, residual=x[0])
+    rows = sampled_rows(N, 48, 14)
+    want = o[rows].float().cpu() @ m.proj.weight.float().cpu().t() + m.proj.bias.float().cpu() + x[0, rows].float().cpu()
+    assert torch.all((y[rows].float().cpu() - want).abs() <= want.abs() * BF16_ULP + 2e-2)
+
+
 def test_attention_block_forward_at_720p_size(c5):
     """RMSNorm -> module -> residual (benchmark configuration 5 as worded): finite, deterministic, and the
     pre-norm agrees with the oracle on sampled rows; the module behind it is covered stage by stage above."""
