@@ -376,6 +376,28 @@ int bsa_linear_bf16_tune(const void* x, int64_t ldx, const void* w, int64_t ldw,
 int bsa_lora_add(const void* org, const void* const* up, const float* multiplier, const float* alpha_scale, int n_loras,
                  void* out, int64_t n, int dtype, void* stream);
 
+/* bsa_fwd_3d for the attention module (attention.py:116-137): q and k arrive as the QKV projection left them
+ * (strided views into its output are fine) and go through the per-head RMSNorm (RMSNorm_FP32, blocks.py:42-53) and
+ * the 3-D RoPE (rope_3d.py:100-120) inside the operator's own passes over them, at the rounding points of
+ * bsa_norm_rope: the pass that takes q's chunk means writes the transformed rows to q_normed ([B, Hn, Tq*Hq*Wq, 128]
+ * through qn_strides; the attention kernel reads q from there), the pass that rewrites k into the attention
+ * kernel's operand order transforms it on the way, so the stand-alone norm / rotation passes over q and k and one
+ * read of q drop out.  rope_table as for bsa_norm_rope with the H and W of the grids (Hq = Hk, Wq = Wk); q sits at
+ * frames t_offset_q.. and k at frames t_offset_k.. of its table_T frames.  bf16 / fp16, 64-token chunks for q and
+ * k with at most 8 positions per axis (BSA_ERR_UNSUPPORTED otherwise: use bsa_qk_norm_rope + bsa_fwd_3d).  Everything else as bsa_fwd_3d; idx_out /
+ * lens_out / score_out refer to the transformed q and k. */
+typedef struct bsa_qk_norm {
+    const void* q_weight;      /* 128 elements of the tensors' type, 16-byte aligned */
+    const void* k_weight;
+    const float* rope_table;
+    int table_T, t_offset_q, t_offset_k;
+    float eps;
+} bsa_qk_norm;
+int bsa_fwd_3d_qknorm(const bsa_3d_params* p, const bsa_qk_norm* n, const void* q, const int64_t q_strides[3],
+                      void* q_normed, const int64_t qn_strides[3], const void* k, const int64_t k_strides[3], const void* v,
+                      const int64_t v_strides[3], void* o, const int64_t o_strides[3], void* workspace, size_t workspace_bytes,
+                      int32_t* idx_out, int32_t* lens_out, void* score_out, void* stream);
+
 /* The engine's own GEMM for the two projections of the attention module (attention.py:111 and :142):
  * out[M,N] = x[M,K] . w[N,K]^T (+ bias[N]) (+ residual[M,N]), bf16 in/out, fp32 accumulation on MFMA, one
  * rounding at the end.  Row strides in elements (ldx, ldw >= K; ldo, ldr >= N; multiples of 8).  N must be a

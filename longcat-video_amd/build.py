@@ -26,7 +26,12 @@ SOURCES = ["bsa_capi.hip", "bsa_permute.hip", "bsa_select.hip", "bsa_fwd.hip", "
 # maxima need no NaN-quieting extra instructions.  Infinities keep their IEEE meaning.
 # The glue kernels restate eager fp32 expressions (x * cos + rot * sin, x * (scale + 1) + shift, x + gate * y)
 # whose products and sums are rounded one by one: no contraction into FMAs there (explicit fmaf stays an FMA).
-EXTRA_FLAGS = {"bsa_fwd.hip": ["-fno-honor-nans"], "bsa_fwd_frag.hip": ["-fno-honor-nans"], "bsa_bwd.hip": ["-fno-honor-nans"], "bsa_glue.hip": ["-ffp-contract=off"]}
+# The fragment pass and the GEMM epilogue share those expressions (bsa_rope.h) beside code that wants its FMAs:
+# contraction stays on for the file and the shared functions switch it off with a pragma, which the compiler only
+# honours under fast-honor-pragmas.
+EXTRA_FLAGS = {"bsa_fwd.hip": ["-fno-honor-nans"], "bsa_fwd_frag.hip": ["-fno-honor-nans", "-ffp-contract=fast-honor-pragmas"],
+               "bsa_bwd.hip": ["-fno-honor-nans"], "bsa_glue.hip": ["-ffp-contract=off"],
+               "bsa_gemm.hip": ["-ffp-contract=fast-honor-pragmas"]}
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -385,7 +385,7 @@ int check_kv_views(const Plan& pl, const int64_t k_strides[3], const int64_t v_s
 // full and their chunk means stored (one pass over each).
 hipError_t prepare_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, const void* q, const int64_t q_strides[3],
                        const void* k, const int64_t k_strides[3], const void* v, const int64_t v_strides[3], bool pool,
-                       hipStream_t st) {
+                       hipStream_t st, const RowTransform* trq = nullptr, const RowTransform* trk = nullptr) {
     hipError_t e;
     const bool padded_k = kv_padded(p);
     if (pool && !(pl.frag && pl.gq.chunk() == 64))
@@ -395,14 +395,14 @@ hipError_t prepare_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, cons
     if (e != hipSuccess) return e;
     if (pool && pl.frag && pl.gq.chunk() == 64) {
         // chunk means of q from the fragment pass run without a destination: the same sums, a faster read
-        e = launch_frag(q, q_strides, nullptr, p->B, p->Hn, pl.gq, p->dtype, false, st, w.qc, nullptr);
+        e = launch_frag(q, q_strides, nullptr, p->B, p->Hn, pl.gq, p->dtype, false, st, w.qc, nullptr, trq);
         if (e != hipSuccess) return e;
     }
     if (pl.frag) {
         // 64-slot chunks: one pass over k gives its fragment order, its chunk means and the validity words
         if (pl.gk.chunk() == 64) {
             e = launch_frag(k, k_strides, w.kp, p->B, p->Hn, pl.gk, p->dtype, false, st, pool ? w.kc : nullptr,
-                            padded_k ? w.valid : nullptr);
+                            padded_k ? w.valid : nullptr, trk);
             if (e != hipSuccess) return e;
             return launch_frag(v, v_strides, w.vp, p->B, p->Hn, pl.gk, p->dtype, true, st);
         }
@@ -510,7 +510,8 @@ namespace {
 int fwd_3d_impl(const Plan& pl, const bsa_3d_params* p, const void* q, const int64_t q_strides[3], const void* k,
                 const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
                 const int64_t o_strides[3], void* workspace, size_t workspace_bytes, int32_t* idx_out,
-                int32_t* lens_out, void* score_out, void* stream) {
+                int32_t* lens_out, void* score_out, void* stream, const bsa_qk_norm* qkn = nullptr, void* q_normed = nullptr,
+                const int64_t* qn_strides = nullptr) {
     Ws w;
     if (!q || !k || !v || !o || !workspace) return set_error(BSA_ERR_BAD_ARG, "fwd_3d: null pointer");
     BSA_TRY(carve(pl, workspace, workspace_bytes, "fwd_3d", &w));
@@ -524,7 +525,16 @@ int fwd_3d_impl(const Plan& pl, const bsa_3d_params* p, const void* q, const int
     hipStream_t st = (hipStream_t)stream;
     hipError_t e;
 #define BSA_HIP(call, what) do { e = (call); if (e != hipSuccess) return hip_fail(e, what); } while (0)
-    if (pl.direct_qo) {
+    if (qkn != nullptr) {
+        // q and k as the projection left them: the pass that takes q's chunk means also normalises and rotates its
+        // rows into q_normed (what the attention kernel then reads), the pass that rewrites k in fragment order
+        // normalises and rotates on the way
+        RowTransform trq = {qkn->q_weight, qkn->rope_table, qkn->t_offset_q, qkn->table_T, qkn->eps, q_normed, qn_strides[0], qn_strides[1], qn_strides[2]};
+        RowTransform trk = {qkn->k_weight, qkn->rope_table, qkn->t_offset_k, qkn->table_T, qkn->eps, nullptr, 0, 0, 0};
+        BSA_HIP(prepare_thw(pl, p, w, q, q_strides, k, k_strides, v, v_strides, true, st, &trq, &trk), "pool, norm, rotate and prepare");
+        q = q_normed;
+        q_strides = qn_strides;
+    } else if (pl.direct_qo) {
         BSA_HIP(prepare_thw(pl, p, w, q, q_strides, k, k_strides, v, v_strides, true, st), "pool and prepare");
     } else {
         BSA_HIP(launch_permute(q, q_strides, w.qp, w.qc, nullptr, p->B, p->Hn, pl.gq, p->D, p->dtype, st), "permute q");
@@ -601,6 +611,31 @@ int bsa_fwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3]
     BSA_TRY(make_plan(p, &pl));
     return fwd_3d_impl(pl, p, q, q_strides, k, k_strides, v, v_strides, o, o_strides, workspace, workspace_bytes, idx_out,
                        lens_out, score_out, stream);
+}
+
+int bsa_fwd_3d_qknorm(const bsa_3d_params* p, const bsa_qk_norm* n, const void* q, const int64_t q_strides[3],
+                      void* q_normed, const int64_t qn_strides[3], const void* k, const int64_t k_strides[3], const void* v,
+                      const int64_t v_strides[3], void* o, const int64_t o_strides[3], void* workspace, size_t workspace_bytes,
+                      int32_t* idx_out, int32_t* lens_out, void* score_out, void* stream) {
+    Plan pl;
+    BSA_TRY(make_plan(p, &pl));
+    if (!n || !n->rope_table || !n->q_weight || !n->k_weight || !q_normed || !qn_strides)
+        return set_error(BSA_ERR_BAD_ARG, "fwd_3d_qknorm: null pointer");
+    if (!(pl.direct_qo && pl.frag && pl.gq.chunk() == 64 && pl.gk.chunk() == 64) || p->tq > 8 || p->hq > 8 || p->wq > 8 ||
+        p->tk > 8 || p->hk > 8 || p->wk > 8)
+        return set_error(BSA_ERR_UNSUPPORTED, "fwd_3d_qknorm: bf16 / fp16 with 64-token chunks of at most 8 positions per axis only "
+                         "(use bsa_qk_norm_rope and bsa_fwd_3d)");
+    if (!(n->eps >= 0.f)) return set_error(BSA_ERR_BAD_ARG, "fwd_3d_qknorm: eps must be non-negative");
+    if (n->t_offset_q < 0 || n->t_offset_k < 0 || n->table_T < n->t_offset_q + p->Tq || n->table_T < n->t_offset_k + p->Tk)
+        return set_error(BSA_ERR_SHAPE, "fwd_3d_qknorm: the frames of q (%d..) or k (%d..) lie outside a table of %d frames",
+                         n->t_offset_q, n->t_offset_k, n->table_T);
+    if (p->Hq != p->Hk || p->Wq != p->Wk)
+        return set_error(BSA_ERR_SHAPE, "fwd_3d_qknorm: q and k share one rotation table, so their H and W must agree");
+    if ((reinterpret_cast<uintptr_t>(n->q_weight) | reinterpret_cast<uintptr_t>(n->k_weight)) & 15u)
+        return set_error(BSA_ERR_BAD_ARG, "fwd_3d_qknorm: norm weights must be 16-byte aligned");
+    BSA_TRY(check_tensor(q_normed, qn_strides, p, "q_normed"));
+    return fwd_3d_impl(pl, p, q, q_strides, k, k_strides, v, v_strides, o, o_strides, workspace, workspace_bytes, idx_out,
+                       lens_out, score_out, stream, n, q_normed, qn_strides);
 }
 
 int bsa_fwd_3d_static(const bsa_3d_params* p, const void* q, const int64_t q_strides[3], const void* k,

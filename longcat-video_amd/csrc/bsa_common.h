@@ -145,8 +145,19 @@ void launch_schedule_choice(const int32_t* lens, int nbq, int tiles_per_block, i
 // For K (transpose = false) of 64-slot chunks the pass can also write the chunk means (pooled, [B*Hn][blocks][128],
 // the bits launch_permute's pooling gives) and the tile validity words; both optional.  dst may be null: the pass
 // then only reads (chunk means of q).
+// tr (optional, transpose = false only): per-head RMSNorm and / or 3-D RoPE of every row on its way through the pass.
+struct RowTransform {
+    const void* norm_w;      // 128 norm weights in the storage type; null: no norm
+    const float* tab;        // rotation table (the layout bsa_norm_rope reads); null: no rotation
+    int t0, Ttab;            // frame offset of the grid inside the table, frames of the table
+    float eps;
+    void* rows_out;          // optional: the transformed rows at their token positions
+    int64_t rB, rH, rS;      // ... element strides {batch, head, token}
+    int head_fastest;        // set by launch_frag: the order in which workgroups take (tile, head)
+};
 hipError_t launch_frag(const void* src, const int64_t strides[3], void* dst, int B, int Hn, const Grid3& g, int dtype,
-                       bool transpose, hipStream_t st, void* pooled = nullptr, uint64_t* tile_valid = nullptr);
+                       bool transpose, hipStream_t st, void* pooled = nullptr, uint64_t* tile_valid = nullptr,
+                       const RowTransform* tr = nullptr);
 // The attention kernel on fragment-order K and V.  q_rows (optional): token row of every blocked-order query
 // slot, -1 for padding; q_st / o_st: element strides {batch, head, row}; lse_rows: rows per (batch, head) of lse.
 hipError_t launch_fwd_frag(const void* q, const void* kf, const void* vf, const int32_t* idx, const int32_t* lens,

@@ -33,6 +33,7 @@
 // follow flash_attn_bsa_varlen_mask.py:242-285: fp32 logits, scale * log2(e) applied after the
 // dot, exp2, P rounded to the storage type for the P V product, fp32 row sum, one final rounding.
 #include "bsa_mfma.h"
+#include "bsa_rope.h"
 
 #include <utility>
 
@@ -51,36 +52,107 @@ constexpr int kListEntries = 4096;    // longest list a work item can walk (its 
 // For K of 64-slot chunks the same pass can also produce what the pooling pass of bsa_permute.hip would: the chunk
 // mean (pooled, in the storage type given by is_bf16; the summation order of permute_kernel is reproduced, so the
 // two routes give the same bits) and the validity word of the tile.
+// With a row transform (TRANSPOSE = false only) every row goes through the per-head RMSNorm and / or the 3-D RoPE
+// of the attention module on its way (bsa_rope.h: the bits of the stand-alone pass), before the chunk means are
+// taken; the transformed rows can also be written out at their token positions (the q of the attention kernel).
 template <typename T, bool TRANSPOSE>
 __global__ __launch_bounds__(256) void frag_kernel(const T* __restrict__ src, int64_t sB, int64_t sH, int64_t sS,
                                                    char* __restrict__ dst, Grid3 g, int Hn, T* __restrict__ pooled,
-                                                   uint64_t* __restrict__ tile_valid, int is_bf16) {
+                                                   uint64_t* __restrict__ tile_valid, int is_bf16, RowTransform tr) {
     // rows padded to 264 B: the transposing reads below walk down a column
     constexpr int kPitch = kD + 4;
     __shared__ __attribute__((aligned(16))) T tile[kTile * kPitch];
     const int tiles_per_chunk = g.chunk() / kTile;
-    const int blk = blockIdx.x / tiles_per_chunk, sub = blockIdx.x % tiles_per_chunk;
-    const int bh = blockIdx.y;
+    // Workgroup -> (tile, batch * head).  For a token-major source (the heads of a token next to each other, as a
+    // QKV projection leaves them) the heads of one tile run side by side, so that the 256-byte rows they fetch share
+    // DRAM pages and cache lines' neighbourhoods; otherwise the tiles of one head do.
+    const int tiles = g.blocks() * tiles_per_chunk;
+    int tile_id, bh;
+    if (tr.head_fastest) {
+        const int per_batch = tiles * Hn, b = blockIdx.x / per_batch, rest = blockIdx.x - b * per_batch;
+        tile_id = rest / Hn;
+        bh = b * Hn + (rest - tile_id * Hn);
+    } else {
+        bh = blockIdx.x / tiles;
+        tile_id = blockIdx.x - bh * tiles;
+    }
+    const int blk = tile_id / tiles_per_chunk, sub = tile_id % tiles_per_chunk;
     const int nw = blk % g.Nw, nh = (blk / g.Nw) % g.Nh, nt = blk / (g.Nw * g.Nh);
     const T* sbase = src + (int64_t)(bh / Hn) * sB + (int64_t)(bh % Hn) * sH;
     const int c16 = threadIdx.x & 15, rg = threadIdx.x >> 4;      // 16 pieces of 16 B per row, 16 rows at a time
+    // Rotation: a chunk spans at most 8 positions per axis, and a rotation pair turns with one axis only, so the
+    // (cos, sin) the 64 rows need are 8 x 64 table entries, fetched once per workgroup instead of per row and head.
+    __shared__ float2 cs[8 * 64];
+    if (!TRANSPOSE && tr.tab != nullptr) {
+        for (int e = threadIdx.x; e < 8 * 64; e += 256) {
+            const int a = e >> 6, pr = e & 63;
+            int at, dsin;
+            if (pr < kRopePairsT) {
+                at = min(tr.t0 + nt * g.t + a, tr.Ttab - 1) * kRopePairsT + pr;
+                dsin = tr.Ttab * kRopePairsT;
+            } else if (pr < kRopePairsT + kRopePairsH) {
+                at = 2 * tr.Ttab * kRopePairsT + min(nh * g.h + a, g.H - 1) * kRopePairsH + pr - kRopePairsT;
+                dsin = g.H * kRopePairsH;
+            } else {
+                at = 2 * tr.Ttab * kRopePairsT + 2 * g.H * kRopePairsH + min(nw * g.w + a, g.W - 1) * kRopePairsW + pr - kRopePairsT - kRopePairsH;
+                dsin = g.W * kRopePairsW;
+            }
+            cs[e] = make_float2(tr.tab[at], tr.tab[at + dsin]);
+        }
+        __syncthreads();
+    }
     uint2 val[4][2];
+    uint4 xs[4];
+    int64_t token_of[4];         // -1: a padded slot
+    int loc[4];                  // position inside the chunk, ti | hi << 8 | wi << 16
+    // all four loads first, then the arithmetic: a row transformed right behind its own load would wait for it
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int r = sub * kTile + rg + 16 * i;                   // slot inside the chunk
         const int wi = r % g.w, hi = (r / g.w) % g.h, ti = r / (g.w * g.h);
         const int tt = nt * g.t + ti, hh = nh * g.h + hi, ww = nw * g.w + wi;
-        uint4 x = make_uint4(0, 0, 0, 0);
-        if (tt < g.T && hh < g.H && ww < g.W)
-            x = *reinterpret_cast<const uint4*>(sbase + (((int64_t)tt * g.H + hh) * g.W + ww) * sS + c16 * 8);
-        val[i][0] = make_uint2(x.x, x.y);
-        val[i][1] = make_uint2(x.z, x.w);
+        xs[i] = make_uint4(0, 0, 0, 0);
+        token_of[i] = -1;
+        loc[i] = ti | (hi << 8) | (wi << 16);
+        if (tt < g.T && hh < g.H && ww < g.W) {
+            token_of[i] = ((int64_t)tt * g.H + hh) * g.W + ww;
+            xs[i] = *reinterpret_cast<const uint4*>(sbase + token_of[i] * sS + c16 * 8);
+        }
+    }
+    if (!TRANSPOSE && (tr.norm_w != nullptr || tr.tab != nullptr)) {
+        uint4 wraw = make_uint4(0, 0, 0, 0);
+        if (tr.norm_w != nullptr) wraw = *reinterpret_cast<const uint4*>(reinterpret_cast<const T*>(tr.norm_w) + c16 * 8);
+        T* rows = tr.rows_out == nullptr ? nullptr
+                                         : reinterpret_cast<T*>(tr.rows_out) + (int64_t)(bh / Hn) * tr.rB + (int64_t)(bh % Hn) * tr.rH + c16 * 8;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (token_of[i] < 0) continue;                         // the 16 lanes of a row go together
+            float c[4] = {1.f, 1.f, 1.f, 1.f}, sn[4] = {0.f, 0.f, 0.f, 0.f};
+            if (tr.tab != nullptr) {
+                const int ti = loc[i] & 255, hi = (loc[i] >> 8) & 255, wi = loc[i] >> 16;
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    const int pr = c16 * 4 + jj;
+                    const float2 a = cs[(pr < kRopePairsT ? ti : pr < kRopePairsT + kRopePairsH ? hi : wi) * 64 + pr];
+                    c[jj] = a.x;
+                    sn[jj] = a.y;
+                }
+            }
+            xs[i] = is_bf16 ? norm_rope_piece<__bf16>(xs[i], wraw, tr.norm_w != nullptr, tr.tab != nullptr, c, sn, tr.eps)
+                            : norm_rope_piece<_Float16>(xs[i], wraw, tr.norm_w != nullptr, tr.tab != nullptr, c, sn, tr.eps);
+            if (rows != nullptr) *reinterpret_cast<uint4*>(rows + token_of[i] * tr.rS) = xs[i];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        val[i][0] = make_uint2(xs[i].x, xs[i].y);
+        val[i][1] = make_uint2(xs[i].z, xs[i].w);
     }
     if (!TRANSPOSE && tile_valid != nullptr && bh == 0 && threadIdx.x < 64) {
         const int r = sub * kTile + threadIdx.x;
         const int wi = r % g.w, hi = (r / g.w) % g.h, ti = r / (g.w * g.h);
         const uint64_t m = __ballot(nt * g.t + ti < g.T && nh * g.h + hi < g.H && nw * g.w + wi < g.W);
-        if (threadIdx.x == 0) tile_valid[blockIdx.x] = m;
+        if (threadIdx.x == 0) tile_valid[tile_id] = m;
     }
     if (!TRANSPOSE && pooled != nullptr) {
         // permute_kernel's order: a thread sums its rows rg, rg + 16, rg + 32, rg + 48 per element, then the 16
@@ -111,7 +183,7 @@ __global__ __launch_bounds__(256) void frag_kernel(const T* __restrict__ src, in
             uint16_t bits;
             if (is_bf16) bits = __builtin_bit_cast(uint16_t, (__bf16)sum);
             else bits = __builtin_bit_cast(uint16_t, (_Float16)sum);
-            reinterpret_cast<uint16_t*>(pooled)[((int64_t)bh * gridDim.x + blockIdx.x) * kD + threadIdx.x] = bits;
+            reinterpret_cast<uint16_t*>(pooled)[((int64_t)bh * tiles + tile_id) * kD + threadIdx.x] = bits;
         }
     }
     if (dst == nullptr) return;                                    // chunk means (and validity words) only
@@ -122,7 +194,7 @@ __global__ __launch_bounds__(256) void frag_kernel(const T* __restrict__ src, in
         *reinterpret_cast<uint2*>(row + 4) = val[i][1];
     }
     __syncthreads();
-    char* out = dst + ((int64_t)bh * gridDim.x + blockIdx.x) * kTileBytes;
+    char* out = dst + ((int64_t)bh * tiles + tile_id) * kTileBytes;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int e = threadIdx.x + 256 * i;                       // 16-byte piece of the output, 0..1023
@@ -669,15 +741,17 @@ hipError_t launch_fwd_frag(const void* q, const void* kf, const void* vf, const 
 }
 
 hipError_t launch_frag(const void* src, const int64_t st3[3], void* dst, int B, int Hn, const Grid3& g, int dtype,
-                       bool transpose, hipStream_t st, void* pooled, uint64_t* tile_valid) {
-    const dim3 grid((unsigned)(g.blocks() * (g.chunk() / kTile)), (unsigned)(B * Hn)), block(256);
+                       bool transpose, hipStream_t st, void* pooled, uint64_t* tile_valid, const RowTransform* tr) {
+    RowTransform t = tr ? *tr : RowTransform{};
+    t.head_fastest = st3[1] < st3[2] ? 1 : 0;
+    const dim3 grid((unsigned)((int64_t)g.blocks() * (g.chunk() / kTile) * B * Hn)), block(256);
     // 16-bit types move as raw bits
     if (transpose)
         hipLaunchKernelGGL((frag_kernel<uint16_t, true>), grid, block, 0, st, (const uint16_t*)src, st3[0], st3[1], st3[2],
-                           (char*)dst, g, Hn, (uint16_t*)nullptr, (uint64_t*)nullptr, 0);
+                           (char*)dst, g, Hn, (uint16_t*)nullptr, (uint64_t*)nullptr, 0, t);
     else
         hipLaunchKernelGGL((frag_kernel<uint16_t, false>), grid, block, 0, st, (const uint16_t*)src, st3[0], st3[1], st3[2],
-                           (char*)dst, g, Hn, (uint16_t*)pooled, tile_valid, dtype == BSA_BF16 ? 1 : 0);
+                           (char*)dst, g, Hn, (uint16_t*)pooled, tile_valid, dtype == BSA_BF16 ? 1 : 0, t);
     return hipGetLastError();
 }
 

@@ -254,6 +254,7 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs a) {
         section = f0 / per_section;
         head = (f0 - section * per_section) >> 7;
         if (section < 2) {
+#pragma clang fp contract(off)       // every product and sum below is rounded on its own, as in the eager expressions
             constexpr int D = 128;
             constexpr int nt = (D - 4 * (D / 6)) / 2, nh = D / 6, nw = D / 6;    // rotation pairs per axis: 22, 21, 21
             const __bf16* nwgt = a.norm_w[section];
@@ -270,7 +271,7 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs a) {
                         ss = fmaf(v, v, ss);
                     }
                 ss += __shfl_xor(ss, 32);
-                const float rs = rsqrtf(ss / (float)D + a.eps);
+                const float rs = __builtin_amdgcn_rsqf(ss * (1.0f / (float)D) + a.eps);    // as bsa_rope.h
                 // position of this lane's token of block j
                 const uint32_t tok = (uint32_t)min(m0 + 32 * j + (lane & 31), a.M - 1);
                 const uint32_t s = tok % (uint32_t)a.S;
@@ -287,7 +288,7 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs a) {
                         float f[4];
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
-                            f[e] = (float)(__bf16)__fmul_rn((float)(__bf16)__fmul_rn(acc[i][j][4 * q + e], rs), (float)wv[e]);
+                            f[e] = (float)(__bf16)((float)(__bf16)(acc[i][j][4 * q + e] * rs) * (float)wv[e]);
 #pragma unroll
                         for (int e = 0; e < 2; ++e) {
                             const int pair = 16 * i + 4 * q + 2 * (int)g + e;
@@ -298,8 +299,8 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const GemmArgs a) {
                             const float c = a.tab[at], sn = a.tab[at + dsin];
                             const float x0 = f[2 * e], x1 = f[2 * e + 1];
                             // two products, then one add, each rounded: the order of operations of the eager expression
-                            acc[i][j][4 * q + 2 * e] = __fadd_rn(__fmul_rn(x0, c), __fmul_rn(-x1, sn));
-                            acc[i][j][4 * q + 2 * e + 1] = __fadd_rn(__fmul_rn(x1, c), __fmul_rn(x0, sn));
+                            acc[i][j][4 * q + 2 * e] = x0 * c + (-x1) * sn;
+                            acc[i][j][4 * q + 2 * e + 1] = x1 * c + x0 * sn;
                         }
                     }
             }

@@ -2,6 +2,7 @@
 // fused per-head QK RMSNorm + 3-D RoPE, and bf16 linear layers (hipBLASLt,
 // a plain library GEMM with bias / residual epilogue).
 #include "bsa_common.h"
+#include "bsa_rope.h"
 
 #include <hipblaslt/hipblaslt.h>
 
@@ -214,59 +215,20 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(const T* __restrict__ sr
     // cos / sin of this lane's four rotation pairs at token s
     auto angles = [&](uint32_t s, float (&c)[4], float (&sn)[4]) {
         const uint32_t u = s / (uint32_t)Wg, v = u / (uint32_t)Hg;
-        const int wi = (int)(s - u * Wg), hi = (int)(u - v * Hg), ti = t0 + (int)v;
-        const float* cos_t = tab;                        const float* sin_t = cos_t + (int64_t)Ttab * nt;
-        const float* cos_h = sin_t + (int64_t)Ttab * nt; const float* sin_h = cos_h + (int64_t)Hg * nh;
-        const float* cos_w = sin_h + (int64_t)Hg * nh;   const float* sin_w = cos_w + (int64_t)Wg * nw;
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-            const int pair = sub * 4 + jj;         // 0..63
-            if (pair < nt) { c[jj] = cos_t[ti * nt + pair]; sn[jj] = sin_t[ti * nt + pair]; }
-            else if (pair < nt + nh) { c[jj] = cos_h[hi * nh + pair - nt]; sn[jj] = sin_h[hi * nh + pair - nt]; }
-            else { c[jj] = cos_w[wi * nw + pair - nt - nh]; sn[jj] = sin_w[wi * nw + pair - nt - nh]; }
-        }
+        rope_angles(tab, Ttab, Hg, Wg, t0 + (int)v, (int)(u - v * Hg), (int)(s - u * Wg), sub, c, sn);
     };
     float c[4] = {1.f, 1.f, 1.f, 1.f}, sn[4] = {0.f, 0.f, 0.f, 0.f};
     if (tab != nullptr && share) angles(s_of[0], c, sn);      // row 0 of a group exists whenever any does
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-    if (o_of[j] == nullptr) continue;
-    T* o = o_of[j];
-    const uint4 raw = raw_of[j];
-    if (w == nullptr && tab == nullptr) {                 // plain move
-        *reinterpret_cast<uint4*>(o + sub * 8) = raw;
-        continue;
-    }
-    const T* e = reinterpret_cast<const T*>(&raw);
-    float f[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = (float)e[i];
-    if (w != nullptr) {
-        const T* we = reinterpret_cast<const T*>(&wraw);
-        float ss = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
-#pragma unroll
-        for (int off = 8; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
-        const float rs = rsqrtf(ss / (float)D + eps);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f[i] = (float)(T)((float)(T)(f[i] * rs) * (float)we[i]);
-    }
-    T res[8];
-    if (tab != nullptr) {
-        if (!share) angles(s_of[j], c, sn);
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-            const float x0 = f[2 * jj], x1 = f[2 * jj + 1];
-            // two products, then one add, each rounded: the order of operations of the eager expression
-            res[2 * jj] = (T)__fadd_rn(__fmul_rn(x0, c[jj]), __fmul_rn(-x1, sn[jj]));
-            res[2 * jj + 1] = (T)__fadd_rn(__fmul_rn(x1, c[jj]), __fmul_rn(x0, sn[jj]));
+        if (o_of[j] == nullptr) continue;
+        T* o = o_of[j];
+        if (w == nullptr && tab == nullptr) {                 // plain move
+            *reinterpret_cast<uint4*>(o + sub * 8) = raw_of[j];
+            continue;
         }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) res[i] = (T)f[i];
-    }
-    *reinterpret_cast<uint4*>(o + sub * 8) = *reinterpret_cast<const uint4*>(res);
+        if (tab != nullptr && !share) angles(s_of[j], c, sn);
+        *reinterpret_cast<uint4*>(o + sub * 8) = norm_rope_piece<T>(raw_of[j], wraw, w != nullptr, tab != nullptr, c, sn, eps);
     }
 }
 

@@ -27,6 +27,11 @@ class Bsa3dParams(C.Structure):
         "tq", "hq", "wq", "tk", "hk", "wk", "k_sel")] + [("sm_scale", C.c_float), ("cdf_threshold", C.c_float)]
 
 
+class BsaQkNorm(C.Structure):
+    _fields_ = [("q_weight", C.c_void_p), ("k_weight", C.c_void_p), ("rope_table", C.c_void_p), ("table_T", C.c_int),
+                ("t_offset_q", C.c_int), ("t_offset_k", C.c_int), ("eps", C.c_float)]
+
+
 _i, _i64, _p, _f = C.c_int, C.c_int64, C.c_void_p, C.c_float
 _strides = C.POINTER(C.c_int64)
 
@@ -50,6 +55,8 @@ SIGNATURES = {
     "bsa_workspace_bytes": (C.c_size_t, [C.POINTER(Bsa3dParams)]),
     "bsa_fwd_3d": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
                         _p, C.c_size_t, _p, _p, _p, _p]),
+    "bsa_fwd_3d_qknorm": (_i, [C.POINTER(Bsa3dParams), C.POINTER(BsaQkNorm), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
+                               _p, _strides, _p, C.c_size_t, _p, _p, _p, _p]),
     "bsa_fwd_3d_static": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
                                _p, _p, _p, _p]),
     "bsa_thw_prepare": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, C.c_size_t, _p]),

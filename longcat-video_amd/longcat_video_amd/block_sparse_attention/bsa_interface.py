@@ -402,11 +402,14 @@ def flash_attn_bsa(q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold,
 # R9: the operator
 # ---------------------------------------------------------------------------
 def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k, want_selection=False, out=None,
-            cdf_threshold=None, static_scratch=False):
+            cdf_threshold=None, static_scratch=False, qk_norm=None):
     """`out`: optional [B,H,Sq,D] view (any B/H/S strides, contiguous D) to write into.  `sparsity` may be
     None when `cdf_threshold` is given (bsa_interface.py:268-277).  `static_scratch`: run through
     bsa_fwd_3d_static, which keeps its scratch memory in a buffer built into the library instead of a
-    workspace tensor (problems beyond that buffer raise; calls on one GPU must not overlap)."""
+    workspace tensor (problems beyond that buffer raise; calls on one GPU must not overlap).
+    `qk_norm` = (q_weight, k_weight, rope_table, table_T, t_offset_q, t_offset_k, eps): q and k are the raw
+    projections and are normalised per head and rotated inside the operator's own passes (bsa_fwd_3d_qknorm;
+    bf16 / fp16 and 64-token chunks only)."""
     _need_gpu(q, k, v)
     B, H, Sq, D = q.shape
     Tq, Hq, Wq = (int(x) for x in latent_shape_q)
@@ -441,7 +444,17 @@ def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k,
         lens = torch.empty(B, H, nbq, dtype=torch.int32, device=q.device)
         score = torch.empty(B, H, nbq, nbk, dtype=q.dtype, device=q.device)
     with torch.cuda.device(q.device):
-        if static_scratch:
+        if qk_norm is not None:
+            qw, kw, tab, table_T, t_off_q, t_off_k, eps = qk_norm
+            qw, kw = qw.to(q.dtype).contiguous(), kw.to(q.dtype).contiguous()
+            q_normed = torch.empty(B, H, Sq, D, dtype=q.dtype, device=q.device)
+            n = _capi.BsaQkNorm(_ptr(qw), _ptr(kw), _ptr(tab), int(table_T), int(t_off_q), int(t_off_k), float(eps))
+            _capi.check(lib.bsa_fwd_3d_qknorm(
+                C.byref(prm), C.byref(n), _ptr(q), _capi.strides3(q.stride()[:3]), _ptr(q_normed),
+                _capi.strides3(q_normed.stride()[:3]), _ptr(k), _capi.strides3(k.stride()[:3]),
+                _ptr(v), _capi.strides3(v.stride()[:3]), _ptr(o), _capi.strides3(o.stride()[:3]),
+                _ptr(ws), need, _ptr(idx), _ptr(lens), _ptr(score), _stream(q)), "flash_attn_bsa_3d (q/k norm inside)")
+        elif static_scratch:
             _capi.check(lib.bsa_fwd_3d_static(
                 C.byref(prm), _ptr(q), _capi.strides3(q.stride()[:3]), _ptr(k), _capi.strides3(k.stride()[:3]),
                 _ptr(v), _capi.strides3(v.stride()[:3]), _ptr(o), _capi.strides3(o.stride()[:3]),

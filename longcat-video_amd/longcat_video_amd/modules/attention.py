@@ -314,8 +314,9 @@ class Attention(nn.Module):
         b = tune_linear(x, self.proj.weight, self.proj.bias, residual=residual)
         return a, b
 
-    def _process_attn(self, q, k, v, shape, out=None):
-        """attention.py:50-105, block-sparse branch; writes into `out` ([B,H,SQ,D] view) if given."""
+    def _process_attn(self, q, k, v, shape, out=None, qk_norm=None):
+        """attention.py:50-105, block-sparse branch; writes into `out` ([B,H,SQ,D] view) if given.  `qk_norm`: q and
+        k are the raw projections, normalised and rotated inside the operator (see _bsa_3d)."""
         B, H, SQ, D = q.shape
         SKV = k.shape[2]
         if not (self.enable_bsa and shape[0] > 1):
@@ -330,7 +331,20 @@ class Attention(nn.Module):
         if prm["sparsity"] is None and prm["cdf_threshold"] is None:
             raise ValueError
         return _bsa_3d(q, k, v, (Tq, Hh, W), (Tk, Hh, W), prm["sparsity"], prm["chunk_3d_shape_q"],
-                       prm["chunk_3d_shape_k"], out=out, cdf_threshold=prm["cdf_threshold"])
+                       prm["chunk_3d_shape_k"], out=out, cdf_threshold=prm["cdf_threshold"], qk_norm=qk_norm)
+
+    def _norm_inside_operator(self, x, shape, num_cond_latents, return_kv):
+        """True when q and k can go to the operator as projected: its passes over them (chunk means of q, k into
+        the attention kernel's operand order) then apply the norm and the rotation, and the two stand-alone passes
+        drop out.  One operator call over the whole grid, 64-token chunks, no k cache wanted."""
+        if return_kv or (num_cond_latents is not None and num_cond_latents > 0) or self.head_dim != 128:
+            return False
+        if not (self.enable_bsa and shape[0] > 1) or x.dtype not in (torch.bfloat16, torch.float16):
+            return False
+        prm = dict(chunk_3d_shape_q=[4, 4, 8], chunk_3d_shape_k=[4, 4, 8])
+        prm.update(self.bsa_params or {})
+        fits = lambda c: int(c[0]) * int(c[1]) * int(c[2]) == 64 and max(int(e) for e in c) <= 8
+        return fits(prm["chunk_3d_shape_q"]) and fits(prm["chunk_3d_shape_k"])
 
     def _project_qkv(self, x):
         B, N, C = x.shape
@@ -348,6 +362,15 @@ class Attention(nn.Module):
         if self._fused_projection(x, shape, return_kv):
             q, k, v = qkv_projection(x, self.qkv.weight, self.qkv.bias, self.q_norm.weight, self.k_norm.weight, shape,
                                      Hn, eps=eps)
+        elif self._norm_inside_operator(x, shape, num_cond_latents, return_kv):
+            # q, k, v stay where the projection left them: the operator's pass over q (chunk means) normalises and
+            # rotates it into a per-head tensor of its own, its pass over k (fragment order) does the same on the way
+            qs, ks, v = self._project_qkv(x)
+            o = torch.empty(B, N, Hn, D, dtype=x.dtype, device=x.device)
+            tab = rope_table(shape, D, x.device)
+            self._process_attn(qs, ks, v, shape, out=o.permute(0, 2, 1, 3),
+                               qk_norm=(self.q_norm.weight, self.k_norm.weight, tab, int(shape[0]), 0, 0, eps))
+            return self._linear(o.view(B, N, C), self.proj, self.proj_loras, residual=residual)
         else:
             # q moves into a per-head tensor on the way (the attention kernel fetches its rows tile by tile); k is
             # normed and rotated where it lies and v stays where it is: the operator reads both once, to rewrite
