@@ -62,7 +62,21 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return out
 
 
-_GEMM_WORKSPACES = {}
+class _Bounded(dict):
+    """A dict that forgets its oldest entry beyond `limit` (insertion order): the caches below are keyed by stream or
+    by grid, and a long-lived process that keeps creating streams or changing resolutions must not grow them forever."""
+
+    def __init__(self, limit: int):
+        super().__init__()
+        self.limit = limit
+
+    def __setitem__(self, key, value):
+        if key not in self and len(self) >= self.limit:
+            del self[next(iter(self))]
+        super().__setitem__(key, value)
+
+
+_GEMM_WORKSPACES = _Bounded(16)          # 64 MiB each
 
 
 def _gemm_workspace(device) -> torch.Tensor:
@@ -190,7 +204,7 @@ def qkv_projection(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
     return qkv[0], qkv[1], qkv[2]
 
 
-_ROPE_TABLES = {}
+_ROPE_TABLES = _Bounded(32)
 
 
 def rope_table(grid_size, head_dim: int, device, base: float = 10000.0) -> torch.Tensor:

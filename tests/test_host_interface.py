@@ -73,3 +73,15 @@ def test_no_cpu_fallback_with_or_without_gradients():
 
 def test_num_selected():
     assert I.num_selected(0.9375, 1440) == 90 and I.num_selected(0.9, 10) == 0
+
+
+def test_module_caches_are_bounded():
+    """The per-stream GEMM workspaces and the per-grid rotation tables forget their oldest entry beyond a limit."""
+    from longcat_video_amd.modules import attention as A
+    d = A._Bounded(3)
+    for i in range(5):
+        d[i] = i
+    assert list(d) == [2, 3, 4]
+    d[3] = 30                                    # rewriting a key evicts nothing
+    assert list(d) == [2, 3, 4] and d[3] == 30
+    assert isinstance(A._GEMM_WORKSPACES, A._Bounded) and isinstance(A._ROPE_TABLES, A._Bounded)
