@@ -122,6 +122,68 @@ def test_fwd_3d_plan_and_workspace():
     assert lib.bsa_fwd_3d(None, *args, ws, need, None, None, None, None) == _capi.BSA_ERR_BAD_ARG
 
 
+def test_gemm_and_qkv_projection_reject_bad_arguments():
+    lib = _capi.load()
+
+    def gemm(x=FAKE, ldx=256, w=FAKE, ldw=256, bias=None, res=None, ldr=0, out=FAKE, ldo=256, M=300, N=256, K=256):
+        return lib.bsa_gemm_bf16(x, ldx, w, ldw, bias, res, ldr, out, ldo, M, N, K, None)
+
+    assert gemm(x=None) == _capi.BSA_ERR_BAD_ARG
+    assert gemm(out=None) == _capi.BSA_ERR_BAD_ARG
+    assert gemm(K=96, ldx=96, ldw=96) == _capi.BSA_ERR_UNSUPPORTED and "64" in _capi.last_error()
+    assert gemm(N=200, ldo=200) == _capi.BSA_ERR_UNSUPPORTED and "128" in _capi.last_error()
+    assert gemm(ldx=128) == _capi.BSA_ERR_BAD_ARG                   # row stride below K
+    assert gemm(ldo=128) == _capi.BSA_ERR_BAD_ARG                   # row stride below N
+    assert gemm(res=FAKE, ldr=100) == _capi.BSA_ERR_BAD_ARG
+    assert gemm(M=0) == _capi.BSA_ERR_BAD_ARG
+    assert gemm(x=C.c_void_p(0x10008)) == _capi.BSA_ERR_BAD_ARG     # 16-byte alignment
+    assert gemm(ldx=1 << 23) == _capi.BSA_ERR_UNSUPPORTED
+
+    st = _capi.strides3([4 * 256 * 128, 256 * 128, 128])
+
+    def qkv(x=FAKE, q=FAKE, tab=FAKE, qw=FAKE, B=1, Hn=4, T=4, H=8, W=8, t0=0, table_T=4, D=128, K=512, eps=1e-6, strides=st):
+        return lib.bsa_qkv_projection(x, K, FAKE, K, None, qw, FAKE, tab, q, FAKE, FAKE, strides, B, Hn, T, H, W, t0, table_T, D, K, eps, None)
+
+    assert qkv(D=64) == _capi.BSA_ERR_UNSUPPORTED
+    assert qkv(x=None) == _capi.BSA_ERR_BAD_ARG
+    assert qkv(q=None) == _capi.BSA_ERR_BAD_ARG
+    assert qkv(tab=None) == _capi.BSA_ERR_BAD_ARG
+    assert qkv(qw=None) == _capi.BSA_ERR_BAD_ARG
+    assert qkv(T=0) == _capi.BSA_ERR_BAD_ARG
+    assert qkv(t0=2) == _capi.BSA_ERR_SHAPE                         # frames 2..6 of a table of 4
+    assert qkv(K=100) == _capi.BSA_ERR_UNSUPPORTED
+    assert qkv(eps=-1.0) == _capi.BSA_ERR_BAD_ARG
+    assert qkv(strides=_capi.strides3([4 * 256 * 128, 256 * 128, 100])) == _capi.BSA_ERR_BAD_ARG
+
+
+def test_fwd_3d_qknorm_rejects_bad_arguments():
+    lib = _capi.load()
+    prm = _capi.Bsa3dParams(1, 4, 128, _capi.BSA_BF16, 4, 8, 8, 4, 8, 8, 4, 4, 4, 4, 4, 4, 2, 0.0883883)
+    need = lib.bsa_workspace_bytes(C.byref(prm))
+    st = _capi.strides3([4 * 256 * 128, 256 * 128, 128])
+    ws = C.c_void_p(0x100000)
+
+    def call(p=prm, n=None, qn=FAKE, q_weight=FAKE, tab=FAKE, table_T=4, t_q=0, t_k=0, eps=1e-6):
+        norm = _capi.BsaQkNorm(q_weight, FAKE, tab, table_T, t_q, t_k, eps) if n is None else n
+        return lib.bsa_fwd_3d_qknorm(C.byref(p), C.byref(norm) if norm is not False else None, FAKE, st, qn, st, FAKE, st, FAKE, st,
+                                     FAKE, st, ws, need, None, None, None, None)
+
+    assert call(n=False) == _capi.BSA_ERR_BAD_ARG
+    assert call(qn=None) == _capi.BSA_ERR_BAD_ARG
+    assert call(q_weight=None) == _capi.BSA_ERR_BAD_ARG
+    assert call(tab=None) == _capi.BSA_ERR_BAD_ARG
+    assert call(table_T=3) == _capi.BSA_ERR_SHAPE
+    assert call(t_k=1) == _capi.BSA_ERR_SHAPE
+    assert call(eps=-1.0) == _capi.BSA_ERR_BAD_ARG
+    assert call(q_weight=C.c_void_p(0x10008)) == _capi.BSA_ERR_BAD_ARG
+    big = _capi.Bsa3dParams(1, 4, 128, _capi.BSA_BF16, 4, 8, 8, 4, 8, 8, 4, 4, 8, 4, 4, 8, 1, 0.0883883)      # 128-token chunks
+    assert call(p=big) == _capi.BSA_ERR_UNSUPPORTED and "64-token" in _capi.last_error()
+    f32 = _capi.Bsa3dParams(1, 4, 128, _capi.BSA_F32, 4, 8, 8, 4, 8, 8, 4, 4, 4, 4, 4, 4, 2, 0.0883883)
+    assert call(p=f32) == _capi.BSA_ERR_UNSUPPORTED
+    long_axis = _capi.Bsa3dParams(1, 4, 128, _capi.BSA_BF16, 4, 8, 16, 4, 8, 16, 1, 4, 16, 1, 4, 16, 2, 0.0883883)  # 16 positions on one axis
+    assert call(p=long_axis) == _capi.BSA_ERR_UNSUPPORTED
+
+
 def test_status_to_exception_mapping():
     lib = _capi.load()
     rc = lib.bsa_topk_from_score(FAKE, FAKE, None, FAKE, 1, 1, 4, 4, 5, _capi.BSA_BF16, None)

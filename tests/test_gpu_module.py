@@ -401,24 +401,24 @@ def test_linear_tuning_keeps_results_and_is_remembered():
     assert torch.equal(after, M().linear_bf16(x, w, b).cpu())          # the remembered choice is deterministic
 
 
-@pytest.mark.parametrize("grid", [(4, 8, 8), (3, 6, 10)])
-def test_operator_with_the_norm_inside_equals_the_separate_passes(grid):
+@pytest.mark.parametrize("grid,dtype", [((4, 8, 8), torch.bfloat16), ((3, 6, 10), torch.bfloat16), ((2, 9, 8), torch.float16)])
+def test_operator_with_the_norm_inside_equals_the_separate_passes(grid, dtype):
     """bsa_fwd_3d_qknorm (q and k normalised and rotated inside the operator's own passes) against bsa_norm_rope
     followed by bsa_fwd_3d: same selection, same output bits; a grid of whole chunks and a ragged one; q and k as
     strided views into a token-major projection output."""
     from longcat_video_amd.block_sparse_attention import bsa_interface as bi
     S = grid[0] * grid[1] * grid[2]
     g = torch.Generator().manual_seed(S)
-    qkv = (torch.randn(2, S, 3, 4, 128, generator=g) * 2).bfloat16().cuda()
-    qw = (1 + 0.1 * torch.randn(128, generator=g)).bfloat16().cuda()
-    kw = (1 + 0.1 * torch.randn(128, generator=g)).bfloat16().cuda()
+    qkv = (torch.randn(2, S, 3, 4, 128, generator=g) * 2).to(dtype).cuda()
+    qw = (1 + 0.1 * torch.randn(128, generator=g)).to(dtype).cuda()
+    kw = (1 + 0.1 * torch.randn(128, generator=g)).to(dtype).cuda()
     qs, ks, vs = qkv.permute(2, 0, 3, 1, 4).unbind(0)
     att = M()
     tab = att.rope_table(grid, 128, qkv.device)
     got, idx, lens, score = bi._bsa_3d(qs, ks, vs, grid, grid, 0.5, (4, 4, 4), (4, 4, 4), True,
                                        qk_norm=(qw, kw, tab, grid[0], 0, 0, 1e-6))
-    q = att.norm_rope(qs, torch.empty(2, 4, S, 128, dtype=torch.bfloat16, device="cuda"), qw, grid)
-    k = att.norm_rope(ks, torch.empty(2, 4, S, 128, dtype=torch.bfloat16, device="cuda"), kw, grid)
+    q = att.norm_rope(qs, torch.empty(2, 4, S, 128, dtype=dtype, device="cuda"), qw, grid)
+    k = att.norm_rope(ks, torch.empty(2, 4, S, 128, dtype=dtype, device="cuda"), kw, grid)
     want, idx2, lens2, score2 = bi._bsa_3d(q, k, vs, grid, grid, 0.5, (4, 4, 4), (4, 4, 4), True)
     assert torch.equal(score, score2) and torch.equal(idx, idx2) and torch.equal(lens, lens2)
     assert torch.equal(got, want)
