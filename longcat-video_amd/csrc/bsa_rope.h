@@ -33,6 +33,12 @@ __device__ inline void rope_angles(const float* __restrict__ tab, int Ttab, int 
     }
 }
 
+// x of the lane N positions further on in its row of 16 lanes (cyclic)
+template <int N>
+__device__ inline float row_ror(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x120 + N, 0xf, 0xf, false));
+}
+
 // The row piece of this lane through the norm (wraw: the lane's 8 weights; skipped when !do_norm) and the rotation
 // (skipped when !do_rope).  The 16 lanes of the row must all be active: the sum of squares crosses them.
 template <typename T>
@@ -48,8 +54,12 @@ __device__ inline uint4 norm_rope_piece(uint4 raw, uint4 wraw, bool do_norm, boo
         float ss = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
-#pragma unroll
-        for (int off = 8; off > 0; off >>= 1) ss = ss + __shfl_xor(ss, off);
+        // sum over the 16 lanes of the row, which are one DPP row: four rotations within the row (8, 4, 2, 1) leave the
+        // total in every lane, without a trip through the LDS crossbar that a lane shuffle by 4 or 8 would take
+        ss = ss + row_ror<8>(ss);
+        ss = ss + row_ror<4>(ss);
+        ss = ss + row_ror<2>(ss);
+        ss = ss + row_ror<1>(ss);
         // the hardware's reciprocal square root (1 ulp) named directly: rsqrtf() expands differently under different
         // floating-point flags, and the files that share this function are compiled with different ones
         const float rs = __builtin_amdgcn_rsqf(ss * (1.0f / (float)kRopeD) + eps);
