@@ -59,8 +59,9 @@ template <typename T, bool TRANSPOSE>
 __global__ __launch_bounds__(256) void frag_kernel(const T* __restrict__ src, int64_t sB, int64_t sH, int64_t sS,
                                                    char* __restrict__ dst, Grid3 g, int Hn, T* __restrict__ pooled,
                                                    uint64_t* __restrict__ tile_valid, int is_bf16, RowTransform tr) {
-    // rows padded to 264 B: the transposing reads below walk down a column
-    constexpr int kPitch = kD + 4;
+    // rows padded to 264 B for K (16-byte pieces read row by row) and to 288 B for V, whose transposing reads
+    // fetch 4 keys x 16 d per 16 lanes: with rows 72 banks apart the four keys of a patch fall on different banks
+    constexpr int kPitch = TRANSPOSE ? kD + 16 : kD + 4;
     __shared__ __attribute__((aligned(16))) T tile[kTile * kPitch];
     const int tiles_per_chunk = g.chunk() / kTile;
     // Workgroup -> (tile, batch * head).  For a token-major source (the heads of a token next to each other, as a
@@ -207,10 +208,14 @@ __global__ __launch_bounds__(256) void frag_kernel(const T* __restrict__ src, in
 #pragma unroll
             for (int j = 0; j < 8; ++j) piece[j] = s[j];
         } else {
+            // ds_read_b64_tr_b16: the 16 lanes of a group point at a 4-key x 16-d patch (lane s at key s / 4,
+            // d 4 (s % 4) .. + 4) and each receives the 4 keys of one d
             const int kh = f >> 3, s2 = (f >> 2) & 1, t = f & 3;
-            const uint16_t* s = reinterpret_cast<const uint16_t*>(tile) + 32 * t + lr;
+            const int s16 = l & 15, g1 = (l >> 4) & 1;
+            const T* src_lo = tile + (32 * kh + 16 * s2 + 4 * lh + (s16 >> 2)) * kPitch + 32 * t + 16 * g1 + 4 * (s16 & 3);
+            const s16x4 lo = lds_read_tr16(src_lo), hi = lds_read_tr16(src_lo + 8 * kPitch);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) piece[j] = s[(32 * kh + 16 * s2 + 8 * (j >> 2) + 4 * lh + (j & 3)) * kPitch];
+            for (int j = 0; j < 4; ++j) { piece[j] = (uint16_t)lo[j]; piece[4 + j] = (uint16_t)hi[j]; }
         }
         *reinterpret_cast<uint4*>(out + (int64_t)e * 16) = *reinterpret_cast<const uint4*>(piece);
     }
