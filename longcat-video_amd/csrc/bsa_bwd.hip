@@ -188,10 +188,14 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
 #pragma unroll
         for (int c = 0; c < 8; ++c) f.v[c] = frag_row<V8>(vr, tile, h, c, lane_off);
     };
-    auto compute = [&](const Frags& f, int64_t tile, int h, uint32_t hv) {
-        V8 kt[8];
+    // The transposed K_s fragments of a half are requested right behind the last MFMA that reads those of the half
+    // before (into the same registers), a whole half ahead of their use.
+    V8 kt[8];
+    auto load_kt = [&](int64_t tile, int h) {
 #pragma unroll
         for (int x = 0; x < 8; ++x) kt[x] = frag_tr<V8>(kst, tile, h, x >> 2, x & 3, lane_off);
+    };
+    auto compute = [&](const Frags& f, uint32_t hv, int64_t next_tile, int next_h) {
         f32x16 s[2], dp[2];
 #pragma unroll
         for (int qq = 0; qq < 2; ++qq)
@@ -223,6 +227,9 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
                 acc[t][1] = mfma32(kt[4 * st + t], ds1, acc[t][1]);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);               // the loads below overwrite what the MFMAs above read
+        load_kt(next_tile, next_h);
+        __builtin_amdgcn_sched_barrier(0);
     };
     const int ntiles = n * nsub;
     auto tile_at = [&](int tp) -> int64_t {
@@ -233,13 +240,14 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
         Frags fa, fb;
         int64_t tile = tile_at(0);
         load(fa, tile, 0);
+        load_kt(tile, 0);
         for (int tp = 0; tp < ntiles; ++tp) {
             const uint64_t valid = tile_valid != nullptr ? tile_valid[tile] : ~0ull;
             load(fb, tile, 1);
-            compute(fa, tile, 0, (uint32_t)valid);
+            compute(fa, (uint32_t)valid, tile, 1);
             const int64_t next = tile_at(tp + 1);
             load(fa, next, 0);                            // behind the last tile: loaded again, not used
-            compute(fb, tile, 1, (uint32_t)(valid >> 32));
+            compute(fb, (uint32_t)(valid >> 32), next, 0);
             tile = next;
         }
     }
@@ -346,14 +354,20 @@ __global__ __launch_bounds__(64) void bwd_dkv_kernel(const T* __restrict__ ks, c
 #pragma unroll
         for (int c = 0; c < 8; ++c) f.q[c] = frag_row<V8>(qr, tile, h, c, lane_off);
     };
-    auto compute = [&](const Rows& f, int64_t tile, int h) {
-        V8 drow[kDK ? 8 : 1], tr[8];
+    // The dO rows (dK) and the transposed fragments of a half are requested right behind the last MFMA that reads
+    // those of the half before (into the same registers): most of a half ahead of their use, at no cost in registers.
+    V8 drow[kDK ? 8 : 1], tr[8];
+    auto load_drow = [&](int64_t tile, int h) {
         if constexpr (kDK) {
 #pragma unroll
             for (int c = 0; c < 8; ++c) drow[c] = frag_row<V8>(dor, tile, h, c, lane_off);
         }
+    };
+    auto load_tr = [&](int64_t tile, int h) {
 #pragma unroll
         for (int x = 0; x < 8; ++x) tr[x] = frag_tr<V8>(trp, tile, h, x >> 2, x & 3, lane_off);
+    };
+    auto compute = [&](const Rows& f, int64_t tile, int h, int64_t next_tile, int next_h) {
         // accumulator i <-> query 8 (i / 4) + 4 lh + i % 4 of the half, key lr (+ 32)
         const int64_t qrow = bh * Sq + tile * kTile + 32 * h + 4 * lh;
         f32x16 s[2], dp[kDK ? 2 : 1];
@@ -367,31 +381,48 @@ __global__ __launch_bounds__(64) void bwd_dkv_kernel(const T* __restrict__ ks, c
 #pragma unroll
         for (int c = 0; c < 8; ++c)
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk) {
-                s[kk] = mfma32(f.q[c], kreg[kk][c], s[kk]);
-                if constexpr (kDK) dp[kk] = mfma32(drow[c], vreg[kk][c], dp[kk]);
-            }
+            for (int kk = 0; kk < 2; ++kk) s[kk] = mfma32(f.q[c], kreg[kk][c], s[kk]);
+        // P = exp2(S - M2); for dK the MFMAs of dP run beside it.  M2 and delta of the four queries of an accumulator
+        // group are fetched where they are used (L1 hits) so that they do not sit in registers through the products.
+        if constexpr (kDK) {
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-            // M2 and delta of the four queries of this accumulator group, fetched where they are used (L1 hits) so
-            // that they do not sit in registers through the products above
-            const float4 mm = *reinterpret_cast<const float4*>(m2 + qrow + 8 * g4);
-            const float mv[4] = {mm.x, mm.y, mm.z, mm.w};
-            float dl[4] = {0.f, 0.f, 0.f, 0.f};
-            if constexpr (kDK) {
-                const float4 dd = *reinterpret_cast<const float4*>(delta + qrow + 8 * g4);
-                dl[0] = dd.x; dl[1] = dd.y; dl[2] = dd.z; dl[3] = dd.w;
-            }
-#pragma unroll
-            for (int kk = 0; kk < 2; ++kk)
+            for (int c = 0; c < 8; ++c) {
+                dp[0] = mfma32(drow[c], vreg[0][c], dp[0]);
+                dp[1] = mfma32(drow[c], vreg[1][c], dp[1]);
+                const int g4 = c >> 1, kk = c & 1;
+                const float4 mm = *reinterpret_cast<const float4*>(m2 + qrow + 8 * g4);
+                const float mv[4] = {mm.x, mm.y, mm.z, mm.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int i = 4 * g4 + j;
-                    float pi = __builtin_amdgcn_exp2f(s[kk][i] - mv[j]);
-                    if (!key_ok[kk]) pi = 0.f;
-                    if constexpr (kDK) pi = pi * (dp[kk][i] - dl[j]);
-                    s[kk][i] = pi;                               // P for dV, dS for dK
+                    const float pi = __builtin_amdgcn_exp2f(s[kk][4 * g4 + j] - mv[j]);
+                    s[kk][4 * g4 + j] = key_ok[kk] ? pi : 0.f;
                 }
+            }
+            __builtin_amdgcn_sched_barrier(0);           // the loads below overwrite what the MFMAs above read
+            load_drow(next_tile, next_h);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const float4 dd = *reinterpret_cast<const float4*>(delta + qrow + 8 * g4);
+                const float dl[4] = {dd.x, dd.y, dd.z, dd.w};
+#pragma unroll
+                for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) s[kk][4 * g4 + j] = s[kk][4 * g4 + j] * (dp[kk][4 * g4 + j] - dl[j]);     // dS
+            }
+        } else {
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const float4 mm = *reinterpret_cast<const float4*>(m2 + qrow + 8 * g4);
+                const float mv[4] = {mm.x, mm.y, mm.z, mm.w};
+#pragma unroll
+                for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float pi = __builtin_amdgcn_exp2f(s[kk][4 * g4 + j] - mv[j]);
+                        s[kk][4 * g4 + j] = key_ok[kk] ? pi : 0.f;                                                    // P
+                    }
+            }
         }
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
@@ -402,6 +433,9 @@ __global__ __launch_bounds__(64) void bwd_dkv_kernel(const T* __restrict__ ks, c
                 acc[t][1] = mfma32(tr[4 * st + t], b1, acc[t][1]);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        load_tr(next_tile, next_h);
+        __builtin_amdgcn_sched_barrier(0);
     };
     const int ntiles = count * qsub;
     auto tile_at = [&](int tp) -> int64_t {
@@ -412,12 +446,14 @@ __global__ __launch_bounds__(64) void bwd_dkv_kernel(const T* __restrict__ ks, c
         Rows fa, fb;
         int64_t tile = tile_at(0);
         load(fa, tile, 0);
+        load_drow(tile, 0);
+        load_tr(tile, 0);
         for (int tp = 0; tp < ntiles; ++tp) {
             load(fb, tile, 1);
-            compute(fa, tile, 0);
-            const int64_t next = tile_at(tp + 1);
-            load(fa, next, 0);                            // behind the last tile: loaded again, not used
-            compute(fb, tile, 1);
+            const int64_t next = tile_at(tp + 1);         // behind the last tile: the last one again, loaded and not used
+            compute(fa, tile, 0, tile, 1);
+            load(fa, next, 0);
+            compute(fb, tile, 1, next, 0);
             tile = next;
         }
     }
