@@ -8,18 +8,19 @@
 //   ds = p * (dp - delta) rounded to the storage type, p rounded to the storage type for dV;
 //   dV = sum p^T do,  dK = sm_scale * sum ds^T q,  dQ = ln 2 * sum ds k_s  (fp32 accumulators, one final rounding).
 //
-// Data movement as in bsa_fwd_frag.hip: every operand that an MFMA reads from memory is first rewritten into
+// Data movement of dQ as in bsa_fwd_frag.hip: every operand that an MFMA reads from memory is first rewritten into
 // fragment order (frag_kernel), so a wavefront loads it with one coalesced 16-byte load per lane and fragment and
 // LDS carries nothing.  "row layout" = the K layout of that file (A operand whose rows are tokens), "transposed
 // layout" = its V layout (A operand whose rows are head-dim columns, contraction over 16 tokens in accumulator
-// order).  Needed: k_s in both layouts and v in row layout (dQ); q and do in both layouts (dK, dV).
+// order).  Needed: k_s in both layouts and v in row layout.
 //
 // dQ: one wavefront per 64 query rows (two halves of 32, so that every K_s and V fragment feeds two MFMAs).
-// S^T = K_s Q^T and dP^T = V dO^T (Q and dO rows in registers as B operands) put one query per lane, so M2 and delta are one scalar per lane and dS^T in the accumulator registers is already
-// the B operand of dQ^T += K_s^T dS^T.
-// dK, dV: one wavefront per 64 keys and one kernel per gradient.  S = Q K_s^T and dP = dO V^T (K_s and V rows in
+// S^T = K_s Q^T and dP^T = V dO^T (Q and dO rows in registers as B operands) put one query per lane, so M2 and
+// delta are one scalar per lane and dS^T in the accumulator registers is already the B operand of
+// dQ^T += K_s^T dS^T.
+// dK, dV: one kernel, a workgroup of two wavefronts per 64 keys.  S = Q K_s^T and dP = dO V^T (K_s and V rows in
 // registers as B operands) put one key per lane; P and dS in the accumulator registers are the B operands of
-// dV^T += dO^T P and dK^T += Q^T dS.
+// dV^T += dO^T P and dK^T += Q^T dS.  Q and dO are read as they lie in memory, through LDS (see that kernel).
 // The query blocks of a KV block come from a bit matrix [KV block][query block] that a small kernel fills from
 // the forward's lists (ascending order for free).  Lists are expected to name a block at most once, as a
 // selection does; for a repeated block dQ follows the list (as the forward does) and dK / dV the bit matrix, like
@@ -267,67 +268,71 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
     }
 }
 
-// ------------------------------------------------------------------ dK, dV
-// One wavefront per 64 keys (one tile), as two halves of 32 so that every streamed Q / dO fragment feeds two MFMAs,
-// and one kernel per gradient - 64 keys of both accumulators (256 registers) plus the resident K_s and V rows and
-// the streamed fragments do not fit one wavefront's 512 registers.  kDK = false: dV (S from Q rows and K_s, P, then
-// dV^T += dO^T P).  kDK = true: dK (S again, dP from dO rows and V, dS, then dK^T += Q^T dS).  S is computed in
-// both: 80 MFMAs per tile pair instead of 64, at half the fragment bytes per MFMA.
-template <typename T, bool kDK>
-__global__ __launch_bounds__(64) void bwd_dkv_kernel(const T* __restrict__ ks, const T* __restrict__ v,
-                                                     const char* __restrict__ q_row, const char* __restrict__ q_tr,
-                                                     const char* __restrict__ do_row, const char* __restrict__ do_tr,
-                                                     const float* __restrict__ m2, const float* __restrict__ delta,
-                                                     const uint32_t* __restrict__ bits,
-                                                     const uint64_t* __restrict__ tile_valid, T* __restrict__ out,
-                                                     int64_t Sq, int64_t Sk, int bs_q, int bs_k, int words, float out_scale,
-                                                     const int32_t* __restrict__ order, int item_begin, int item_end, int round) {
+// ------------------------------------------------------------------ dK and dV in one kernel, Q and dO through LDS
+// One workgroup of two wavefronts per 64 keys; wavefront w owns keys 32 w .. 32 w + 31 and both of their gradients
+// (128 accumulator registers).  The Q and dO tiles of a query tile (64 rows x 256 B each, as they lie in memory)
+// go from global memory straight into LDS once per workgroup (global_load_lds_dwordx4; wavefront 0 brings Q and
+// the queries' M2 and delta, wavefront 1 brings dO), in halves of 32 queries, four stages deep (one in use, three on
+// their way), and both wavefronts take every operand from there: the row fragments (the A operands of S = Q K_s^T and
+// dP = dO V^T) with ds_read_b128, the transposed
+// ones (the A operands of dV^T += dO^T P and dK^T += Q^T dS) with ds_read_b64_tr_b16.  Per tile pair 32 KB leave
+// the caches instead of the 80 KB of fragment-order copies that separate dK and dV kernels stream, S is computed
+// once instead of twice (128 MFMAs per tile pair instead of 160), and no fragment-order copy of q or dO is made.
+// The LDS side of the DMA is linear in the lane index, so the swizzle that keeps both kinds of read free of bank
+// conflicts is applied on the global side: the 16-byte slot p of row r receives unit p ^ f(r),
+// f(r) = ((r << 1) & 14) | ((r >> 3) & 1): 16 consecutive rows, and the 4 consecutive rows of a transposing read,
+// land on different banks.
+constexpr int kBwdHalfTile = kTileBytes / 2;                 // 32 query rows of Q or of dO
+constexpr int kBwdStats = 1024;                              // M2 (128 B), delta (128 B), the rest filled blindly by the 64-lane DMA
+constexpr int kBwdStage = 2 * kBwdHalfTile + kBwdStats;      // one half tile of queries: Q rows, dO rows, M2, delta
+constexpr int kBwdStages = 4;                                // one in use, three on their way: a tile and a half ahead
+
+template <typename T>
+__global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, const T* __restrict__ dout,
+                                                       const T* __restrict__ ks, const T* __restrict__ v,
+                                                       const float* __restrict__ m2, const float* __restrict__ delta,
+                                                       const uint32_t* __restrict__ bits,
+                                                       const uint64_t* __restrict__ tile_valid, T* __restrict__ dk,
+                                                       T* __restrict__ dv, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int words,
+                                                       float dk_scale, const int32_t* __restrict__ order, int n_items, int round) {
     typedef typename Vec8<T>::type V8;
-    const int lane = threadIdx.x, lr = lane & 31, lh = lane >> 5;
-    const uint32_t lane_off = (uint32_t)lane * 16u;
+    extern __shared__ __attribute__((aligned(1024))) char bwd_lds[];
+    const int lane = threadIdx.x & 63, lr = lane & 31, lh = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int64_t groups = Sk / kTile;
-    // Items are taken longest list first (order: the tiles of every (batch, head) by descending number of query
-    // blocks), in groups of `round` workgroups of which every XCD (workgroup b runs on XCD b % 8) takes a contiguous
-    // run: the wavefronts that run side by side have lists of similar length, so they walk the query blocks at a
-    // similar pace and share Q / dO tiles in L2, and the long lists do not end up alone at the tail.
+    // items longest list first, every XCD on a contiguous run of each group of `round` (see launch_bwd)
     int64_t item;
     {
         const int local = blockIdx.x, r0 = local / round * round;
-        const int n = min(round, item_end - item_begin - r0), w = local - r0, x = w & 7;
-        item = order[item_begin + r0 + x * (n >> 3) + min(x, n & 7) + (w >> 3)];
+        const int n = min(round, n_items - r0), w = local - r0, x = w & 7;
+        item = order[r0 + x * (n >> 3) + min(x, n & 7) + (w >> 3)];
     }
     const int64_t bh = item / groups;
     const int64_t krow0 = (item % groups) * kTile;
     const int nbq = (int)(Sq / bs_q), nbk = (int)(Sk / bs_k), qsub = bs_q / kTile;
     const int kblk = (int)(krow0 / bs_k);
     const uint32_t* mask_row = bits + (bh * nbk + kblk) * words;
-    const int64_t q_tiles = Sq / kTile;
-    const char* qr = q_row + bh * q_tiles * kTileBytes;
-    const char* trp = (kDK ? q_tr : do_tr) + bh * q_tiles * kTileBytes;     // transposed operand of the last product
-    const char* dor = do_row + bh * q_tiles * kTileBytes;
 
-    V8 kreg[2][8], vreg[kDK ? 2 : 1][8];
-    bool key_ok[2] = {true, true};
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-        const int64_t row = bh * Sk + krow0 + 32 * kk + lr;
+    // resident: K_s and V rows of this wavefront's 32 keys, as B operands (lane = key lr, 8 consecutive d)
+    V8 kreg[8], vreg[8];
+    {
+        const int64_t row = bh * Sk + krow0 + 32 * wave + lr;
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
-            kreg[kk][c] = *reinterpret_cast<const V8*>(ks + row * kD + 16 * c + 8 * lh);
-            if constexpr (kDK) vreg[kk][c] = *reinterpret_cast<const V8*>(v + row * kD + 16 * c + 8 * lh);
+            kreg[c] = *reinterpret_cast<const V8*>(ks + row * kD + 16 * c + 8 * lh);
+            vreg[c] = *reinterpret_cast<const V8*>(v + row * kD + 16 * c + 8 * lh);
         }
-        if (tile_valid != nullptr) key_ok[kk] = (tile_valid[krow0 / kTile] >> (32 * kk + lr)) & 1ull;
     }
-    f32x16 acc[4][2];
+    bool key_ok = true;
+    if (tile_valid != nullptr) key_ok = (tile_valid[krow0 / kTile] >> (32 * wave + lr)) & 1ull;
+    f32x16 acc_dk[4], acc_dv[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[t][kk][i] = 0.f;
+        for (int i = 0; i < 16; ++i) { acc_dk[t][i] = 0.f; acc_dv[t][i] = 0.f; }
 
-    // the query blocks of this KV block, ascending, from the bit matrix into LDS
-    extern __shared__ int32_t qlist[];
+    // the query blocks of this KV block, ascending, from the bit matrix into LDS (behind the stages)
+    int32_t* qlist = reinterpret_cast<int32_t*>(bwd_lds + kBwdStages * kBwdStage);
     int count = 0;
     for (int w0 = 0; w0 < words; w0 += 64) {
         const int w = w0 + lane;
@@ -340,152 +345,169 @@ __global__ __launch_bounds__(64) void bwd_dkv_kernel(const T* __restrict__ ks, c
             if (lane >= off) upto += t;
         }
         int pos = count + upto - mine;
-        while (word != 0u) {
-            qlist[pos++] = 32 * w + __builtin_ctz(word);
-            word &= word - 1u;
-        }
+        if (wave == 0)
+            while (word != 0u) {
+                qlist[pos++] = 32 * w + __builtin_ctz(word);
+                word &= word - 1u;
+            }
         count += __shfl(upto, 63);
     }
     __syncthreads();
-    // The Q row fragments of a half tile of queries are requested one half ahead of their use, into two register
-    // buffers that take turns; the dO rows (dK) and the transposed fragments at the start of the half that uses them.
-    struct Rows { V8 q[8]; };
-    auto load = [&](Rows& f, int64_t tile, int h) {
-#pragma unroll
-        for (int c = 0; c < 8; ++c) f.q[c] = frag_row<V8>(qr, tile, h, c, lane_off);
-    };
-    // The dO rows (dK) and the transposed fragments of a half are requested right behind the last MFMA that reads
-    // those of the half before (into the same registers): most of a half ahead of their use, at no cost in registers.
-    V8 drow[kDK ? 8 : 1], tr[8];
-    auto load_drow = [&](int64_t tile, int h) {
-        if constexpr (kDK) {
-#pragma unroll
-            for (int c = 0; c < 8; ++c) drow[c] = frag_row<V8>(dor, tile, h, c, lane_off);
-        }
-    };
-    auto load_tr = [&](int64_t tile, int h) {
-#pragma unroll
-        for (int x = 0; x < 8; ++x) tr[x] = frag_tr<V8>(trp, tile, h, x >> 2, x & 3, lane_off);
-    };
-    auto compute = [&](const Rows& f, int64_t tile, int h, int64_t next_tile, int next_h) {
-        // accumulator i <-> query 8 (i / 4) + 4 lh + i % 4 of the half, key lr (+ 32)
-        const int64_t qrow = bh * Sq + tile * kTile + 32 * h + 4 * lh;
-        f32x16 s[2], dp[kDK ? 2 : 1];
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                s[kk][i] = 0.f;
-                if constexpr (kDK) dp[kk][i] = 0.f;
-            }
-#pragma unroll
-        for (int c = 0; c < 8; ++c)
-#pragma unroll
-            for (int kk = 0; kk < 2; ++kk) s[kk] = mfma32(f.q[c], kreg[kk][c], s[kk]);
-        // P = exp2(S - M2); for dK the MFMAs of dP run beside it.  M2 and delta of the four queries of an accumulator
-        // group are fetched where they are used (L1 hits) so that they do not sit in registers through the products.
-        if constexpr (kDK) {
-#pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                dp[0] = mfma32(drow[c], vreg[0][c], dp[0]);
-                dp[1] = mfma32(drow[c], vreg[1][c], dp[1]);
-                const int g4 = c >> 1, kk = c & 1;
-                const float4 mm = *reinterpret_cast<const float4*>(m2 + qrow + 8 * g4);
-                const float mv[4] = {mm.x, mm.y, mm.z, mm.w};
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float pi = __builtin_amdgcn_exp2f(s[kk][4 * g4 + j] - mv[j]);
-                    s[kk][4 * g4 + j] = key_ok[kk] ? pi : 0.f;
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);           // the loads below overwrite what the MFMAs above read
-            load_drow(next_tile, next_h);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const float4 dd = *reinterpret_cast<const float4*>(delta + qrow + 8 * g4);
-                const float dl[4] = {dd.x, dd.y, dd.z, dd.w};
-#pragma unroll
-                for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) s[kk][4 * g4 + j] = s[kk][4 * g4 + j] * (dp[kk][4 * g4 + j] - dl[j]);     // dS
-            }
-        } else {
-#pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const float4 mm = *reinterpret_cast<const float4*>(m2 + qrow + 8 * g4);
-                const float mv[4] = {mm.x, mm.y, mm.z, mm.w};
-#pragma unroll
-                for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const float pi = __builtin_amdgcn_exp2f(s[kk][4 * g4 + j] - mv[j]);
-                        s[kk][4 * g4 + j] = key_ok[kk] ? pi : 0.f;                                                    // P
-                    }
-            }
-        }
-#pragma unroll
-        for (int st = 0; st < 2; ++st) {
-            const V8 b0 = pack8<T, V8>(s[0], st), b1 = pack8<T, V8>(s[1], st);
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                acc[t][0] = mfma32(tr[4 * st + t], b0, acc[t][0]);
-                acc[t][1] = mfma32(tr[4 * st + t], b1, acc[t][1]);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        load_tr(next_tile, next_h);
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    const int ntiles = count * qsub;
+    const int ntiles = __builtin_amdgcn_readfirstlane(count) * qsub;          // the same in every lane; the compiler cannot tell
     auto tile_at = [&](int tp) -> int64_t {
         const int tc = min(tp, ntiles - 1);
-        return (int64_t)qlist[tc / qsub] * qsub + tc % qsub;
+        return (int64_t)__builtin_amdgcn_readfirstlane(qlist[tc / qsub]) * qsub + tc % qsub;
     };
-    if (ntiles > 0) {
-        Rows fa, fb;
-        int64_t tile = tile_at(0);
-        load(fa, tile, 0);
-        load_drow(tile, 0);
-        load_tr(tile, 0);
-        for (int tp = 0; tp < ntiles; ++tp) {
-            load(fb, tile, 1);
-            const int64_t next = tile_at(tp + 1);         // behind the last tile: the last one again, loaded and not used
-            compute(fa, tile, 0, tile, 1);
-            load(fa, next, 0);
-            compute(fb, tile, 1, next, 0);
-            tile = next;
+
+    // ---- global -> LDS
+    const uint32_t lds0 = lds_address(bwd_lds);
+    uint32_t voff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = 4 * i + (lane >> 4);                                     // + 16 j
+        const int f = ((row << 1) & 14) | ((row >> 3) & 1);
+        voff[i] = (uint32_t)(row * 256 + (((lane & 15) ^ f) << 4));
+    }
+    const uint32_t stat_gap = (uint32_t)(reinterpret_cast<const char*>(m2) - reinterpret_cast<const char*>(delta));
+    const uint32_t voff_stats = ((lane & 15) < 8 ? stat_gap : 0u) + (uint32_t)((lane & 7) * 16);
+    const char* tile_src = reinterpret_cast<const char*>(wave == 0 ? q : dout) + bh * Sq * (int64_t)(kD * 2);
+    const char* stat_src = reinterpret_cast<const char*>(delta) + bh * Sq * 4;
+    const int nhalves = 2 * ntiles;
+    // half hp = query half hp & 1 of the walk's tile hp / 2, into stage hp % kBwdStages
+    auto issue = [&](int hp, int stage) {
+        if (hp >= nhalves) return;
+        const int64_t tile = (int64_t)__builtin_amdgcn_readfirstlane((int)tile_at(hp >> 1));
+        const int h = hp & 1;
+        const char* src = tile_src + tile * kTileBytes + h * kBwdHalfTile;
+        const uint32_t dst = lds0 + stage * kBwdStage + wave * kBwdHalfTile;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) load_to_lds_16(src + j * 4096, voff[i], dst + j * 4096 + i * 1024);
+        if (wave == 0)
+            load_to_lds_16(stat_src + tile * (kTile * 4) + h * 128, voff_stats, lds0 + stage * kBwdStage + 2 * kBwdHalfTile);
+    };
+
+    // ---- LDS -> fragments
+    const uint32_t fl = (uint32_t)(((lr << 1) & 14) | ((lr >> 3) & 1));
+    uint32_t roff[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) roff[c] = (uint32_t)(lr * 256) + ((((uint32_t)(2 * c + lh)) ^ fl) << 4);
+    const int s16 = lane & 15, g1 = (lane >> 4) & 1, tx = s16 >> 2, ty = (s16 & 3) >> 1, tz = s16 & 1;
+    uint32_t toff[4][2];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi)
+            toff[t][hi] = (uint32_t)((4 * lh + tx + 8 * hi) * 256) + ((((uint32_t)(4 * t + 2 * g1 + ty)) ^ (uint32_t)((8 * lh + 2 * tx) | hi)) << 4) +
+                          (uint32_t)(tz * 8);
+    auto frag_tr_lds = [&](const char* part, int st2, int t) -> V8 {
+        const char* base = part + (16 * st2) * 256;
+        const s16x4 lo = lds_read_tr16(base + toff[t][0]), hi = lds_read_tr16(base + toff[t][1]);
+        return __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+    // one half tile of queries (32) against this wavefront's 32 keys: 32 MFMAs
+    auto compute = [&](const char* stage) {
+        const char* qt = stage;
+        const char* dt = stage + kBwdHalfTile;
+        const float* st_m2 = reinterpret_cast<const float*>(stage + 2 * kBwdHalfTile);
+        const float* st_dl = st_m2 + 32;
+        // S and dP accumulate in ordinary registers (the exponentials read them there): MFMAs from inline assembly,
+        // behind which the compiler adds no wait states, so the wait for the last one is written out
+        f32x16 s, dp;
+        mfma_s<true, false>(s, *reinterpret_cast<const V8*>(qt + roff[0]), kreg[0]);
+        mfma_s<true, false>(dp, *reinterpret_cast<const V8*>(dt + roff[0]), vreg[0]);
+#pragma unroll
+        for (int c = 1; c < 8; ++c) {
+            mfma_s<false, false>(s, *reinterpret_cast<const V8*>(qt + roff[c]), kreg[c]);
+            mfma_s<false, false>(dp, *reinterpret_cast<const V8*>(dt + roff[c]), vreg[c]);
+        }
+        asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        // accumulator i <-> query 8 (i / 4) + 4 lh + i % 4 of the half, key lr
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            const float4 mm = *reinterpret_cast<const float4*>(st_m2 + 8 * g4 + 4 * lh);
+            const float4 dd = *reinterpret_cast<const float4*>(st_dl + 8 * g4 + 4 * lh);
+            const float mv[4] = {mm.x, mm.y, mm.z, mm.w}, dl[4] = {dd.x, dd.y, dd.z, dd.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int i = 4 * g4 + j;
+                float pi = __builtin_amdgcn_exp2f(s[i] - mv[j]);
+                if (!key_ok) pi = 0.f;
+                s[i] = pi;                                   // P
+                dp[i] = pi * (dp[i] - dl[j]);                // dS
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int st2 = 0; st2 < 2; ++st2) {
+            const V8 bp = pack8<T, V8>(s, st2), bds = pack8<T, V8>(dp, st2);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                acc_dv[t] = mfma32(frag_tr_lds(dt, st2, t), bp, acc_dv[t]);
+                acc_dk[t] = mfma32(frag_tr_lds(qt, st2, t), bds, acc_dk[t]);
+            }
+        }
+    };
+    // At the end of half hp the loads of half hp + 1 must have landed; the two halves requested after it may still
+    // be on their way (wavefront 0 issues 9 loads per half, wavefront 1 issues 8).
+    auto await_next = [&](int hp) {
+        if (hp + 3 < nhalves) {
+            if (wave == 0) asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        }
+        __builtin_amdgcn_s_barrier();
+    };
+    if (nhalves > 0) {
+        issue(0, 0);
+        issue(1, 1);
+        issue(2, 2);
+        if (nhalves > 2) {
+            if (wave == 0) asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        __builtin_amdgcn_s_barrier();
+        for (int hp = 0; hp < nhalves; ++hp) {
+            // half hp + 3 takes the stage that half hp - 1 was read from: both wavefronts are past the barrier behind it
+            issue(hp + 3, (hp + 3) & 3);
+            compute(bwd_lds + (hp & 3) * kBwdStage);
+            await_next(hp);
         }
     }
-    // accumulator i of d tile t <-> d = 32 t + 8 (i / 4) + 4 lh + i % 4, key lr (+ 32)
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-        T* orow = out + (bh * Sk + krow0 + 32 * kk + lr) * kD;
+    // accumulator i of d tile t <-> d = 32 t + 8 (i / 4) + 4 lh + i % 4, key lr
+    {
+        const int64_t row = bh * Sk + krow0 + 32 * wave + lr;
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
-                T x[4];
+                T xk[4], xv[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const float a = acc[t][kk][4 * g4 + j];
-                    x[j] = kDK ? (T)(a * out_scale) : (T)a;
+                    xk[j] = (T)(acc_dk[t][4 * g4 + j] * dk_scale);
+                    xv[j] = (T)acc_dv[t][4 * g4 + j];
                 }
-                *reinterpret_cast<uint2*>(orow + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(x);
+                *reinterpret_cast<uint2*>(dk + row * kD + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(xk);
+                *reinterpret_cast<uint2*>(dv + row * kD + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(xv);
             }
     }
 }
 
 }  // namespace
 
-// Workspace of the backward, in bytes: seven fragment-order copies ([B*Hn][S/64][16 KB]: q and do in both
-// layouts, k_s in both, v in row layout), k_s in blocked order, delta and M2, the bit matrix, the lists in the dQ
-// kernel's visiting order, per KV block its number of query blocks, the KV tiles of every head by that number.
+// Workspace of the backward, in bytes: three fragment-order copies ([B*Hn][Sk/64][16 KB]: k_s in both layouts,
+// v in row layout), k_s in blocked order, delta and M2, the bit matrix, the lists in the dQ kernel's visiting
+// order, per KV block its number of query blocks, the KV tiles of every head by that number.
 size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride) {
     const size_t bh = (size_t)B * Hn;
     auto up = [](size_t x) { return (x + 255) / 256 * 256; };
     const size_t words = (size_t)((Sq / bs_q + 31) / 32);
-    return 4 * up(bh * Sq * kD * 2) + 4 * up(bh * Sk * kD * 2) + 2 * up(bh * Sq * 4) + up(bh * (Sk / bs_k) * words * 4) +
+    return 4 * up(bh * Sk * kD * 2) + 2 * up(bh * Sq * 4) + up(bh * (Sk / bs_k) * words * 4) +
            up(bh * (Sq / bs_q) * (size_t)idx_stride * 4) + up(bh * (Sk / bs_k) * 4) + up(bh * (Sk / kTile) * 4);
 }
 
@@ -497,10 +519,6 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     auto up = [](size_t x) { return (x + 255) / 256 * 256; };
     char* ws = static_cast<char*>(workspace);
     auto take = [&](size_t n) { char* p = ws; ws += up(n); return p; };
-    char* q_row = take(bh * Sq * kD * 2);
-    char* q_tr = take(bh * Sq * kD * 2);
-    char* do_row = take(bh * Sq * kD * 2);
-    char* do_tr = take(bh * Sq * kD * 2);
     char* ks_row = take(bh * Sk * kD * 2);
     char* ks_tr = take(bh * Sk * kD * 2);
     char* v_row = take(bh * Sk * kD * 2);
@@ -533,29 +551,29 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     hipLaunchKernelGGL(bwd_mask_kernel, dim3((unsigned)((lrows + 3) / 4)), dim3(256), 0, st, idx, lens, bits, nbq, nbk, idx_stride,
                        words, lrows);
     // blocked-order tensors as a grid of 64-token chunks along one axis
-    const Grid3 gq = make_grid((int)(Sq / kTile), 1, kTile, 1, 1, kTile), gk = make_grid((int)(Sk / kTile), 1, kTile, 1, 1, kTile);
-    const int64_t stq[3] = {(int64_t)Hn * Sq * kD, Sq * kD, kD}, stk[3] = {(int64_t)Hn * Sk * kD, Sk * kD, kD};
+    const Grid3 gk = make_grid((int)(Sk / kTile), 1, kTile, 1, 1, kTile);
+    const int64_t stk[3] = {(int64_t)Hn * Sk * kD, Sk * kD, kD};
     hipError_t e;
     hipLaunchKernelGGL(bwd_count_kernel, dim3((unsigned)((bh * nbk + 255) / 256)), dim3(256), 0, st, bits, counts, words, (int64_t)(bh * nbk));
     if ((e = launch_order_by_length(counts, order, (int)bh, nbk, bs_k / kTile, nbq, st)) != hipSuccess) return e;
     // dQ walks every list in the forward kernel's visiting order when the list is ascending (a selection in block
     // order); any other order is walked as given.  The order only moves fp32 roundings of the dQ sum.
     if ((e = launch_pace_order(idx, paced, lens, (int64_t)bh * nbq, nbk, idx_stride, st)) != hipSuccess) return e;
-    if ((e = launch_frag(q, stq, q_row, B, Hn, gq, dtype, false, st)) != hipSuccess) return e;
-    if ((e = launch_frag(q, stq, q_tr, B, Hn, gq, dtype, true, st)) != hipSuccess) return e;
-    if ((e = launch_frag(dout, stq, do_row, B, Hn, gq, dtype, false, st)) != hipSuccess) return e;
-    if ((e = launch_frag(dout, stq, do_tr, B, Hn, gq, dtype, true, st)) != hipSuccess) return e;
     if ((e = launch_frag(ks, stk, ks_row, B, Hn, gk, dtype, false, st)) != hipSuccess) return e;
     if ((e = launch_frag(ks, stk, ks_tr, B, Hn, gk, dtype, true, st)) != hipSuccess) return e;
     if ((e = launch_frag(v, stk, v_row, B, Hn, gk, dtype, false, st)) != hipSuccess) return e;
 
     const dim3 block(64);
-    const size_t lds = (size_t)nbq * sizeof(int32_t);         // a KV block's query blocks (bwd_dkv_kernel)
+    // the dK / dV kernel's LDS: four stages of half a Q tile, half a dO tile and the queries' M2 / delta, then a KV block's query blocks
+    const size_t lds = (size_t)kBwdStages * kBwdStage + (size_t)nbq * sizeof(int32_t);
+    if (lds > 160 * 1024) return hipErrorInvalidValue;
+    if (dtype == BSA_BF16) e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_dkdv_kernel<__bf16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    else e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_dkdv_kernel<_Float16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
     const dim3 grid_k((unsigned)(bh * (Sk / kTile)));
     // dQ: rounds of as many wavefronts as the device runs at once (one per SIMD), two rounds per launch.  The dK / dV
-    // kernels run as one grid each, longest list first: their lists (the query blocks of a KV block) differ in
-    // length, and rounds that wait for the longest list cost more than they bring (measured at the 720p geometry:
-    // one grid in tile order 60.6 ms for the whole backward, rounds 62-75 ms, one grid longest first 54.1 ms).
+    // kernel runs as one grid, longest list first: its lists (the query blocks of a KV block) differ in length, and
+    // rounds that wait for the longest list cost more than they bring.
     int cus = 256, dev = 0;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     const int round = 4 * (cus > 0 ? cus : 256), span = 2 * round;
@@ -566,10 +584,9 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
             hipLaunchKernelGGL((bwd_dq_kernel<__bf16>), dim3(end - first), block, 0, st, (const __bf16*)q, (const __bf16*)dout, ks_row,
                                ks_tr, v_row, m2, delta, paced, lens, tile_valid, (__bf16*)dq, Sq, Sk, bs_q, bs_k, idx_stride, first, end, round);
         }
-        hipLaunchKernelGGL((bwd_dkv_kernel<__bf16, false>), grid_k, block, lds, st, (const __bf16*)ks, (const __bf16*)v, q_row, q_tr,
-                           do_row, do_tr, m2, delta, bits, tile_valid, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words, 1.0f, order, 0, total_k, round);
-        hipLaunchKernelGGL((bwd_dkv_kernel<__bf16, true>), grid_k, block, lds, st, (const __bf16*)ks, (const __bf16*)v, q_row, q_tr,
-                           do_row, do_tr, m2, delta, bits, tile_valid, (__bf16*)dk, Sq, Sk, bs_q, bs_k, words, sm_scale, order, 0, total_k, round);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<__bf16>), grid_k, dim3(128), lds, st, (const __bf16*)q, (const __bf16*)dout, (const __bf16*)ks,
+                           (const __bf16*)v, m2, delta, bits, tile_valid, (__bf16*)dk, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words, sm_scale, order,
+                           total_k, round);
     } else {
         for (int first = 0; first < total_q; first += span) {
             const int end = first + span < total_q ? first + span : total_q;
@@ -577,10 +594,9 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
                                ks_row, ks_tr, v_row, m2, delta, paced, lens, tile_valid, (_Float16*)dq, Sq, Sk, bs_q, bs_k, idx_stride, first,
                                end, round);
         }
-        hipLaunchKernelGGL((bwd_dkv_kernel<_Float16, false>), grid_k, block, lds, st, (const _Float16*)ks, (const _Float16*)v, q_row,
-                           q_tr, do_row, do_tr, m2, delta, bits, tile_valid, (_Float16*)dv, Sq, Sk, bs_q, bs_k, words, 1.0f, order, 0, total_k, round);
-        hipLaunchKernelGGL((bwd_dkv_kernel<_Float16, true>), grid_k, block, lds, st, (const _Float16*)ks, (const _Float16*)v, q_row,
-                           q_tr, do_row, do_tr, m2, delta, bits, tile_valid, (_Float16*)dk, Sq, Sk, bs_q, bs_k, words, sm_scale, order, 0, total_k, round);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<_Float16>), grid_k, dim3(128), lds, st, (const _Float16*)q, (const _Float16*)dout,
+                           (const _Float16*)ks, (const _Float16*)v, m2, delta, bits, tile_valid, (_Float16*)dk, (_Float16*)dv, Sq, Sk, bs_q, bs_k,
+                           words, sm_scale, order, total_k, round);
     }
     return hipGetLastError();
 }

@@ -51,5 +51,36 @@ __device__ inline uint32_t lds_address(const void* p) {
 __device__ inline s16x4 lds_read_tr16(const void* p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
 }
+
+// S^T accumulators must sit in ordinary VGPRs, where the softmax reads them, while the (four times larger)
+// output accumulators belong in AGPRs.  For a kernel that may use more than 256 registers the compiler puts
+// the result of every builtin MFMA into AGPRs, so the S^T MFMAs are written as inline assembly with VGPR
+// operands.  The compiler does not see that such a statement is an MFMA and adds no wait states behind it:
+// the code keeps every VALU access to these accumulators at least eight MFMAs (256 clocks) behind the MFMA
+// that writes them, or puts explicit s_nop there.
+// kAgprB: the B operand (the Q fragment) lives in an AGPR.  The queries 32 .. 63 of a work item are kept there,
+// the queries 0 .. 31 in VGPRs, which balances the two register files (VGPR: S^T, P^T, the K ring, half of Q;
+// AGPR: the output accumulators, the V ring, the other half of Q).
+template <bool kFirst, bool kAgprB>
+__device__ inline void mfma_s(f32x16& acc, bf16x8 a, bf16x8 b) {
+    if (kFirst) {
+        if (kAgprB) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));
+        else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
+    } else {
+        if (kAgprB) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));
+        else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+    }
+}
+template <bool kFirst, bool kAgprB>
+__device__ inline void mfma_s(f32x16& acc, f16x8 a, f16x8 b) {
+    if (kFirst) {
+        if (kAgprB) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(b));
+        else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "v"(b));
+    } else {
+        if (kAgprB) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(b));
+        else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+    }
+}
+
 }  // namespace mfma
 }  // namespace bsa
