@@ -406,30 +406,44 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
         const s16x4 lo = lds_read_tr16(base + toff[t][0]), hi = lds_read_tr16(base + toff[t][1]);
         return __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
     };
-    // one half tile of queries (32) against this wavefront's 32 keys: 32 MFMAs
-    auto compute = [&](const char* stage) {
-        const char* qt = stage;
-        const char* dt = stage + kBwdHalfTile;
-        const float* st_m2 = reinterpret_cast<const float*>(stage + 2 * kBwdHalfTile);
+    // One half tile of queries (32) against this wavefront's 32 keys is 32 MFMAs in two groups with the exponentials
+    // between them.  A wavefront has a SIMD to itself, so it overlaps them on its own: the S and dP products of the
+    // NEXT half (into a second pair of accumulators) are issued between the exponentials of this one.  S and dP
+    // accumulate in ordinary registers, where the exponentials read them: MFMAs from inline assembly, behind which
+    // the compiler adds no wait states - a pair is read a whole group of 16 MFMAs after it was written.
+    auto products_and_exponentials = [&](int hp, f32x16& s, f32x16& dp, f32x16& s_next, f32x16& dp_next) {
+        const char* qn = bwd_lds + ((hp + 1) & 3) * kBwdStage;
+        const char* dn = qn + kBwdHalfTile;
+        const float* st_m2 = reinterpret_cast<const float*>(bwd_lds + (hp & 3) * kBwdStage + 2 * kBwdHalfTile);
         const float* st_dl = st_m2 + 32;
-        // S and dP accumulate in ordinary registers (the exponentials read them there): MFMAs from inline assembly,
-        // behind which the compiler adds no wait states, so the wait for the last one is written out
-        f32x16 s, dp;
-        mfma_s<true, false>(s, *reinterpret_cast<const V8*>(qt + roff[0]), kreg[0]);
-        mfma_s<true, false>(dp, *reinterpret_cast<const V8*>(dt + roff[0]), vreg[0]);
-#pragma unroll
-        for (int c = 1; c < 8; ++c) {
-            mfma_s<false, false>(s, *reinterpret_cast<const V8*>(qt + roff[c]), kreg[c]);
-            mfma_s<false, false>(dp, *reinterpret_cast<const V8*>(dt + roff[c]), vreg[c]);
-        }
-        asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-        // accumulator i <-> query 8 (i / 4) + 4 lh + i % 4 of the half, key lr
+        // Volatile assembly keeps the compiler from moving LDS reads across it, so the operands of a group of four
+        // MFMAs (and the statistics of four accumulators) are requested a group ahead by hand.
+        V8 fq[2][2], fd[2][2];
+        float4 mm[2], dd[2];
+        auto request = [&](int g, int b) {
+            fq[b][0] = *reinterpret_cast<const V8*>(qn + roff[2 * g]);
+            fd[b][0] = *reinterpret_cast<const V8*>(dn + roff[2 * g]);
+            fq[b][1] = *reinterpret_cast<const V8*>(qn + roff[2 * g + 1]);
+            fd[b][1] = *reinterpret_cast<const V8*>(dn + roff[2 * g + 1]);
+            mm[b] = *reinterpret_cast<const float4*>(st_m2 + 8 * g + 4 * lh);
+            dd[b] = *reinterpret_cast<const float4*>(st_dl + 8 * g + 4 * lh);
+        };
+        request(0, 0);
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
-            const float4 mm = *reinterpret_cast<const float4*>(st_m2 + 8 * g4 + 4 * lh);
-            const float4 dd = *reinterpret_cast<const float4*>(st_dl + 8 * g4 + 4 * lh);
-            const float mv[4] = {mm.x, mm.y, mm.z, mm.w}, dl[4] = {dd.x, dd.y, dd.z, dd.w};
+            const int c = 2 * g4, b = g4 & 1;
+            if (g4 < 3) request(g4 + 1, b ^ 1);
+            if (g4 == 0) {
+                mfma_s<true, false>(s_next, fq[b][0], kreg[0]);
+                mfma_s<true, false>(dp_next, fd[b][0], vreg[0]);
+            } else {
+                mfma_s<false, false>(s_next, fq[b][0], kreg[c]);
+                mfma_s<false, false>(dp_next, fd[b][0], vreg[c]);
+            }
+            mfma_s<false, false>(s_next, fq[b][1], kreg[c + 1]);
+            mfma_s<false, false>(dp_next, fd[b][1], vreg[c + 1]);
+            // accumulator i <-> query 8 (i / 4) + 4 lh + i % 4 of the half, key lr
+            const float mv[4] = {mm[b].x, mm[b].y, mm[b].z, mm[b].w}, dl[4] = {dd[b].x, dd[b].y, dd[b].z, dd[b].w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int i = 4 * g4 + j;
@@ -439,10 +453,13 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
                 dp[i] = pi * (dp[i] - dl[j]);                // dS
             }
         }
-        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto gradients = [&](int hp, const f32x16& p, const f32x16& ds) {
+        const char* qt = bwd_lds + (hp & 3) * kBwdStage;
+        const char* dt = qt + kBwdHalfTile;
 #pragma unroll
         for (int st2 = 0; st2 < 2; ++st2) {
-            const V8 bp = pack8<T, V8>(s, st2), bds = pack8<T, V8>(dp, st2);
+            const V8 bp = pack8<T, V8>(p, st2), bds = pack8<T, V8>(ds, st2);
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 acc_dv[t] = mfma32(frag_tr_lds(dt, st2, t), bp, acc_dv[t]);
@@ -450,12 +467,17 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
             }
         }
     };
-    // At the end of half hp the loads of half hp + 1 must have landed; the two halves requested after it may still
-    // be on their way (wavefront 0 issues 9 loads per half, wavefront 1 issues 8).
-    auto await_next = [&](int hp) {
+    // During half hp the rows of half hp + 1 are read, so at its end the loads of half hp + 2 must have landed; the
+    // half requested after it may still be on its way (wavefront 0 issues 9 loads per half, wavefront 1 issues 8).
+    auto step = [&](int hp, f32x16& s, f32x16& dp, f32x16& s_next, f32x16& dp_next) {
+        // half hp + 3 takes the stage that half hp - 1 was read from: both wavefronts are past the barrier behind it
+        issue(hp + 3, (hp + 3) & 3);
+        products_and_exponentials(hp, s, dp, s_next, dp_next);
+        __builtin_amdgcn_sched_barrier(0);
+        gradients(hp, s, dp);
         if (hp + 3 < nhalves) {
-            if (wave == 0) asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)" ::: "memory");
-            else asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+            if (wave == 0) asm volatile("s_waitcnt vmcnt(9) lgkmcnt(0)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
         } else {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         }
@@ -466,17 +488,28 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
         issue(1, 1);
         issue(2, 2);
         if (nhalves > 2) {
-            if (wave == 0) asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
-            else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+            if (wave == 0) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         } else {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         __builtin_amdgcn_s_barrier();
-        for (int hp = 0; hp < nhalves; ++hp) {
-            // half hp + 3 takes the stage that half hp - 1 was read from: both wavefronts are past the barrier behind it
-            issue(hp + 3, (hp + 3) & 3);
-            compute(bwd_lds + (hp & 3) * kBwdStage);
-            await_next(hp);
+        f32x16 s0, dp0, s1, dp1;
+        {
+            const char* qn = bwd_lds;
+            const char* dn = qn + kBwdHalfTile;
+            mfma_s<true, false>(s0, *reinterpret_cast<const V8*>(qn + roff[0]), kreg[0]);
+            mfma_s<true, false>(dp0, *reinterpret_cast<const V8*>(dn + roff[0]), vreg[0]);
+#pragma unroll
+            for (int c = 1; c < 8; ++c) {
+                mfma_s<false, false>(s0, *reinterpret_cast<const V8*>(qn + roff[c]), kreg[c]);
+                mfma_s<false, false>(dp0, *reinterpret_cast<const V8*>(dn + roff[c]), vreg[c]);
+            }
+            asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+        }
+        for (int hp = 0; hp < nhalves; hp += 2) {                                // halves come in pairs
+            step(hp, s0, dp0, s1, dp1);
+            step(hp + 1, s1, dp1, s0, dp0);
         }
     }
     // accumulator i of d tile t <-> d = 32 t + 8 (i / 4) + 4 lh + i % 4, key lr
