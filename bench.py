@@ -48,18 +48,21 @@ def source_sha16(paths=ATTENTION_SOURCES):
     return h.hexdigest()[:16]
 
 
-def recorded_traffic(workload):
-    """HBM-side bytes per layer of the attention kernel (rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled as the profile
-    summary says), as recorded in profiles/bsa_operator_<workload>_*.md on a line
+BACKWARD_SOURCES = [os.path.join(ROOT, "longcat-video_amd", "csrc", "bsa_bwd.hip")]
+
+
+def recorded_traffic(workload, summaries="bsa_operator_%s_*.md", sources=ATTENTION_SOURCES):
+    """HBM-side bytes per layer of the workload's dominant kernels (rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled as the
+    profile summary says), as recorded in a summary under profiles/ on a line
     `traffic_record: {"workload": ..., "source_sha16": ..., "bytes_per_layer": ...}` - or None when there is no
     record for this workload or the kernel source has changed since it was taken (a stale figure is not reported)."""
     import glob
-    for path in glob.glob(os.path.join(ROOT, "profiles", "bsa_operator_%s_*.md" % workload)):
+    for path in glob.glob(os.path.join(ROOT, "profiles", summaries % workload if "%s" in summaries else summaries)):
         with open(path) as f:
             for line in f:
                 if line.startswith("traffic_record:"):
                     rec = json.loads(line[len("traffic_record:"):])
-                    if rec.get("workload") == workload and rec.get("source_sha16") == source_sha16():
+                    if rec.get("workload") == workload and rec.get("source_sha16") == source_sha16(sources):
                         return float(rec["bytes_per_layer"])
     return None
 
@@ -297,7 +300,8 @@ def run_bwd(torch, args):
                    "block_pairs": pairs},
         "roofline": {"kernel": "bwd_dq_kernel<bf16> + bwd_dkdv_kernel<bf16> (with the passes before them)", "bound": "mfma",
                      "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": None, "ms": round(ms, 4)}}
+                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4),
+                     "traffic": recorded_traffic("bwd", "bsa_backward_*.md", BACKWARD_SOURCES), "ms": round(ms, 4)}}
     if not args.no_cpu_baseline:
         from oracle import bsa_oracle as O
         cores = os.cpu_count() or 1

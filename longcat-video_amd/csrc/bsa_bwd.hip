@@ -272,7 +272,7 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
 // One workgroup of two wavefronts per 64 keys; wavefront w owns keys 32 w .. 32 w + 31 and both of their gradients
 // (128 accumulator registers).  The Q and dO tiles of a query tile (64 rows x 256 B each, as they lie in memory)
 // go from global memory straight into LDS once per workgroup (global_load_lds_dwordx4; wavefront 0 brings Q and
-// the queries' M2 and delta, wavefront 1 brings dO), in halves of 32 queries, four stages deep (one in use, three on
+// the queries' M2 and delta, wavefront 1 brings dO), in halves of 32 queries, four stages deep (two in use, two on
 // their way), and both wavefronts take every operand from there: the row fragments (the A operands of S = Q K_s^T and
 // dP = dO V^T) with ds_read_b128, the transposed
 // ones (the A operands of dV^T += dO^T P and dK^T += Q^T dS) with ds_read_b64_tr_b16.  Per tile pair 32 KB leave
@@ -285,7 +285,7 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
 constexpr int kBwdHalfTile = kTileBytes / 2;                 // 32 query rows of Q or of dO
 constexpr int kBwdStats = 1024;                              // M2 (128 B), delta (128 B), the rest filled blindly by the 64-lane DMA
 constexpr int kBwdStage = 2 * kBwdHalfTile + kBwdStats;      // one half tile of queries: Q rows, dO rows, M2, delta
-constexpr int kBwdStages = 4;                                // one in use, three on their way: a tile and a half ahead
+constexpr int kBwdStages = 4;                                // two in use (this half, the next half's rows), two on their way
 
 template <typename T>
 __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, const T* __restrict__ dout,
