@@ -153,26 +153,18 @@ constexpr int kMaxSel = 4096;   // longest list: the score-order ranking keeps a
 __device__ inline uint32_t ord_of(uint16_t s) { return ord16(s); }
 __device__ inline uint32_t ord_of(uint32_t s) { return ord32(s); }
 
-// Selection of one score row by one wavefront; lane l holds the order-preserving images of columns l, l + 64,
-// ... in registers (0 for columns past the end of the row).
-//   1. the k-th largest score value t: for 16-bit scores from a histogram of the codes just below the row
-//      maximum, otherwise (and for rows whose winners reach further down) by a bitwise binary search whose
-//      counting step is a ballot + popcount;
-//   2. every score above t wins, and of the scores equal to t the ones with the lowest column
-//      index, as many as are still needed; walking the registers in column order hands out the
-//      positions of the ascending-block-order list at the same time (no sort);
-//   3. only when the score-order list is wanted: rank the winners by (score desc, index asc).
-// raw_at(i): the stored score of column i.  mine: one key of LDS per list entry (SCORE_ORDER only); h: 256 words of LDS.
-template <typename S, int NPL, bool SCORE_ORDER, typename RawAt>
-__device__ inline void select_row(const uint32_t (&val)[NPL], RawAt raw_at, int lane, int nbk, int k_sel,
-                                  int32_t* __restrict__ idx_row, int32_t* __restrict__ idx_sorted_row,
-                                  typename KeyOf<S>::type* mine, uint32_t* h) {
-    typedef typename KeyOf<S>::type K;
-    constexpr int kValueBits = 8 * (int)sizeof(S);
-    // The k-th largest score value t: every column above it wins, and of the columns equal to it the first
-    // need_eq in column order.
-    uint32_t thr = 0;
-    int cnt_gt = 0;
+// The k-th largest score value t of a row that a wavefront holds as val[N] per lane (order-preserving images;
+// in_range(x): element x of this lane is a column of the row): every column above t wins, and of the columns equal
+// to t the first k_sel - cnt_gt in column order.  thr = t, cnt_gt = columns above t, cnt_eq = columns equal to t.
+// For 16-bit scores t is first looked for in a histogram of the codes just below the row maximum, otherwise (and for
+// rows whose winners reach further down) by a bitwise binary search whose counting step is a ballot + popcount.
+// h: 256 words of LDS of this wavefront.
+template <int kValueBits, int N, typename InRange>
+__device__ inline void kth_value(const uint32_t (&val)[N], InRange in_range, int lane, int k_sel, uint32_t* h,
+                                 uint32_t& thr, int& cnt_gt, int& cnt_eq) {
+    thr = 0;
+    cnt_gt = 0;
+    cnt_eq = 0;
     bool found = false;
     if (kValueBits == 16) {
         // 16-bit scores: the winners of a row usually lie within a few hundred codes of the row maximum, so one
@@ -180,16 +172,16 @@ __device__ inline void select_row(const uint32_t (&val)[NPL], RawAt raw_at, int 
         // and one scan find t.  Rows whose k_sel largest values reach further down take the search below.
         uint32_t mx = 0;
 #pragma unroll
-        for (int j = 0; j < NPL; ++j) mx = max(mx, val[j]);
+        for (int j = 0; j < N; ++j) mx = max(mx, val[j]);
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, o));
         *reinterpret_cast<uint4*>(h + 4 * lane) = make_uint4(0u, 0u, 0u, 0u);
         __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int j = 0; j < NPL; ++j) {
+        for (int j = 0; j < N; ++j) {
             const uint32_t d = mx - val[j];
-            if (j * 64 + lane < nbk && d < 255u) atomicAdd(h + d, 1u);
+            if (in_range(j) && d < 255u) atomicAdd(h + d, 1u);
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);
         __builtin_amdgcn_wave_barrier();
@@ -204,13 +196,14 @@ __device__ inline void select_row(const uint32_t (&val)[NPL], RawAt raw_at, int 
         const int before = upto - own;
         const uint64_t holder = __ballot(before < k_sel && k_sel <= upto);
         if (holder != 0) {
-            int bin = 4 * lane, run = before;
-            if (run + (int)c.x < k_sel) { run += (int)c.x; ++bin;
-                if (run + (int)c.y < k_sel) { run += (int)c.y; ++bin;
-                    if (run + (int)c.z < k_sel) { run += (int)c.z; ++bin; } } }
+            int bin = 4 * lane, run = before, in_bin = (int)c.x;
+            if (run + (int)c.x < k_sel) { run += (int)c.x; ++bin; in_bin = (int)c.y;
+                if (run + (int)c.y < k_sel) { run += (int)c.y; ++bin; in_bin = (int)c.z;
+                    if (run + (int)c.z < k_sel) { run += (int)c.z; ++bin; in_bin = (int)c.w; } } }
             const int src = __builtin_ctzll(holder);
             thr = mx - (uint32_t)__shfl(bin, src);
             cnt_gt = __shfl(run, src);
+            cnt_eq = __shfl(in_bin, src);
             found = true;
         }
     }
@@ -223,16 +216,38 @@ __device__ inline void select_row(const uint32_t (&val)[NPL], RawAt raw_at, int 
             const uint32_t cand = thr | (1u << bit);
             int cnt = 0;
 #pragma unroll
-            for (int j = 0; j < NPL; ++j) cnt += __popcll(__ballot(val[j] >= cand));
+            for (int j = 0; j < N; ++j) cnt += __popcll(__ballot(val[j] >= cand));
             if (cnt >= k_sel) {
                 thr = cand;
                 if (cnt == k_sel) break;
             }
         }
         cnt_gt = 0;
+        cnt_eq = 0;
 #pragma unroll
-        for (int j = 0; j < NPL; ++j) cnt_gt += __popcll(__ballot(val[j] > thr));
+        for (int j = 0; j < N; ++j) {
+            cnt_gt += __popcll(__ballot(val[j] > thr));
+            cnt_eq += __popcll(__ballot(val[j] == thr && in_range(j)));      // thr may be 0, like the padding of val
+        }
     }
+}
+
+// Selection of one score row by one wavefront; lane l holds the order-preserving images of columns l, l + 64,
+// ... in registers (0 for columns past the end of the row).
+//   1. the k-th largest score value t (kth_value);
+//   2. every score above t wins, and of the scores equal to t the ones with the lowest column
+//      index, as many as are still needed; walking the registers in column order hands out the
+//      positions of the ascending-block-order list at the same time (no sort);
+//   3. only when the score-order list is wanted: rank the winners by (score desc, index asc).
+// raw_at(i): the stored score of column i.  mine: one key of LDS per list entry (SCORE_ORDER only); h: 256 words of LDS.
+template <typename S, int NPL, bool SCORE_ORDER, typename RawAt>
+__device__ inline void select_row(const uint32_t (&val)[NPL], RawAt raw_at, int lane, int nbk, int k_sel,
+                                  int32_t* __restrict__ idx_row, int32_t* __restrict__ idx_sorted_row,
+                                  typename KeyOf<S>::type* mine, uint32_t* h) {
+    typedef typename KeyOf<S>::type K;
+    uint32_t thr;
+    int cnt_gt, cnt_eq;
+    kth_value<8 * (int)sizeof(S)>(val, [&](int j) { return j * 64 + lane < nbk; }, lane, k_sel, h, thr, cnt_gt, cnt_eq);
     const int need_eq = k_sel - cnt_gt;
 
     int pos = 0, eq_seen = 0;
@@ -300,6 +315,96 @@ __global__ __launch_bounds__(256) void topk_kernel(const S* __restrict__ score,
                                     idx_out ? idx_out + row * stride : nullptr,
                                     idx_sorted_out ? idx_sorted_out + row * stride : nullptr,
                                     reinterpret_cast<K*>(topk_keys) + (SCORE_ORDER ? (size_t)wave * stride : 0), hist[wave]);
+}
+
+// Top-k of 16-bit scores when only the ascending-block-order list is wanted and rows are 16-byte aligned (nbk a
+// multiple of 8): the same selection as select_row with another assignment of columns to lanes.  Lane l holds the
+// columns 512 j + 8 l .. 8 l + 7 (one 16-byte load per j instead of eight 2-byte loads), so the ascending list
+// position of a winner is (winners in earlier j) + (winners in lower lanes: one prefix sum per j) + (winners
+// below it in its own lane) - one scan per 512 columns instead of two ballots per 64.
+template <int NCH>
+__global__ __launch_bounds__(256) void topk_blocked_kernel(const uint16_t* __restrict__ score,
+                                                           int32_t* __restrict__ idx_sorted_out,
+                                                           int32_t* __restrict__ lens_out, int64_t rows, int nbk, int k_all,
+                                                           const int32_t* __restrict__ k_rows, int stride) {
+    __shared__ __attribute__((aligned(16))) uint32_t hist[4][256];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    if (row >= rows) return;
+    const int k_sel = k_rows != nullptr ? k_rows[row] : k_all;
+    if (lane == 0) lens_out[row] = k_sel;
+    int32_t* out = idx_sorted_out + row * stride;
+    for (int e = k_sel + lane; e < stride; e += 64) out[e] = -1;          // unused tail of the row's list
+    if (k_sel == 0) return;
+
+    const uint16_t* srow = score + row * nbk;
+    uint32_t val[NCH * 8];                   // ord(score); 0 for columns past the end of the row
+    bool in[NCH];
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        const int col0 = 512 * j + 8 * lane;
+        in[j] = col0 < nbk;
+        const uint4 raw = *reinterpret_cast<const uint4*>(srow + (in[j] ? col0 : 0));   // unconditional load, masked afterwards
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint16_t r = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+            val[8 * j + e] = in[j] ? ord16(r) : 0u;
+        }
+    }
+    uint32_t thr;
+    int cnt_gt, cnt_eq;
+    kth_value<16>(val, [&](int x) { return in[x >> 3]; }, lane, k_sel, hist[wave], thr, cnt_gt, cnt_eq);
+    const int need_eq = k_sel - cnt_gt;
+    const bool all_equal_win = need_eq >= cnt_eq;            // the same in every lane: no tie is cut
+
+    int pos = 0, eq_seen = 0;                                  // winners / columns equal to t in the chunks before j
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        if (512 * j >= nbk) break;
+        uint32_t win = 0;                                      // bit e: column 512 j + 8 lane + e wins
+        if (all_equal_win) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) win |= (val[8 * j + e] >= thr && in[j]) ? (1u << e) : 0u;
+        } else {
+            uint32_t gt = 0, eq = 0;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                gt |= (val[8 * j + e] > thr) ? (1u << e) : 0u;
+                eq |= (val[8 * j + e] == thr && in[j]) ? (1u << e) : 0u;
+            }
+            // of the columns equal to t the first need_eq in column order win
+            const int n_eq = __popc(eq);
+            int upto = n_eq;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int t = __shfl_up(upto, o);
+                if (lane >= o) upto += t;
+            }
+            int take = min(max(need_eq - (eq_seen + upto - n_eq), 0), n_eq);
+            eq_seen += __shfl(upto, 63);
+            win = gt;
+            while (take > 0) {
+                const uint32_t low = eq & (0u - eq);
+                win |= low;
+                eq ^= low;
+                --take;
+            }
+        }
+        const int n_win = __popc(win);
+        int upto = n_win;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int t = __shfl_up(upto, o);
+            if (lane >= o) upto += t;
+        }
+        int p = pos + upto - n_win;
+        pos += __shfl(upto, 63);
+        while (win != 0u) {
+            out[p++] = 512 * j + 8 * lane + __builtin_ctz(win);
+            win &= win - 1u;
+        }
+    }
 }
 
 // ---------------------------------------------------------------- visiting order
@@ -489,6 +594,18 @@ template <typename S>
 hipError_t launch_topk_t(const S* score, int32_t* idx, int32_t* idx_sorted, int32_t* lens, int64_t rows,
                          int nbk, int k_sel, const int32_t* k_rows, int stride, hipStream_t st) {
     dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+    if (sizeof(S) == 2 && idx == nullptr && idx_sorted != nullptr && nbk % 8 == 0 && (reinterpret_cast<uintptr_t>(score) & 15) == 0) {
+        const uint16_t* sc = reinterpret_cast<const uint16_t*>(score);
+#define BSA_TOPK_BLOCKED(N) hipLaunchKernelGGL((topk_blocked_kernel<N>), grid, block, 0, st, sc, idx_sorted, lens, rows, nbk, k_sel, k_rows, stride)
+        if (nbk <= 512) BSA_TOPK_BLOCKED(1);
+        else if (nbk <= 1024) BSA_TOPK_BLOCKED(2);
+        else if (nbk <= 1536) BSA_TOPK_BLOCKED(3);
+        else if (nbk <= 2048) BSA_TOPK_BLOCKED(4);
+        else if (nbk <= 3072) BSA_TOPK_BLOCKED(6);
+        else BSA_TOPK_BLOCKED(8);
+#undef BSA_TOPK_BLOCKED
+        return hipGetLastError();
+    }
     // the score-order ranking keeps the winners of the workgroup's four rows in LDS
     const size_t lds = idx != nullptr ? (size_t)4 * stride * sizeof(typename KeyOf<S>::type) : 0;
 #define BSA_TOPK(N)                                                                                \

@@ -64,6 +64,36 @@ def test_topk_bit_exact_with_ties(nbq, nbk, k_sel):
     assert torch.equal(got, want)
 
 
+def topk_block_order_only_gpu(score, k_sel):
+    """The C-ABI top-k asked for the ascending-block-order list alone (what the operator asks for): for 16-bit scores
+    with a multiple of 8 columns this takes the kernel that holds 8 consecutive columns per lane."""
+    from longcat_video_amd import _capi
+    B, H, nbq, nbk = score.shape
+    s = score.cuda().contiguous()
+    srt = torch.full((B * H * nbq * max(k_sel, 1),), -7, dtype=torch.int32, device="cuda")
+    lens = torch.empty(B, H, nbq, dtype=torch.int32, device="cuda")
+    code = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}[score.dtype]
+    _capi.check(_capi.load().bsa_topk_from_score(s.data_ptr(), None, srt.data_ptr(), lens.data_ptr(), B, H, nbq, nbk, k_sel, code,
+                                                  torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    return srt[: B * H * nbq * k_sel].view(B, H, nbq, k_sel).cpu().long(), lens.cpu()
+
+
+@pytest.mark.parametrize("nbq,nbk,k_sel", [(4, 8, 2), (5, 40, 9), (3, 64, 64), (7, 200, 0), (3, 624, 39), (2, 520, 17), (2, 512, 511),
+                                             (2, 1440, 90), (2, 1248, 156), (1, 2048, 300), (3, 2056, 1500), (1, 4096, 1024),
+                                             (5, 4096, 3000), (2, 3080, 77), (3, 37, 9), (2, 585, 36)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_topk_block_order_list_alone(nbq, nbk, k_sel, dtype):
+    g = torch.Generator().manual_seed(nbk + k_sel)
+    # few distinct values => ties that the selection has to cut at the lowest indices; then plain random scores
+    for score in ((torch.randint(-6, 7, (1, 2, nbq, nbk), generator=g).float() / 4).to(dtype),
+                  torch.randn(1, 2, nbq, nbk, generator=g).to(dtype)):
+        got, lens = topk_block_order_only_gpu(score, k_sel)
+        want, want_lens = O.select_topk(score, k_sel)
+        assert torch.equal(lens, want_lens)
+        assert torch.equal(got, torch.sort(want, dim=-1).values)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_topk_random_scores_all_dtypes(dtype):
     g = torch.Generator().manual_seed(7)
