@@ -440,8 +440,9 @@ __global__ __launch_bounds__(64) void pace_order_kernel(const int32_t* in, int32
         return;
     }
     const int groups = (n + kPaceWidth - 1) / kPaceWidth;
-    const int64_t span = (int64_t)nbk * kPaceWidth;
-    auto group_of = [&](int32_t b) { return (int)min((int64_t)b * n / span, (int64_t)groups - 1); };
+    // n <= stride < 2^13 (the LDS that launch_pace_order asks for bounds it) and b < nbk: 32-bit products and quotients
+    const uint32_t span = (uint32_t)nbk * kPaceWidth;
+    auto group_of = [&](int32_t b) { return (int)min((uint32_t)b * (uint32_t)n / span, (uint32_t)groups - 1u); };
     for (int e = lane; e < n; e += 64) {
         lst[e] = min(max(src[e], 0), nbk - 1);
         slots[e] = -1;
