@@ -62,7 +62,8 @@ def words_of(valid):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("bs_q,bs_k,nbq,nbk,width", [(64, 64, 9, 14, 5), (128, 64, 4, 11, 4), (64, 128, 6, 5, 3), (128, 128, 3, 4, 2)])
+@pytest.mark.parametrize("bs_q,bs_k,nbq,nbk,width", [(64, 64, 9, 14, 5), (128, 64, 4, 11, 4), (64, 128, 6, 5, 3), (128, 128, 3, 4, 2),
+                                                       (256, 64, 3, 9, 4), (64, 256, 7, 3, 2), (64, 64, 40, 6, 3), (64, 64, 1, 5, 5)])
 def test_against_the_restated_reference_backward(dtype, bs_q, bs_k, nbq, nbk, width):
     sm = 1 / math.sqrt(128)
     q, k, v, do, idx, lens = make_case(nbq * 100 + nbk, 2, nbq, nbk, width, dtype, bs_q, bs_k)
