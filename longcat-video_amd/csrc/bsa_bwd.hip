@@ -8,11 +8,10 @@
 //   ds = p * (dp - delta) rounded to the storage type, p rounded to the storage type for dV;
 //   dV = sum p^T do,  dK = sm_scale * sum ds^T q,  dQ = ln 2 * sum ds k_s  (fp32 accumulators, one final rounding).
 //
-// Data movement of dQ as in bsa_fwd_frag.hip: every operand that an MFMA reads from memory is first rewritten into
-// fragment order (frag_kernel), so a wavefront loads it with one coalesced 16-byte load per lane and fragment and
-// LDS carries nothing.  "row layout" = the K layout of that file (A operand whose rows are tokens), "transposed
-// layout" = its V layout (A operand whose rows are head-dim columns, contraction over 16 tokens in accumulator
-// order).  Needed: k_s in both layouts and v in row layout.
+// Data movement of dQ as in bsa_fwd_frag.hip: k_s and v are first rewritten into fragment order (frag_kernel, "row
+// layout" = the K layout of that file: A operand whose rows are tokens), so a wavefront loads a fragment with one
+// coalesced 16-byte load per lane.  The transposed K_s fragments (A operand whose rows are head-dim columns,
+// contraction over 16 tokens in accumulator order) are made in the kernel from the row fragments, through LDS.
 //
 // dQ: one wavefront per 64 query rows (two halves of 32, so that every K_s and V fragment feeds two MFMAs).
 // S^T = K_s Q^T and dP^T = V dO^T (Q and dO rows in registers as B operands) put one query per lane, so M2 and
@@ -125,9 +124,11 @@ __device__ __forceinline__ V8 pack8(const f32x16& x, int s) {
 }
 
 // ------------------------------------------------------------------ dQ
+constexpr int kDqLds = 32 * 256;                             // the K_s rows of a half tile, on their way to being transposed
+
 template <typename T>
 __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, const T* __restrict__ dout,
-                                                    const char* __restrict__ ks_row, const char* __restrict__ ks_tr,
+                                                    const char* __restrict__ ks_row,
                                                     const char* __restrict__ v_row, const float* __restrict__ m2,
                                                     const float* __restrict__ delta, const int32_t* __restrict__ idx,
                                                     const int32_t* __restrict__ lens,
@@ -155,7 +156,6 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
     const int32_t* list = idx + lrow * stride;
     const int64_t kv_tiles = Sk / kTile;
     const char* ksr = ks_row + bh * kv_tiles * kTileBytes;
-    const char* kst = ks_tr + bh * kv_tiles * kTileBytes;
     const char* vr = v_row + bh * kv_tiles * kTileBytes;
 
     // two query halves of 32 rows: every K_s / V fragment feeds two MFMAs
@@ -189,19 +189,44 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
 #pragma unroll
         for (int c = 0; c < 8; ++c) f.v[c] = frag_row<V8>(vr, tile, h, c, lane_off);
     };
-    // The transposed K_s fragments of a half are requested right behind the last MFMA that reads those of the half
-    // before (into the same registers), a whole half ahead of their use.
+    // The transposed K_s fragments of a half (the A operands of dQ^T += K_s^T dS^T) are made from its row fragments:
+    // every lane parks its 16-byte pieces in the wavefront's 8 KB of LDS and ds_read_b64_tr_b16 hands them back with
+    // rows and columns exchanged, which saves a third of the bytes that the wavefront pulls through the L1 path and a
+    // fragment-order copy of k_s.  Piece u of key row r lies in slot u ^ f(r), f(r) = ((r << 1) & 14) | ((r >> 3) & 1):
+    // neither the writes (16 consecutive rows) nor the 4-row patches of a transposing read collide on a bank.
+    extern __shared__ __attribute__((aligned(16))) char dq_lds[];
     V8 kt[8];
-    auto load_kt = [&](int64_t tile, int h) {
+    const uint32_t fl = (uint32_t)(((lr << 1) & 14) | ((lr >> 3) & 1));
+    uint32_t woff[8];
 #pragma unroll
-        for (int x = 0; x < 8; ++x) kt[x] = frag_tr<V8>(kst, tile, h, x >> 2, x & 3, lane_off);
+    for (int c = 0; c < 8; ++c) woff[c] = (uint32_t)(lr * 256) + ((((uint32_t)(2 * c + lh)) ^ fl) << 4);
+    const int s16 = lane & 15, g1 = (lane >> 4) & 1, tx = s16 >> 2, ty = (s16 & 3) >> 1, tz = s16 & 1;
+    uint32_t toff[4][2];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi)
+            toff[t][hi] = (uint32_t)((4 * lh + tx + 8 * hi) * 256) + ((((uint32_t)(4 * t + 2 * g1 + ty)) ^ (uint32_t)((8 * lh + 2 * tx) | hi)) << 4) +
+                          (uint32_t)(tz * 8);
+    auto park_rows = [&](const V8 (&krow)[8]) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) *reinterpret_cast<V8*>(dq_lds + woff[c]) = krow[c];
     };
-    auto compute = [&](const Frags& f, uint32_t hv, int64_t next_tile, int next_h) {
+    auto take_transposed = [&]() {
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            const char* base = dq_lds + (16 * (x >> 2)) * 256;
+            const s16x4 lo = lds_read_tr16(base + toff[x & 3][0]), hi = lds_read_tr16(base + toff[x & 3][1]);
+            kt[x] = __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+    };
+    auto compute = [&](const Frags& f, uint32_t hv) {
         f32x16 s[2], dp[2];
 #pragma unroll
         for (int qq = 0; qq < 2; ++qq)
 #pragma unroll
             for (int i = 0; i < 16; ++i) { s[qq][i] = 0.f; dp[qq][i] = 0.f; }
+        park_rows(f.k);
 #pragma unroll
         for (int c = 0; c < 8; ++c)
 #pragma unroll
@@ -209,6 +234,7 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
                 s[qq] = mfma32(f.k[c], qreg[qq][c], s[qq]);
                 dp[qq] = mfma32(f.v[c], doreg[qq][c], dp[qq]);
             }
+        take_transposed();
         // accumulator i <-> key 8 (i / 4) + 4 lh + i % 4 of the half, query lr (+ 32)
 #pragma unroll
         for (int qq = 0; qq < 2; ++qq)
@@ -228,9 +254,6 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
                 acc[t][1] = mfma32(kt[4 * st + t], ds1, acc[t][1]);
             }
         }
-        __builtin_amdgcn_sched_barrier(0);               // the loads below overwrite what the MFMAs above read
-        load_kt(next_tile, next_h);
-        __builtin_amdgcn_sched_barrier(0);
     };
     const int ntiles = n * nsub;
     auto tile_at = [&](int tp) -> int64_t {
@@ -241,14 +264,13 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
         Frags fa, fb;
         int64_t tile = tile_at(0);
         load(fa, tile, 0);
-        load_kt(tile, 0);
         for (int tp = 0; tp < ntiles; ++tp) {
             const uint64_t valid = tile_valid != nullptr ? tile_valid[tile] : ~0ull;
             load(fb, tile, 1);
-            compute(fa, (uint32_t)valid, tile, 1);
+            compute(fa, (uint32_t)valid);
             const int64_t next = tile_at(tp + 1);
             load(fa, next, 0);                            // behind the last tile: loaded again, not used
-            compute(fb, (uint32_t)(valid >> 32), next, 0);
+            compute(fb, (uint32_t)(valid >> 32));
             tile = next;
         }
     }
@@ -533,14 +555,14 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
 
 }  // namespace
 
-// Workspace of the backward, in bytes: three fragment-order copies ([B*Hn][Sk/64][16 KB]: k_s in both layouts,
-// v in row layout), k_s in blocked order, delta and M2, the bit matrix, the lists in the dQ kernel's visiting
+// Workspace of the backward, in bytes: two fragment-order copies ([B*Hn][Sk/64][16 KB]: k_s and v in row layout),
+// k_s in blocked order, delta and M2, the bit matrix, the lists in the dQ kernel's visiting
 // order, per KV block its number of query blocks, the KV tiles of every head by that number.
 size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride) {
     const size_t bh = (size_t)B * Hn;
     auto up = [](size_t x) { return (x + 255) / 256 * 256; };
     const size_t words = (size_t)((Sq / bs_q + 31) / 32);
-    return 4 * up(bh * Sk * kD * 2) + 2 * up(bh * Sq * 4) + up(bh * (Sk / bs_k) * words * 4) +
+    return 3 * up(bh * Sk * kD * 2) + 2 * up(bh * Sq * 4) + up(bh * (Sk / bs_k) * words * 4) +
            up(bh * (Sq / bs_q) * (size_t)idx_stride * 4) + up(bh * (Sk / bs_k) * 4) + up(bh * (Sk / kTile) * 4);
 }
 
@@ -553,7 +575,6 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     char* ws = static_cast<char*>(workspace);
     auto take = [&](size_t n) { char* p = ws; ws += up(n); return p; };
     char* ks_row = take(bh * Sk * kD * 2);
-    char* ks_tr = take(bh * Sk * kD * 2);
     char* v_row = take(bh * Sk * kD * 2);
     char* ks = take(bh * Sk * kD * 2);
     float* delta = reinterpret_cast<float*>(take(bh * Sq * 4));
@@ -593,7 +614,6 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     // order); any other order is walked as given.  The order only moves fp32 roundings of the dQ sum.
     if ((e = launch_pace_order(idx, paced, lens, (int64_t)bh * nbq, nbk, idx_stride, st)) != hipSuccess) return e;
     if ((e = launch_frag(ks, stk, ks_row, B, Hn, gk, dtype, false, st)) != hipSuccess) return e;
-    if ((e = launch_frag(ks, stk, ks_tr, B, Hn, gk, dtype, true, st)) != hipSuccess) return e;
     if ((e = launch_frag(v, stk, v_row, B, Hn, gk, dtype, false, st)) != hipSuccess) return e;
 
     const dim3 block(64);
@@ -614,8 +634,8 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     if (dtype == BSA_BF16) {
         for (int first = 0; first < total_q; first += span) {
             const int end = first + span < total_q ? first + span : total_q;
-            hipLaunchKernelGGL((bwd_dq_kernel<__bf16>), dim3(end - first), block, 0, st, (const __bf16*)q, (const __bf16*)dout, ks_row,
-                               ks_tr, v_row, m2, delta, paced, lens, tile_valid, (__bf16*)dq, Sq, Sk, bs_q, bs_k, idx_stride, first, end, round);
+            hipLaunchKernelGGL((bwd_dq_kernel<__bf16>), dim3(end - first), block, kDqLds, st, (const __bf16*)q, (const __bf16*)dout, ks_row,
+                               v_row, m2, delta, paced, lens, tile_valid, (__bf16*)dq, Sq, Sk, bs_q, bs_k, idx_stride, first, end, round);
         }
         hipLaunchKernelGGL((bwd_dkdv_kernel<__bf16>), grid_k, dim3(128), lds, st, (const __bf16*)q, (const __bf16*)dout, (const __bf16*)ks,
                            (const __bf16*)v, m2, delta, bits, tile_valid, (__bf16*)dk, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words, sm_scale, order,
@@ -623,8 +643,8 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     } else {
         for (int first = 0; first < total_q; first += span) {
             const int end = first + span < total_q ? first + span : total_q;
-            hipLaunchKernelGGL((bwd_dq_kernel<_Float16>), dim3(end - first), block, 0, st, (const _Float16*)q, (const _Float16*)dout,
-                               ks_row, ks_tr, v_row, m2, delta, paced, lens, tile_valid, (_Float16*)dq, Sq, Sk, bs_q, bs_k, idx_stride, first,
+            hipLaunchKernelGGL((bwd_dq_kernel<_Float16>), dim3(end - first), block, kDqLds, st, (const _Float16*)q, (const _Float16*)dout,
+                               ks_row, v_row, m2, delta, paced, lens, tile_valid, (_Float16*)dq, Sq, Sk, bs_q, bs_k, idx_stride, first,
                                end, round);
         }
         hipLaunchKernelGGL((bwd_dkdv_kernel<_Float16>), grid_k, dim3(128), lds, st, (const _Float16*)q, (const _Float16*)dout,
