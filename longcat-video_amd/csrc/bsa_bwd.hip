@@ -234,6 +234,14 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
                 s[qq] = mfma32(f.k[c], qreg[qq][c], s[qq]);
                 dp[qq] = mfma32(f.v[c], doreg[qq][c], dp[qq]);
             }
+        // The 16 loads of the next half (requested by the caller just before this step) go out one behind every
+        // third MFMA of this step: a load that finds the CU's address unit busy holds up the wavefront's next
+        // instructions, and four wavefronts that each ask for 16 KB in one burst keep it busy for most of a step.
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
         take_transposed();
         // accumulator i <-> key 8 (i / 4) + 4 lh + i % 4 of the half, query lr (+ 32)
 #pragma unroll
