@@ -169,6 +169,17 @@ def test_topk_special_values():
             assert got.flatten().tolist() == want.flatten().tolist()
 
 
+def test_topk_special_values_block_order_list_alone():
+    inf = float("inf")
+    row = torch.tensor([0.0, -0.0, 1.0, -inf, inf, -0.0, 0.0, -1.0, inf, 3.0, 2.0, -2.0, 0.0, -0.0, 5.0, -inf])
+    for dt in (torch.bfloat16, torch.float16):
+        score = row.to(dt).view(1, 1, 1, -1)
+        for k in (1, 3, 6, 10, 16):
+            got, _ = topk_block_order_only_gpu(score, k)
+            want, _ = O.select_topk(score, k)
+            assert got.flatten().tolist() == sorted(want.flatten().tolist())
+
+
 def test_score_topk_pipeline_matches_oracle_given_gpu_scores():
     g = torch.Generator().manual_seed(9)
     qc = torch.randn(1, 4, 312, 128, generator=g).bfloat16() * 0.2
