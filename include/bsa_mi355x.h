@@ -226,10 +226,9 @@ int bsa_fwd_3d(const bsa_3d_params* p,
  *   q, o, d_o, dq [B, Hn, Sq, D]; k, v, dk, dv [B, Hn, Sk, D]: contiguous, blocked order, bf16 / fp16, D == 128.
  *   lse [B, Hn, Sq] fp32 (natural log) and idx / lens as bsa_fwd took and returned them (a row names a block at
  *   most once); tile_valid as in bsa_fwd (padded keys get no gradient and give none).
- *   workspace: bsa_bwd_workspace_bytes() bytes, 256-byte aligned (the scaled k and two fragment-order copies
- *   of k / v sized tensors, two fp32 vectors per query row, a bit matrix [kv block][query block], a copy of the
- *   lists, two small per-block tables).  Ascending lists are walked in bsa_visit_order's order by the dQ kernel
- *   (fp32 roundings only).
+ *   workspace: bsa_bwd_workspace_bytes() bytes, 256-byte aligned (the scaled k, two fp32 vectors per query row, a
+ *   bit matrix [kv block][query block], a copy of the lists, two small per-block tables).  Ascending lists are
+ *   walked in bsa_visit_order's order by the dQ kernel (fp32 roundings only).
  */
 size_t bsa_bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int D, int bs_q, int bs_k, int idx_stride, int dtype);
 int bsa_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,

@@ -8,10 +8,10 @@
 //   ds = p * (dp - delta) rounded to the storage type, p rounded to the storage type for dV;
 //   dV = sum p^T do,  dK = sm_scale * sum ds^T q,  dQ = ln 2 * sum ds k_s  (fp32 accumulators, one final rounding).
 //
-// Data movement of dQ as in bsa_fwd_frag.hip: k_s and v are first rewritten into fragment order (frag_kernel, "row
-// layout" = the K layout of that file: A operand whose rows are tokens), so a wavefront loads a fragment with one
-// coalesced 16-byte load per lane.  The transposed K_s fragments (A operand whose rows are head-dim columns,
-// contraction over 16 tokens in accumulator order) are made in the kernel from the row fragments, through LDS.
+// Data movement: k (pre-scaled) and v, q and dO are read as they lie in memory, in blocked order, through LDS
+// (global_load_lds_dwordx4): no fragment-order copies.  Row fragments (A operand whose rows are tokens) come out of
+// LDS with ds_read_b128, transposed ones (A operand whose rows are head-dim columns, contraction over 16 tokens in
+// accumulator order) with ds_read_b64_tr_b16.
 //
 // dQ: one wavefront per 64 query rows (two halves of 32, so that every K_s and V fragment feeds two MFMAs).
 // S^T = K_s Q^T and dP^T = V dO^T (Q and dO rows in registers as B operands) put one query per lane, so M2 and
@@ -32,6 +32,7 @@ namespace {
 using namespace mfma;
 
 constexpr float kRcpLn2 = 1.4426950408889634f;
+constexpr int kBwdHalfTileBytes = kTileBytes / 2;            // 32 rows of 256 B
 
 // ------------------------------------------------------------------ small passes
 // delta[row] = sum_d o * do (fp32), m2[row] = lse * log2(e), +inf for rows without any key (their p is then 0).
@@ -104,17 +105,6 @@ __global__ __launch_bounds__(256) void bwd_count_kernel(const uint32_t* __restri
     counts[row] = c;
 }
 
-// ------------------------------------------------------------------ fragment access
-// row layout: [tile][half h][d step c][lane][8];  transposed layout: [tile][half h][16-row step s][d tile t][lane][8]
-template <typename V8>
-__device__ __forceinline__ V8 frag_row(const char* base, int64_t tile, int h, int c, uint32_t lane_off) {
-    return *reinterpret_cast<const V8*>(base + tile * kTileBytes + h * (kTileBytes / 2) + c * 1024 + lane_off);
-}
-template <typename V8>
-__device__ __forceinline__ V8 frag_tr(const char* base, int64_t tile, int h, int s, int t, uint32_t lane_off) {
-    return *reinterpret_cast<const V8*>(base + tile * kTileBytes + h * (kTileBytes / 2) + (4 * s + t) * 1024 + lane_off);
-}
-
 template <typename T, typename V8>
 __device__ __forceinline__ V8 pack8(const f32x16& x, int s) {
     V8 r;
@@ -124,24 +114,35 @@ __device__ __forceinline__ V8 pack8(const f32x16& x, int s) {
 }
 
 // ------------------------------------------------------------------ dQ
-constexpr int kDqLds = 32 * 256;                             // the K_s rows of a half tile, on their way to being transposed
+// One wavefront per 64 query rows, as two halves of 32 so that every K_s and V fragment feeds two MFMAs.  The K_s and
+// V rows of a half tile (32 keys x 256 B each, as they lie in memory - no fragment-order copies) go from global
+// memory straight into the wavefront's own LDS (global_load_lds_dwordx4, two stages of 16 KB: one being read, one on
+// its way, completion counted by hand), the row fragments come from there with ds_read_b128 and the transposed K_s
+// fragments with ds_read_b64_tr_b16 (slot p of row r holds 16-byte unit p ^ f(r), f(r) = ((r << 1) & 14) | ((r >> 3) & 1),
+// applied on the global side of the DMA, so that neither kind of read collides on a bank).  That leaves the registers
+// for two sets of S^T / dP^T accumulators, so the products of the next half are issued between the exponentials of
+// this one: the wavefront has its SIMD to itself and nothing else fills the MFMA pipe while it computes
+// exponentials.  S^T and dP^T accumulate in ordinary registers (MFMAs from inline assembly, Q and dO named in the
+// accumulation registers they are kept in); the compiler adds no wait states behind such an MFMA and moves no LDS
+// read across it, so a set is first read a whole group of MFMAs after it was written and the row fragments are
+// requested a group ahead by hand.
+constexpr int kDqStage = 2 * kBwdHalfTileBytes;              // K_s rows and V rows of 32 keys
+constexpr int kDqRingLds = 2 * kDqStage;
 
-template <typename T>
-__global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, const T* __restrict__ dout,
-                                                    const char* __restrict__ ks_row,
-                                                    const char* __restrict__ v_row, const float* __restrict__ m2,
-                                                    const float* __restrict__ delta, const int32_t* __restrict__ idx,
-                                                    const int32_t* __restrict__ lens,
-                                                    const uint64_t* __restrict__ tile_valid, T* __restrict__ dq,
-                                                    int64_t Sq, int64_t Sk, int bs_q, int bs_k, int stride, int item_begin,
-                                                    int item_end, int round) {
+// kMasked: the caller has a validity word per KV tile (padding keys exist); without one the test of every P element
+// is compiled out - three of its seven instructions, in a kernel whose time is its instruction issue.
+template <typename T, bool kMasked>
+__global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q, const T* __restrict__ dout,
+                                                        const T* __restrict__ ks, const T* __restrict__ v,
+                                                        const float* __restrict__ m2, const float* __restrict__ delta,
+                                                        const int32_t* __restrict__ idx, const int32_t* __restrict__ lens,
+                                                        const uint64_t* __restrict__ tile_valid, T* __restrict__ dq,
+                                                        int64_t Sq, int64_t Sk, int bs_q, int bs_k, int stride, int item_begin,
+                                                        int item_end, int round) {
     typedef typename Vec8<T>::type V8;
+    extern __shared__ __attribute__((aligned(1024))) char dq_ring[];
     const int lane = threadIdx.x, lr = lane & 31, lh = lane >> 5;
-    const uint32_t lane_off = (uint32_t)lane * 16u;
     const int64_t groups = Sq / kTile;
-    // The launch's items are taken in rounds of `round` (a multiple of 8) in workgroup order; workgroup b runs on
-    // XCD b % 8 and within a round every XCD takes a contiguous run of the round's items, as in the forward kernel:
-    // the items of a round walk their lists together and share K_s / V tiles in L2.
     int64_t item;
     {
         const int local = blockIdx.x, r0 = local / round * round;
@@ -152,13 +153,11 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
     const int64_t qrow0 = (item % groups) * kTile;
     const int nbq = (int)(Sq / bs_q), nbk = (int)(Sk / bs_k), nsub = bs_k / kTile;
     const int64_t lrow = bh * nbq + qrow0 / bs_q;
-    const int n = min(max(lens[lrow], 0), stride);
+    const int n = __builtin_amdgcn_readfirstlane(min(max(lens[lrow], 0), stride));
     const int32_t* list = idx + lrow * stride;
-    const int64_t kv_tiles = Sk / kTile;
-    const char* ksr = ks_row + bh * kv_tiles * kTileBytes;
-    const char* vr = v_row + bh * kv_tiles * kTileBytes;
+    const char* k_src = reinterpret_cast<const char*>(ks) + bh * Sk * (int64_t)(kD * 2);
+    const char* v_src = reinterpret_cast<const char*>(v) + bh * Sk * (int64_t)(kD * 2);
 
-    // two query halves of 32 rows: every K_s / V fragment feeds two MFMAs
     V8 qreg[2][8], doreg[2][8];
     float m_row[2], d_row[2];
 #pragma unroll
@@ -180,26 +179,38 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[t][qq][i] = 0.f;
 
-    // The row fragments of a half tile (K_s rows, V rows: 16 KB) are requested one half ahead of their use, into two
-    // register buffers that take turns; the transposed K_s fragments at the start of the half that uses them.
-    struct Frags { V8 k[8], v[8]; };
-    auto load = [&](Frags& f, int64_t tile, int h) {
-#pragma unroll
-        for (int c = 0; c < 8; ++c) f.k[c] = frag_row<V8>(ksr, tile, h, c, lane_off);
-#pragma unroll
-        for (int c = 0; c < 8; ++c) f.v[c] = frag_row<V8>(vr, tile, h, c, lane_off);
+    const int ntiles = n * nsub, nhalves = 2 * ntiles;
+    auto tile_at = [&](int tp) -> int64_t {
+        const int tc = min(tp, ntiles - 1);
+        return (int64_t)min(max(list[tc / nsub], 0), nbk - 1) * nsub + tc % nsub;
     };
-    // The transposed K_s fragments of a half (the A operands of dQ^T += K_s^T dS^T) are made from its row fragments:
-    // every lane parks its 16-byte pieces in the wavefront's 8 KB of LDS and ds_read_b64_tr_b16 hands them back with
-    // rows and columns exchanged, which saves a third of the bytes that the wavefront pulls through the L1 path and a
-    // fragment-order copy of k_s.  Piece u of key row r lies in slot u ^ f(r), f(r) = ((r << 1) & 14) | ((r >> 3) & 1):
-    // neither the writes (16 consecutive rows) nor the 4-row patches of a transposing read collide on a bank.
-    extern __shared__ __attribute__((aligned(16))) char dq_lds[];
-    V8 kt[8];
-    const uint32_t fl = (uint32_t)(((lr << 1) & 14) | ((lr >> 3) & 1));
-    uint32_t woff[8];
+    // ---- global -> LDS: 16 loads of 1 KB per half
+    const uint32_t lds0 = lds_address(dq_ring);
+    uint32_t voff[4];
 #pragma unroll
-    for (int c = 0; c < 8; ++c) woff[c] = (uint32_t)(lr * 256) + ((((uint32_t)(2 * c + lh)) ^ fl) << 4);
+    for (int i = 0; i < 4; ++i) {
+        const int row = 4 * i + (lane >> 4);                                     // + 16 j
+        const int f = ((row << 1) & 14) | ((row >> 3) & 1);
+        voff[i] = (uint32_t)(row * 256 + (((lane & 15) ^ f) << 4));
+    }
+    auto issue = [&](int hp) {
+        if (hp >= nhalves) return;
+        const int64_t tile = (int64_t)__builtin_amdgcn_readfirstlane((int)tile_at(hp >> 1));
+        const int64_t off = tile * kTileBytes + (hp & 1) * kBwdHalfTileBytes;
+        const uint32_t dst = lds0 + (hp & 1) * kDqStage;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                load_to_lds_16(k_src + off + j * 4096, voff[i], dst + j * 4096 + i * 1024);
+                load_to_lds_16(v_src + off + j * 4096, voff[i], dst + kBwdHalfTileBytes + j * 4096 + i * 1024);
+            }
+    };
+    // ---- LDS -> fragments
+    const uint32_t fl = (uint32_t)(((lr << 1) & 14) | ((lr >> 3) & 1));
+    uint32_t roff[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) roff[c] = (uint32_t)(lr * 256) + ((((uint32_t)(2 * c + lh)) ^ fl) << 4);
     const int s16 = lane & 15, g1 = (lane >> 4) & 1, tx = s16 >> 2, ty = (s16 & 3) >> 1, tz = s16 & 1;
     uint32_t toff[4][2];
 #pragma unroll
@@ -208,51 +219,58 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
         for (int hi = 0; hi < 2; ++hi)
             toff[t][hi] = (uint32_t)((4 * lh + tx + 8 * hi) * 256) + ((((uint32_t)(4 * t + 2 * g1 + ty)) ^ (uint32_t)((8 * lh + 2 * tx) | hi)) << 4) +
                           (uint32_t)(tz * 8);
-    auto park_rows = [&](const V8 (&krow)[8]) {
-#pragma unroll
-        for (int c = 0; c < 8; ++c) *reinterpret_cast<V8*>(dq_lds + woff[c]) = krow[c];
-    };
-    auto take_transposed = [&]() {
+    V8 kt[8];                                    // the transposed K_s fragments of the half whose dQ products come next
+    auto take_transposed = [&](int hp) {
+        const char* part = dq_ring + (hp & 1) * kDqStage;
 #pragma unroll
         for (int x = 0; x < 8; ++x) {
-            const char* base = dq_lds + (16 * (x >> 2)) * 256;
+            const char* base = part + (16 * (x >> 2)) * 256;
             const s16x4 lo = lds_read_tr16(base + toff[x & 3][0]), hi = lds_read_tr16(base + toff[x & 3][1]);
             kt[x] = __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         }
     };
-    auto compute = [&](const Frags& f, uint32_t hv) {
-        f32x16 s[2], dp[2];
+    // accumulator i <-> key 8 (i / 4) + 4 lh + i % 4 of the half, query lr (+ 32)
+    auto exponentials = [&](f32x16 (&s)[2], f32x16 (&dp)[2], uint32_t hv, int qq, int i0, int count) {
 #pragma unroll
-        for (int qq = 0; qq < 2; ++qq)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) { s[qq][i] = 0.f; dp[qq][i] = 0.f; }
-        park_rows(f.k);
-#pragma unroll
-        for (int c = 0; c < 8; ++c)
-#pragma unroll
-            for (int qq = 0; qq < 2; ++qq) {
-                s[qq] = mfma32(f.k[c], qreg[qq][c], s[qq]);
-                dp[qq] = mfma32(f.v[c], doreg[qq][c], dp[qq]);
-            }
-        // The 16 loads of the next half (requested by the caller just before this step) go out one behind every
-        // third MFMA of this step: a load that finds the CU's address unit busy holds up the wavefront's next
-        // instructions, and four wavefronts that each ask for 16 KB in one burst keep it busy for most of a step.
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        }
-        take_transposed();
-        // accumulator i <-> key 8 (i / 4) + 4 lh + i % 4 of the half, query lr (+ 32)
-#pragma unroll
-        for (int qq = 0; qq < 2; ++qq)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
+        for (int i = i0; i < i0 + count; ++i) {
+            float p = __builtin_amdgcn_exp2f(s[qq][i] - m_row[qq]);
+            if (kMasked) {
                 const int key = 8 * (i / 4) + 4 * lh + (i % 4);
-                float p = __builtin_amdgcn_exp2f(s[qq][i] - m_row[qq]);
                 if (!((hv >> key) & 1u)) p = 0.f;
-                s[qq][i] = p * (dp[qq][i] - d_row[qq]);
             }
+            s[qq][i] = p * (dp[qq][i] - d_row[qq]);
+        }
+    };
+    // S^T and dP^T of half hp (both query halves) into (s, dp); between its groups of four MFMAs the exponentials of
+    // the half before, on (ps, pdp), eight accumulators per group.
+    auto products = [&](int hp, f32x16 (&s)[2], f32x16 (&dp)[2], auto&& between) {
+        const char* kp = dq_ring + (hp & 1) * kDqStage;
+        const char* vp = kp + kBwdHalfTileBytes;
+        V8 fk[2], fv[2];
+        fk[0] = *reinterpret_cast<const V8*>(kp + roff[0]);
+        fv[0] = *reinterpret_cast<const V8*>(vp + roff[0]);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const int b = c & 1;
+            if (c < 7) {
+                fk[b ^ 1] = *reinterpret_cast<const V8*>(kp + roff[c + 1]);
+                fv[b ^ 1] = *reinterpret_cast<const V8*>(vp + roff[c + 1]);
+            }
+            if (c == 0) {
+                mfma_s<true, true>(s[0], fk[b], qreg[0][0]);
+                mfma_s<true, true>(dp[0], fv[b], doreg[0][0]);
+                mfma_s<true, true>(s[1], fk[b], qreg[1][0]);
+                mfma_s<true, true>(dp[1], fv[b], doreg[1][0]);
+            } else {
+                mfma_s<false, true>(s[0], fk[b], qreg[0][c]);
+                mfma_s<false, true>(dp[0], fv[b], doreg[0][c]);
+                mfma_s<false, true>(s[1], fk[b], qreg[1][c]);
+                mfma_s<false, true>(dp[1], fv[b], doreg[1][c]);
+            }
+            between(c);
+        }
+    };
+    auto gradients = [&](const f32x16 (&s)[2]) {
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
             const V8 ds0 = pack8<T, V8>(s[0], st), ds1 = pack8<T, V8>(s[1], st);
@@ -263,23 +281,37 @@ __global__ __launch_bounds__(64) void bwd_dq_kernel(const T* __restrict__ q, con
             }
         }
     };
-    const int ntiles = n * nsub;
-    auto tile_at = [&](int tp) -> int64_t {
-        const int tc = min(tp, ntiles - 1);
-        return (int64_t)min(max(list[tc / nsub], 0), nbk - 1) * nsub + tc % nsub;
+    auto valid_half = [&](int hp) -> uint32_t {
+        if (!kMasked) return ~0u;
+        const uint64_t w = tile_valid[tile_at(min(hp, nhalves - 1) >> 1)];
+        return (uint32_t)(w >> (32 * (hp & 1)));
     };
-    if (ntiles > 0) {
-        Frags fa, fb;
-        int64_t tile = tile_at(0);
-        load(fa, tile, 0);
-        for (int tp = 0; tp < ntiles; ++tp) {
-            const uint64_t valid = tile_valid != nullptr ? tile_valid[tile] : ~0ull;
-            load(fb, tile, 1);
-            compute(fa, (uint32_t)valid);
-            const int64_t next = tile_at(tp + 1);
-            load(fa, next, 0);                            // behind the last tile: loaded again, not used
-            compute(fb, (uint32_t)(valid >> 32));
-            tile = next;
+    // (s, dp): this half, products done; (ns, ndp): the next half
+    auto step = [&](int hp, f32x16 (&s)[2], f32x16 (&dp)[2], f32x16 (&ns)[2], f32x16 (&ndp)[2]) {
+        const uint32_t hv = valid_half(hp);
+        // the stage that this half was read from (rows and transposed fragments are in registers) takes half hp + 2
+        issue(hp + 2);
+        if (hp + 2 < nhalves) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        products(hp + 1, ns, ndp, [&](int c) { exponentials(s, dp, hv, c >> 2, 4 * (c & 3), 4); });
+        __builtin_amdgcn_sched_barrier(0);
+        gradients(s);
+        __builtin_amdgcn_sched_barrier(0);
+        take_transposed(hp + 1);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    if (nhalves > 0) {
+        f32x16 sa[2], dpa[2], sb[2], dpb[2];
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the Q / dO rows: from here on the DMA loads are counted by hand
+        issue(0);
+        issue(1);
+        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        products(0, sa, dpa, [&](int) {});
+        take_transposed(0);
+        asm volatile("s_nop 15\n\ts_nop 7\n\ts_waitcnt lgkmcnt(0)" ::: "memory");
+        for (int hp = 0; hp < nhalves; hp += 2) {                                // halves come in pairs
+            step(hp, sa, dpa, sb, dpb);
+            step(hp + 1, sb, dpb, sa, dpa);
         }
     }
     // accumulator i of d tile t <-> d = 32 t + 8 (i / 4) + 4 lh + i % 4, query lr (+ 32)
@@ -563,14 +595,13 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
 
 }  // namespace
 
-// Workspace of the backward, in bytes: two fragment-order copies ([B*Hn][Sk/64][16 KB]: k_s and v in row layout),
-// k_s in blocked order, delta and M2, the bit matrix, the lists in the dQ kernel's visiting
+// Workspace of the backward, in bytes: k_s in blocked order, delta and M2, the bit matrix, the lists in the dQ kernel's visiting
 // order, per KV block its number of query blocks, the KV tiles of every head by that number.
 size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride) {
     const size_t bh = (size_t)B * Hn;
     auto up = [](size_t x) { return (x + 255) / 256 * 256; };
     const size_t words = (size_t)((Sq / bs_q + 31) / 32);
-    return 3 * up(bh * Sk * kD * 2) + 2 * up(bh * Sq * 4) + up(bh * (Sk / bs_k) * words * 4) +
+    return up(bh * Sk * kD * 2) + 2 * up(bh * Sq * 4) + up(bh * (Sk / bs_k) * words * 4) +
            up(bh * (Sq / bs_q) * (size_t)idx_stride * 4) + up(bh * (Sk / bs_k) * 4) + up(bh * (Sk / kTile) * 4);
 }
 
@@ -582,8 +613,6 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     auto up = [](size_t x) { return (x + 255) / 256 * 256; };
     char* ws = static_cast<char*>(workspace);
     auto take = [&](size_t n) { char* p = ws; ws += up(n); return p; };
-    char* ks_row = take(bh * Sk * kD * 2);
-    char* v_row = take(bh * Sk * kD * 2);
     char* ks = take(bh * Sk * kD * 2);
     float* delta = reinterpret_cast<float*>(take(bh * Sq * 4));
     float* m2 = reinterpret_cast<float*>(take(bh * Sq * 4));
@@ -612,17 +641,12 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     const int64_t lrows = (int64_t)bh * nbq;
     hipLaunchKernelGGL(bwd_mask_kernel, dim3((unsigned)((lrows + 3) / 4)), dim3(256), 0, st, idx, lens, bits, nbq, nbk, idx_stride,
                        words, lrows);
-    // blocked-order tensors as a grid of 64-token chunks along one axis
-    const Grid3 gk = make_grid((int)(Sk / kTile), 1, kTile, 1, 1, kTile);
-    const int64_t stk[3] = {(int64_t)Hn * Sk * kD, Sk * kD, kD};
     hipError_t e;
     hipLaunchKernelGGL(bwd_count_kernel, dim3((unsigned)((bh * nbk + 255) / 256)), dim3(256), 0, st, bits, counts, words, (int64_t)(bh * nbk));
     if ((e = launch_order_by_length(counts, order, (int)bh, nbk, bs_k / kTile, nbq, st)) != hipSuccess) return e;
     // dQ walks every list in the forward kernel's visiting order when the list is ascending (a selection in block
     // order); any other order is walked as given.  The order only moves fp32 roundings of the dQ sum.
     if ((e = launch_pace_order(idx, paced, lens, (int64_t)bh * nbq, nbk, idx_stride, st)) != hipSuccess) return e;
-    if ((e = launch_frag(ks, stk, ks_row, B, Hn, gk, dtype, false, st)) != hipSuccess) return e;
-    if ((e = launch_frag(v, stk, v_row, B, Hn, gk, dtype, false, st)) != hipSuccess) return e;
 
     const dim3 block(64);
     // the dK / dV kernel's LDS: four stages of half a Q tile, half a dO tile and the queries' M2 / delta, then a KV block's query blocks
@@ -642,8 +666,14 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     if (dtype == BSA_BF16) {
         for (int first = 0; first < total_q; first += span) {
             const int end = first + span < total_q ? first + span : total_q;
-            hipLaunchKernelGGL((bwd_dq_kernel<__bf16>), dim3(end - first), block, kDqLds, st, (const __bf16*)q, (const __bf16*)dout, ks_row,
-                               v_row, m2, delta, paced, lens, tile_valid, (__bf16*)dq, Sq, Sk, bs_q, bs_k, idx_stride, first, end, round);
+            if (tile_valid != nullptr)
+                hipLaunchKernelGGL((bwd_dq_lds_kernel<__bf16, true>), dim3(end - first), block, kDqRingLds, st, (const __bf16*)q,
+                                   (const __bf16*)dout, (const __bf16*)ks, (const __bf16*)v, m2, delta, paced, lens, tile_valid, (__bf16*)dq, Sq, Sk,
+                                   bs_q, bs_k, idx_stride, first, end, round);
+            else
+                hipLaunchKernelGGL((bwd_dq_lds_kernel<__bf16, false>), dim3(end - first), block, kDqRingLds, st, (const __bf16*)q,
+                                   (const __bf16*)dout, (const __bf16*)ks, (const __bf16*)v, m2, delta, paced, lens, tile_valid, (__bf16*)dq, Sq, Sk,
+                                   bs_q, bs_k, idx_stride, first, end, round);
         }
         hipLaunchKernelGGL((bwd_dkdv_kernel<__bf16>), grid_k, dim3(128), lds, st, (const __bf16*)q, (const __bf16*)dout, (const __bf16*)ks,
                            (const __bf16*)v, m2, delta, bits, tile_valid, (__bf16*)dk, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words, sm_scale, order,
@@ -651,9 +681,14 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     } else {
         for (int first = 0; first < total_q; first += span) {
             const int end = first + span < total_q ? first + span : total_q;
-            hipLaunchKernelGGL((bwd_dq_kernel<_Float16>), dim3(end - first), block, kDqLds, st, (const _Float16*)q, (const _Float16*)dout,
-                               ks_row, v_row, m2, delta, paced, lens, tile_valid, (_Float16*)dq, Sq, Sk, bs_q, bs_k, idx_stride, first,
-                               end, round);
+            if (tile_valid != nullptr)
+                hipLaunchKernelGGL((bwd_dq_lds_kernel<_Float16, true>), dim3(end - first), block, kDqRingLds, st, (const _Float16*)q,
+                                   (const _Float16*)dout, (const _Float16*)ks, (const _Float16*)v, m2, delta, paced, lens, tile_valid, (_Float16*)dq,
+                                   Sq, Sk, bs_q, bs_k, idx_stride, first, end, round);
+            else
+                hipLaunchKernelGGL((bwd_dq_lds_kernel<_Float16, false>), dim3(end - first), block, kDqRingLds, st, (const _Float16*)q,
+                                   (const _Float16*)dout, (const _Float16*)ks, (const _Float16*)v, m2, delta, paced, lens, tile_valid, (_Float16*)dq,
+                                   Sq, Sk, bs_q, bs_k, idx_stride, first, end, round);
         }
         hipLaunchKernelGGL((bwd_dkdv_kernel<_Float16>), grid_k, dim3(128), lds, st, (const _Float16*)q, (const _Float16*)dout,
                            (const _Float16*)ks, (const _Float16*)v, m2, delta, bits, tile_valid, (_Float16*)dk, (_Float16*)dv, Sq, Sk, bs_q, bs_k,
