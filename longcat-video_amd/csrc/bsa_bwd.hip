@@ -126,6 +126,15 @@ __device__ __forceinline__ V8 pack8(const f32x16& x, int s) {
 // accumulation registers they are kept in); the compiler adds no wait states behind such an MFMA and moves no LDS
 // read across it, so a set is first read a whole group of MFMAs after it was written and the row fragments are
 // requested a group ahead by hand.
+// First MFMA of a chain that starts from a block of registers instead of zero (B operand in an accumulation
+// register): S^T - M2 comes out of the products, and the exponentials need no subtraction.
+__device__ inline void mfma_from(f32x16& acc, bf16x8 a, bf16x8 b, const f32x16& init) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), "a"(b), "v"(init));
+}
+__device__ inline void mfma_from(f32x16& acc, f16x8 a, f16x8 b, const f32x16& init) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), "a"(b), "v"(init));
+}
+
 constexpr int kDqStage = 2 * kBwdHalfTileBytes;              // K_s rows and V rows of 32 keys
 constexpr int kDqRingLds = 2 * kDqStage;
 
@@ -178,6 +187,11 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
         for (int qq = 0; qq < 2; ++qq)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[t][qq][i] = 0.f;
+    f32x16 neg_m[2];                             // what the S^T accumulators of a query half start from
+#pragma unroll
+    for (int qq = 0; qq < 2; ++qq)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) neg_m[qq][i] = -m_row[qq];
 
     const int ntiles = n * nsub, nhalves = 2 * ntiles;
     auto tile_at = [&](int tp) -> int64_t {
@@ -233,7 +247,7 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
     auto exponentials = [&](f32x16 (&s)[2], f32x16 (&dp)[2], uint32_t hv, int qq, int i0, int count) {
 #pragma unroll
         for (int i = i0; i < i0 + count; ++i) {
-            float p = __builtin_amdgcn_exp2f(s[qq][i] - m_row[qq]);
+            float p = __builtin_amdgcn_exp2f(s[qq][i]);              // s holds S^T - M2
             if (kMasked) {
                 const int key = 8 * (i / 4) + 4 * lh + (i % 4);
                 if (!((hv >> key) & 1u)) p = 0.f;
@@ -257,9 +271,9 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
                 fv[b ^ 1] = *reinterpret_cast<const V8*>(vp + roff[c + 1]);
             }
             if (c == 0) {
-                mfma_s<true, true>(s[0], fk[b], qreg[0][0]);
+                mfma_from(s[0], fk[b], qreg[0][0], neg_m[0]);
                 mfma_s<true, true>(dp[0], fv[b], doreg[0][0]);
-                mfma_s<true, true>(s[1], fk[b], qreg[1][0]);
+                mfma_from(s[1], fk[b], qreg[1][0], neg_m[1]);
                 mfma_s<true, true>(dp[1], fv[b], doreg[1][0]);
             } else {
                 mfma_s<false, true>(s[0], fk[b], qreg[0][c]);
