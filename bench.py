@@ -298,7 +298,7 @@ def run_bwd(torch, args):
         "data": "synthetic N(0,1) q/k/v with per-head RMS-normalised q/k and N(0,1) output gradient, seeded on the GPU",
         "config": {"workload": "bwd: backward of the c3 layer in blocked order, 32 heads x 128, 1440 x 1440 blocks of 64, 90 per row",
                    "block_pairs": pairs},
-        "roofline": {"kernel": "bwd_dq_kernel<bf16> + bwd_dkdv_kernel<bf16> (with the passes before them)", "bound": "mfma",
+        "roofline": {"kernel": "bwd_dq_lds_kernel<bf16> + bwd_dkdv_kernel<bf16> (with the passes before them)", "bound": "mfma",
                      "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / PEAK_BF16_TFLOPS, 4),
                      "traffic": recorded_traffic("bwd", "bsa_backward_*.md", BACKWARD_SOURCES), "ms": round(ms, 4)}}
