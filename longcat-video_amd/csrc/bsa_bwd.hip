@@ -35,7 +35,8 @@ constexpr float kRcpLn2 = 1.4426950408889634f;
 constexpr int kBwdHalfTileBytes = kTileBytes / 2;            // 32 rows of 256 B
 
 // ------------------------------------------------------------------ small passes
-// delta[row] = sum_d o * do (fp32), m2[row] = lse * log2(e), +inf for rows without any key (their p is then 0).
+// Per query row, both negated because the kernels below add them (as the start value of an MFMA chain):
+// delta[row] = -sum_d o * do (fp32), m2[row] = -lse * log2(e), -inf for rows without any key (their p is then 0).
 // One 16-lane group per row.
 template <typename T>
 __global__ __launch_bounds__(256) void bwd_rows_kernel(const T* __restrict__ o, const T* __restrict__ dout,
@@ -54,9 +55,9 @@ __global__ __launch_bounds__(256) void bwd_rows_kernel(const T* __restrict__ o, 
 #pragma unroll
     for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off);
     if (row < rows && c == 0) {
-        delta[row] = s;
+        delta[row] = -s;
         const float l = lse[row];
-        m2[row] = l == -INFINITY ? INFINITY : l * kRcpLn2;
+        m2[row] = l == -INFINITY ? -INFINITY : -(l * kRcpLn2);
     }
 }
 
@@ -134,6 +135,13 @@ __device__ inline void mfma_from(f32x16& acc, bf16x8 a, bf16x8 b, const f32x16& 
 __device__ inline void mfma_from(f32x16& acc, f16x8 a, f16x8 b, const f32x16& init) {
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), "a"(b), "v"(init));
 }
+// the same with the B operand in an ordinary register
+__device__ inline void mfma_from_v(f32x16& acc, bf16x8 a, bf16x8 b, const f32x16& init) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), "v"(b), "v"(init));
+}
+__device__ inline void mfma_from_v(f32x16& acc, f16x8 a, f16x8 b, const f32x16& init) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), "v"(b), "v"(init));
+}
 
 constexpr int kDqStage = 2 * kBwdHalfTileBytes;              // K_s rows and V rows of 32 keys
 constexpr int kDqRingLds = 2 * kDqStage;
@@ -191,7 +199,7 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
 #pragma unroll
     for (int qq = 0; qq < 2; ++qq)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) neg_m[qq][i] = -m_row[qq];
+        for (int i = 0; i < 16; ++i) neg_m[qq][i] = m_row[qq];       // m2 and delta come negated
 
     const int ntiles = n * nsub, nhalves = 2 * ntiles;
     auto tile_at = [&](int tp) -> int64_t {
@@ -252,7 +260,7 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
                 const int key = 8 * (i / 4) + 4 * lh + (i % 4);
                 if (!((hv >> key) & 1u)) p = 0.f;
             }
-            s[qq][i] = p * (dp[qq][i] - d_row[qq]);
+            s[qq][i] = p * (dp[qq][i] + d_row[qq]);
         }
     };
     // S^T and dP^T of half hp (both query halves) into (s, dp); between its groups of four MFMAs the exponentials of
@@ -363,7 +371,8 @@ constexpr int kBwdStats = 1024;                              // M2 (128 B), delt
 constexpr int kBwdStage = 2 * kBwdHalfTile + kBwdStats;      // one half tile of queries: Q rows, dO rows, M2, delta
 constexpr int kBwdStages = 4;                                // two in use (this half, the next half's rows), two on their way
 
-template <typename T>
+// kMasked: as in the dQ kernel - without validity words no key is padding and the test is compiled out.
+template <typename T, bool kMasked>
 __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, const T* __restrict__ dout,
                                                        const T* __restrict__ ks, const T* __restrict__ v,
                                                        const float* __restrict__ m2, const float* __restrict__ delta,
@@ -400,7 +409,7 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
         }
     }
     bool key_ok = true;
-    if (tile_valid != nullptr) key_ok = (tile_valid[krow0 / kTile] >> (32 * wave + lr)) & 1ull;
+    if (kMasked) key_ok = (tile_valid[krow0 / kTile] >> (32 * wave + lr)) & 1ull;
     f32x16 acc_dk[4], acc_dv[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
@@ -490,19 +499,27 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
     auto products_and_exponentials = [&](int hp, f32x16& s, f32x16& dp, f32x16& s_next, f32x16& dp_next) {
         const char* qn = bwd_lds + ((hp + 1) & 3) * kBwdStage;
         const char* dn = qn + kBwdHalfTile;
-        const float* st_m2 = reinterpret_cast<const float*>(bwd_lds + (hp & 3) * kBwdStage + 2 * kBwdHalfTile);
+        // The chains of the next half start from its queries' -M2 and -delta (accumulator i <-> query
+        // 8 (i / 4) + 4 lh + i % 4 of the half, key lr), so S - M2 and dP - delta come out of the products and the
+        // exponentials need no subtraction.
+        const float* st_m2 = reinterpret_cast<const float*>(qn + 2 * kBwdHalfTile);
         const float* st_dl = st_m2 + 32;
+        f32x16 from_m, from_d;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const float4 mm = *reinterpret_cast<const float4*>(st_m2 + 8 * g + 4 * lh);
+            const float4 dd = *reinterpret_cast<const float4*>(st_dl + 8 * g + 4 * lh);
+            from_m[4 * g] = mm.x; from_m[4 * g + 1] = mm.y; from_m[4 * g + 2] = mm.z; from_m[4 * g + 3] = mm.w;
+            from_d[4 * g] = dd.x; from_d[4 * g + 1] = dd.y; from_d[4 * g + 2] = dd.z; from_d[4 * g + 3] = dd.w;
+        }
         // Volatile assembly keeps the compiler from moving LDS reads across it, so the operands of a group of four
-        // MFMAs (and the statistics of four accumulators) are requested a group ahead by hand.
+        // MFMAs are requested a group ahead by hand.
         V8 fq[2][2], fd[2][2];
-        float4 mm[2], dd[2];
         auto request = [&](int g, int b) {
             fq[b][0] = *reinterpret_cast<const V8*>(qn + roff[2 * g]);
             fd[b][0] = *reinterpret_cast<const V8*>(dn + roff[2 * g]);
             fq[b][1] = *reinterpret_cast<const V8*>(qn + roff[2 * g + 1]);
             fd[b][1] = *reinterpret_cast<const V8*>(dn + roff[2 * g + 1]);
-            mm[b] = *reinterpret_cast<const float4*>(st_m2 + 8 * g + 4 * lh);
-            dd[b] = *reinterpret_cast<const float4*>(st_dl + 8 * g + 4 * lh);
         };
         request(0, 0);
 #pragma unroll
@@ -510,23 +527,21 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
             const int c = 2 * g4, b = g4 & 1;
             if (g4 < 3) request(g4 + 1, b ^ 1);
             if (g4 == 0) {
-                mfma_s<true, false>(s_next, fq[b][0], kreg[0]);
-                mfma_s<true, false>(dp_next, fd[b][0], vreg[0]);
+                mfma_from_v(s_next, fq[b][0], kreg[0], from_m);
+                mfma_from_v(dp_next, fd[b][0], vreg[0], from_d);
             } else {
                 mfma_s<false, false>(s_next, fq[b][0], kreg[c]);
                 mfma_s<false, false>(dp_next, fd[b][0], vreg[c]);
             }
             mfma_s<false, false>(s_next, fq[b][1], kreg[c + 1]);
             mfma_s<false, false>(dp_next, fd[b][1], vreg[c + 1]);
-            // accumulator i <-> query 8 (i / 4) + 4 lh + i % 4 of the half, key lr
-            const float mv[4] = {mm[b].x, mm[b].y, mm[b].z, mm[b].w}, dl[4] = {dd[b].x, dd[b].y, dd[b].z, dd[b].w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int i = 4 * g4 + j;
-                float pi = __builtin_amdgcn_exp2f(s[i] - mv[j]);
-                if (!key_ok) pi = 0.f;
+                float pi = __builtin_amdgcn_exp2f(s[i]);        // s holds S - M2, dp holds dP - delta
+                if (kMasked && !key_ok) pi = 0.f;
                 s[i] = pi;                                   // P
-                dp[i] = pi * (dp[i] - dl[j]);                // dS
+                dp[i] = pi * dp[i];                          // dS
             }
         }
     };
@@ -574,8 +589,18 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
         {
             const char* qn = bwd_lds;
             const char* dn = qn + kBwdHalfTile;
-            mfma_s<true, false>(s0, *reinterpret_cast<const V8*>(qn + roff[0]), kreg[0]);
-            mfma_s<true, false>(dp0, *reinterpret_cast<const V8*>(dn + roff[0]), vreg[0]);
+            const float* st_m2 = reinterpret_cast<const float*>(qn + 2 * kBwdHalfTile);
+            const float* st_dl = st_m2 + 32;
+            f32x16 from_m, from_d;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 mm = *reinterpret_cast<const float4*>(st_m2 + 8 * g + 4 * lh);
+                const float4 dd = *reinterpret_cast<const float4*>(st_dl + 8 * g + 4 * lh);
+                from_m[4 * g] = mm.x; from_m[4 * g + 1] = mm.y; from_m[4 * g + 2] = mm.z; from_m[4 * g + 3] = mm.w;
+                from_d[4 * g] = dd.x; from_d[4 * g + 1] = dd.y; from_d[4 * g + 2] = dd.z; from_d[4 * g + 3] = dd.w;
+            }
+            mfma_from_v(s0, *reinterpret_cast<const V8*>(qn + roff[0]), kreg[0], from_m);
+            mfma_from_v(dp0, *reinterpret_cast<const V8*>(dn + roff[0]), vreg[0], from_d);
 #pragma unroll
             for (int c = 1; c < 8; ++c) {
                 mfma_s<false, false>(s0, *reinterpret_cast<const V8*>(qn + roff[c]), kreg[c]);
@@ -666,9 +691,12 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
     // the dK / dV kernel's LDS: four stages of half a Q tile, half a dO tile and the queries' M2 / delta, then a KV block's query blocks
     const size_t lds = (size_t)kBwdStages * kBwdStage + (size_t)nbq * sizeof(int32_t);
     if (lds > 160 * 1024) return hipErrorInvalidValue;
-    if (dtype == BSA_BF16) e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_dkdv_kernel<__bf16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    else e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_dkdv_kernel<_Float16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
+    const bool masked = tile_valid != nullptr;
+    const void* dkdv = dtype == BSA_BF16
+                           ? (masked ? reinterpret_cast<const void*>(bwd_dkdv_kernel<__bf16, true>) : reinterpret_cast<const void*>(bwd_dkdv_kernel<__bf16, false>))
+                           : (masked ? reinterpret_cast<const void*>(bwd_dkdv_kernel<_Float16, true>)
+                                     : reinterpret_cast<const void*>(bwd_dkdv_kernel<_Float16, false>));
+    if ((e = hipFuncSetAttribute(dkdv, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess) return e;
     const dim3 grid_k((unsigned)(bh * (Sk / kTile)));
     // dQ: rounds of as many wavefronts as the device runs at once (one per SIMD), two rounds per launch.  The dK / dV
     // kernel runs as one grid, longest list first: its lists (the query blocks of a KV block) differ in length, and
@@ -689,9 +717,14 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
                                    (const __bf16*)dout, (const __bf16*)ks, (const __bf16*)v, m2, delta, paced, lens, tile_valid, (__bf16*)dq, Sq, Sk,
                                    bs_q, bs_k, idx_stride, first, end, round);
         }
-        hipLaunchKernelGGL((bwd_dkdv_kernel<__bf16>), grid_k, dim3(128), lds, st, (const __bf16*)q, (const __bf16*)dout, (const __bf16*)ks,
-                           (const __bf16*)v, m2, delta, bits, tile_valid, (__bf16*)dk, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words, sm_scale, order,
-                           total_k, round);
+        if (masked)
+            hipLaunchKernelGGL((bwd_dkdv_kernel<__bf16, true>), grid_k, dim3(128), lds, st, (const __bf16*)q, (const __bf16*)dout,
+                               (const __bf16*)ks, (const __bf16*)v, m2, delta, bits, tile_valid, (__bf16*)dk, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words,
+                               sm_scale, order, total_k, round);
+        else
+            hipLaunchKernelGGL((bwd_dkdv_kernel<__bf16, false>), grid_k, dim3(128), lds, st, (const __bf16*)q, (const __bf16*)dout,
+                               (const __bf16*)ks, (const __bf16*)v, m2, delta, bits, tile_valid, (__bf16*)dk, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words,
+                               sm_scale, order, total_k, round);
     } else {
         for (int first = 0; first < total_q; first += span) {
             const int end = first + span < total_q ? first + span : total_q;
@@ -704,9 +737,14 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
                                    (const _Float16*)dout, (const _Float16*)ks, (const _Float16*)v, m2, delta, paced, lens, tile_valid, (_Float16*)dq,
                                    Sq, Sk, bs_q, bs_k, idx_stride, first, end, round);
         }
-        hipLaunchKernelGGL((bwd_dkdv_kernel<_Float16>), grid_k, dim3(128), lds, st, (const _Float16*)q, (const _Float16*)dout,
-                           (const _Float16*)ks, (const _Float16*)v, m2, delta, bits, tile_valid, (_Float16*)dk, (_Float16*)dv, Sq, Sk, bs_q, bs_k,
-                           words, sm_scale, order, total_k, round);
+        if (masked)
+            hipLaunchKernelGGL((bwd_dkdv_kernel<_Float16, true>), grid_k, dim3(128), lds, st, (const _Float16*)q, (const _Float16*)dout,
+                               (const _Float16*)ks, (const _Float16*)v, m2, delta, bits, tile_valid, (_Float16*)dk, (_Float16*)dv, Sq, Sk, bs_q,
+                               bs_k, words, sm_scale, order, total_k, round);
+        else
+            hipLaunchKernelGGL((bwd_dkdv_kernel<_Float16, false>), grid_k, dim3(128), lds, st, (const _Float16*)q, (const _Float16*)dout,
+                               (const _Float16*)ks, (const _Float16*)v, m2, delta, bits, tile_valid, (_Float16*)dk, (_Float16*)dv, Sq, Sk, bs_q,
+                               bs_k, words, sm_scale, order, total_k, round);
     }
     return hipGetLastError();
 }
