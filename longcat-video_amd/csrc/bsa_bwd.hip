@@ -496,7 +496,7 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
     // NEXT half (into a second pair of accumulators) are issued between the exponentials of this one.  S and dP
     // accumulate in ordinary registers, where the exponentials read them: MFMAs from inline assembly, behind which
     // the compiler adds no wait states - a pair is read a whole group of 16 MFMAs after it was written.
-    auto products_and_exponentials = [&](int hp, f32x16& s, f32x16& dp, f32x16& s_next, f32x16& dp_next) {
+    auto products_and_exponentials = [&](int hp, f32x16& s, f32x16& dp, f32x16& s_next, f32x16& dp_next, auto&& behind_requests) {
         const char* qn = bwd_lds + ((hp + 1) & 3) * kBwdStage;
         const char* dn = qn + kBwdHalfTile;
         // The chains of the next half start from its queries' -M2 and -delta (accumulator i <-> query
@@ -522,6 +522,7 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
             fd[b][1] = *reinterpret_cast<const V8*>(dn + roff[2 * g + 1]);
         };
         request(0, 0);
+        behind_requests();                       // the DMA set-up runs while the first LDS reads are on their way
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
             const int c = 2 * g4, b = g4 & 1;
@@ -562,8 +563,7 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
     // half requested after it may still be on its way (wavefront 0 issues 9 loads per half, wavefront 1 issues 8).
     auto step = [&](int hp, f32x16& s, f32x16& dp, f32x16& s_next, f32x16& dp_next) {
         // half hp + 3 takes the stage that half hp - 1 was read from: both wavefronts are past the barrier behind it
-        issue(hp + 3, (hp + 3) & 3);
-        products_and_exponentials(hp, s, dp, s_next, dp_next);
+        products_and_exponentials(hp, s, dp, s_next, dp_next, [&]() { issue(hp + 3, (hp + 3) & 3); });
         __builtin_amdgcn_sched_barrier(0);
         gradients(hp, s, dp);
         if (hp + 3 < nhalves) {
