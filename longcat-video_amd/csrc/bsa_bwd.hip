@@ -265,12 +265,13 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
     };
     // S^T and dP^T of half hp (both query halves) into (s, dp); between its groups of four MFMAs the exponentials of
     // the half before, on (ps, pdp), eight accumulators per group.
-    auto products = [&](int hp, f32x16 (&s)[2], f32x16 (&dp)[2], auto&& between) {
+    auto products = [&](int hp, f32x16 (&s)[2], f32x16 (&dp)[2], auto&& behind_requests, auto&& between) {
         const char* kp = dq_ring + (hp & 1) * kDqStage;
         const char* vp = kp + kBwdHalfTileBytes;
         V8 fk[2], fv[2];
         fk[0] = *reinterpret_cast<const V8*>(kp + roff[0]);
         fv[0] = *reinterpret_cast<const V8*>(vp + roff[0]);
+        behind_requests();                       // the DMA set-up runs while the first LDS reads are on their way
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
             const int b = c & 1;
@@ -311,11 +312,10 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
     // (s, dp): this half, products done; (ns, ndp): the next half
     auto step = [&](int hp, f32x16 (&s)[2], f32x16 (&dp)[2], f32x16 (&ns)[2], f32x16 (&ndp)[2]) {
         const uint32_t hv = valid_half(hp);
-        // the stage that this half was read from (rows and transposed fragments are in registers) takes half hp + 2
-        issue(hp + 2);
-        if (hp + 2 < nhalves) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        products(hp + 1, ns, ndp, [&](int c) { exponentials(s, dp, hv, c >> 2, 4 * (c & 3), 4); });
+        // The next half's rows must have landed; the stage that this half was read from (rows and transposed
+        // fragments are in registers) takes half hp + 2.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        products(hp + 1, ns, ndp, [&]() { issue(hp + 2); }, [&](int c) { exponentials(s, dp, hv, c >> 2, 4 * (c & 3), 4); });
         __builtin_amdgcn_sched_barrier(0);
         gradients(s);
         __builtin_amdgcn_sched_barrier(0);
@@ -328,7 +328,7 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
         issue(0);
         issue(1);
         asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-        products(0, sa, dpa, [&](int) {});
+        products(0, sa, dpa, [&]() {}, [&](int) {});
         take_transposed(0);
         asm volatile("s_nop 15\n\ts_nop 7\n\ts_waitcnt lgkmcnt(0)" ::: "memory");
         for (int hp = 0; hp < nhalves; hp += 2) {                                // halves come in pairs
