@@ -228,6 +228,61 @@ int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, con
     return e == hipSuccess ? BSA_OK : hip_fail(e, "fwd launch");
 }
 
+// ---- the fragment-order kernel for blocked-order callers --------------------------------------------------
+static int check_fwd_fragment(const void* q, const void* k, const void* v, const int32_t* idx, const int32_t* lens, void* o,
+                              int B, int Hn, int64_t Sq, int64_t Sk, int D, int bs_q, int bs_k, int idx_stride, float sm_scale,
+                              int dtype) {
+    if (dtype != BSA_BF16 && dtype != BSA_F16)
+        return set_error(BSA_ERR_UNSUPPORTED, "fwd_fragment: dtype %d is not built (bf16, fp16; fp32 runs through bsa_fwd)", dtype);
+    if (D != 128) return set_error(BSA_ERR_UNSUPPORTED, "fwd_fragment: head dim %d is not built (only 128)", D);
+    if (B <= 0 || Hn <= 0 || Sq <= 0 || Sk <= 0 || idx_stride < 0)
+        return set_error(BSA_ERR_BAD_ARG, "fwd_fragment: sizes must be positive (B=%d heads=%d Sq=%lld Sk=%lld)", B, Hn, (long long)Sq, (long long)Sk);
+    if ((int64_t)B * Hn > 65535) return set_error(BSA_ERR_UNSUPPORTED, "B*heads exceeds 65535");
+    if (bs_q <= 0 || bs_k <= 0 || bs_q % 64 != 0 || bs_k % 64 != 0)
+        return set_error(BSA_ERR_UNSUPPORTED, "fwd_fragment: chunk sizes %d/%d must be multiples of 64", bs_q, bs_k);
+    if (Sq % bs_q != 0 || Sk % bs_k != 0)
+        return set_error(BSA_ERR_SHAPE, "fwd_fragment: Sq=%lld / Sk=%lld are not multiples of the chunk sizes %d / %d", (long long)Sq, (long long)Sk, bs_q, bs_k);
+    if (idx_stride > 4096) return set_error(BSA_ERR_UNSUPPORTED, "fwd_fragment: lists of %d entries exceed the limit of 4096", idx_stride);
+    if ((Sq / 64) * (int64_t)B * Hn > 0x7fffffffLL || Sk / 64 > 0x7fffff)
+        return set_error(BSA_ERR_UNSUPPORTED, "fwd_fragment: problem too large (32-bit work item indices, 2^23 KV tiles per head)");
+    return BSA_OK;
+}
+
+size_t bsa_fwd_fragment_workspace_bytes(int B, int Hn, int64_t Sk, int D, int dtype) {
+    if ((dtype != BSA_BF16 && dtype != BSA_F16) || D != 128 || B <= 0 || Hn <= 0 || Sk <= 0 || Sk % 64 != 0) {
+        set_error(BSA_ERR_UNSUPPORTED, "fwd_fragment: bf16 / fp16, head dim 128, Sk a positive multiple of 64");
+        return 0;
+    }
+    const size_t one = ((size_t)B * Hn * (size_t)Sk * D * 2 + 255) & ~(size_t)255;
+    return 2 * one;
+}
+
+int bsa_fwd_fragment(const void* q, const void* k, const void* v, const int32_t* idx, const int32_t* lens,
+                     const uint64_t* tile_valid, void* o, float* lse, int B, int Hn, int64_t Sq, int64_t Sk, int D,
+                     int bs_q, int bs_k, int idx_stride, float sm_scale, int dtype, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+    if (!q || !k || !v || !lens || !o || !workspace || (!idx && idx_stride > 0)) return set_error(BSA_ERR_BAD_ARG, "fwd_fragment: null pointer");
+    BSA_TRY(check_fwd_fragment(q, k, v, idx, lens, o, B, Hn, Sq, Sk, D, bs_q, bs_k, idx_stride, sm_scale, dtype));
+    if (!(sm_scale > 0.f) || !std::isfinite(sm_scale)) return set_error(BSA_ERR_BAD_ARG, "fwd_fragment: sm_scale must be positive and finite");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return set_error(BSA_ERR_BAD_ARG, "fwd_fragment: q/k/v/o must be 16-byte aligned, the workspace 256-byte aligned");
+    const size_t need = bsa_fwd_fragment_workspace_bytes(B, Hn, Sk, D, dtype);
+    if (workspace_bytes < need) return set_error(BSA_ERR_WORKSPACE, "fwd_fragment: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+    // a blocked-order tensor is a (Sk / 64, 8, 8) grid cut into (1, 8, 8) chunks: tile i = rows 64 i .. 64 i + 63
+    const Grid3 g = make_grid((int)(Sk / 64), 8, 8, 1, 8, 8);
+    const int64_t kv_st[3] = {(int64_t)Hn * Sk * D, Sk * D, D};
+    const int64_t q_st[3] = {(int64_t)Hn * Sq * D, Sq * D, D};
+    char* kf = static_cast<char*>(workspace);
+    char* vf = kf + need / 2;
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = launch_frag(k, kv_st, kf, B, Hn, g, dtype, false, st);
+    if (e == hipSuccess) e = launch_frag(v, kv_st, vf, B, Hn, g, dtype, true, st);
+    if (e == hipSuccess)
+        e = launch_fwd_frag(q, kf, vf, idx, lens, tile_valid, o, lse, B, Hn, Sq, Sk, bs_q, bs_k, idx_stride, sm_scale, dtype, st,
+                            nullptr, q_st, q_st, Sq);
+    return e == hipSuccess ? BSA_OK : hip_fail(e, "fwd_fragment");
+}
+
 static int check_bwd_shape(int B, int Hn, int64_t Sq, int64_t Sk, int D, int bs_q, int bs_k, int dtype) {
     if (dtype != BSA_BF16 && dtype != BSA_F16) return set_error(BSA_ERR_UNSUPPORTED, "bwd: dtype %d is not built (bf16, fp16)", dtype);
     if (D != 128) return set_error(BSA_ERR_UNSUPPORTED, "bwd: head dim %d is not built (only 128)", D);

@@ -10,6 +10,7 @@
 #include <mutex>
 #include <shared_mutex>
 #include <tuple>
+#include <vector>
 
 namespace bsa {
 namespace {
@@ -255,11 +256,39 @@ struct LtState {
 };
 LtState& lt_state() { static LtState s; return s; }
 constexpr int kMaxLtDevices = 64;
+// A thread's handles go back to a per-device pool when the thread ends and are taken from there by the next thread
+// that needs one, so the number of handles ever created is bounded by the number of threads alive at one time, not
+// by the number of threads that ever called.  Nothing is destroyed: a thread may end while the HIP runtime is
+// being torn down, and the pool itself is never freed for the same reason.
+struct HandlePool {
+    std::mutex mu;
+    std::vector<hipblasLtHandle_t> idle[kMaxLtDevices];
+};
+HandlePool& handle_pool() { static HandlePool* p = new HandlePool; return *p; }
+struct ThreadHandles {
+    hipblasLtHandle_t h[kMaxLtDevices] = {};
+    ~ThreadHandles() {
+        HandlePool& pool = handle_pool();
+        std::lock_guard<std::mutex> lock(pool.mu);
+        for (int d = 0; d < kMaxLtDevices; ++d)
+            if (h[d]) pool.idle[d].push_back(h[d]);
+    }
+};
 hipblasLtHandle_t thread_handle(int device) {
-    thread_local hipblasLtHandle_t handles[kMaxLtDevices] = {};
+    thread_local ThreadHandles mine;
     if (device < 0 || device >= kMaxLtDevices) return nullptr;
-    if (!handles[device] && hipblasLtCreate(&handles[device]) != HIPBLAS_STATUS_SUCCESS) handles[device] = nullptr;
-    return handles[device];
+    if (!mine.h[device]) {
+        HandlePool& pool = handle_pool();
+        {
+            std::lock_guard<std::mutex> lock(pool.mu);
+            if (!pool.idle[device].empty()) {
+                mine.h[device] = pool.idle[device].back();
+                pool.idle[device].pop_back();
+            }
+        }
+        if (!mine.h[device] && hipblasLtCreate(&mine.h[device]) != HIPBLAS_STATUS_SUCCESS) mine.h[device] = nullptr;
+    }
+    return mine.h[device];
 }
 
 }  // namespace

@@ -23,6 +23,7 @@ from __future__ import annotations
 
 import ctypes as C
 import math
+import threading
 from typing import Optional, Sequence, Tuple
 
 import torch
@@ -58,6 +59,31 @@ def _rows_ok(t: torch.Tensor) -> torch.Tensor:
     es = t.element_size()
     ok = t.stride(3) == 1 and t.data_ptr() % 16 == 0 and all((t.stride(i) * es) % 16 == 0 for i in range(3))
     return t if ok else t.contiguous()
+
+
+_WORKSPACES: dict = {}
+
+
+def _workspace(nbytes: int, device: torch.device) -> torch.Tensor:
+    """The engine's scratch memory for a call on the current stream of `device`: one uint8 buffer per (device,
+    stream, host thread), grown when a call needs more and otherwise reused, so that a steady-state call allocates
+    nothing.  Calls that one thread enqueues on one stream run in order and may share a buffer; another stream or
+    another thread gets its own.  Under stream capture the buffer is a fresh allocation from the graph's own pool
+    (it then lives as long as the graph does, and a later regrowth here cannot pull it from under a replay)."""
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream, threading.get_ident())
+    buf = _WORKSPACES.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+        _WORKSPACES[key] = buf
+    return buf
+
+
+def release_workspaces() -> None:
+    """Drops the cached scratch buffers (they are re-created on demand)."""
+    _WORKSPACES.clear()
 
 
 def num_selected(sparsity: float, n_kv_blocks: int) -> int:
@@ -285,9 +311,11 @@ def get_select_indices_from_score(score, sparsity, cdf_threshold, sm_scale=None)
 # R5 / R6: the attention kernel on blocked-order tensors
 # ---------------------------------------------------------------------------
 def attn_fwd_bsa_varlen(q, k, v, sm_scale, block_indices, block_indices_lens, chunk_size_q, chunk_size_k,
-                        sparsity=None, tile_valid: Optional[torch.Tensor] = None):
+                        sparsity=None, tile_valid: Optional[torch.Tensor] = None, kernel: Optional[str] = None):
     """bsa_interface.py:290-341 (attn_fwd_bsa_varlen_triton).  Returns ``(o, lse)``
-    with ``lse`` the natural-log sum-exp, fp32 [B,H,S]."""
+    with ``lse`` the natural-log sum-exp, fp32 [B,H,S].  ``kernel``: "fragment" (bsa_fwd_fragment: the
+    operator's attention kernel, with k and v rewritten once into its operand order; bf16 / fp16, the default
+    for them) or "lds" (bsa_fwd: the LDS-tiled kernel, no workspace; the only one for fp32)."""
     _need_gpu(q, k, v, block_indices, block_indices_lens)
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
@@ -296,13 +324,25 @@ def attn_fwd_bsa_varlen(q, k, v, sm_scale, block_indices, block_indices_lens, ch
     idx = block_indices.to(torch.int32).contiguous()
     lens = block_indices_lens.to(torch.int32).contiguous()
     assert idx.shape[:3] == (B, H, Sq // chunk_size_q) and lens.shape == idx.shape[:3]
+    if kernel is None:
+        kernel = "lds" if q.dtype == torch.float32 or idx.shape[3] > 4096 else "fragment"
+    assert kernel in ("fragment", "lds")
     o = torch.empty_like(q)
     lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device)
     lib = _capi.load()
     with torch.cuda.device(q.device):
-        _capi.check(lib.bsa_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(idx), _ptr(lens), _ptr(tile_valid), _ptr(o), _ptr(lse),
-                                B, H, Sq, Sk, D, int(chunk_size_q), int(chunk_size_k), idx.shape[3],
-                                float(sm_scale), _code(q), _stream(q)), "bsa_fwd")
+        if kernel == "fragment":
+            need = lib.bsa_fwd_fragment_workspace_bytes(B, H, Sk, D, _code(q))
+            if need == 0:
+                raise NotImplementedError("bsa_fwd_fragment: " + _capi.last_error())
+            ws = _workspace(need, q.device)
+            _capi.check(lib.bsa_fwd_fragment(_ptr(q), _ptr(k), _ptr(v), _ptr(idx), _ptr(lens), _ptr(tile_valid), _ptr(o),
+                                             _ptr(lse), B, H, Sq, Sk, D, int(chunk_size_q), int(chunk_size_k), idx.shape[3],
+                                             float(sm_scale), _code(q), _ptr(ws), need, _stream(q)), "bsa_fwd_fragment")
+        else:
+            _capi.check(lib.bsa_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(idx), _ptr(lens), _ptr(tile_valid), _ptr(o), _ptr(lse),
+                                    B, H, Sq, Sk, D, int(chunk_size_q), int(chunk_size_k), idx.shape[3],
+                                    float(sm_scale), _code(q), _stream(q)), "bsa_fwd")
     return o, lse
 
 
@@ -331,7 +371,7 @@ def attn_bwd_bsa_varlen(do, q, k, v, o, dq, dk, dv, sm_scale, M, block_indices, 
     need = lib.bsa_bwd_workspace_bytes(B, H, Sq, Sk, D, int(chunk_size_q), int(chunk_size_k), idx.shape[3], _code(q))
     if need == 0:
         raise RuntimeError("bsa_bwd: " + lib.bsa_last_error().decode())
-    ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+    ws = _workspace(need, q.device)
     with torch.cuda.device(q.device):
         _capi.check(lib.bsa_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(idx), _ptr(lens),
                                 _ptr(tile_valid), _ptr(dq), _ptr(dk), _ptr(dv), B, H, Sq, Sk, D, int(chunk_size_q),
@@ -435,7 +475,7 @@ def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k,
     if need == 0:
         _capi.check(lib.bsa_fwd_3d(C.byref(prm), None, None, None, None, None, None, None, None, None, 0,
                                    None, None, None, None), "flash_attn_bsa_3d")
-    ws = None if static_scratch else torch.empty(need, dtype=torch.uint8, device=q.device)
+    ws = None if static_scratch else _workspace(need, q.device)
     o = torch.empty(B, H, Sq, D, dtype=q.dtype, device=q.device) if out is None else out
     assert o.shape == (B, H, Sq, D) and o.dtype == q.dtype and o.stride(3) == 1
     idx = lens = score = None

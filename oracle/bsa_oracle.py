@@ -360,7 +360,7 @@ def inverse_block_lists(idx: torch.Tensor, lens: torch.Tensor, n_kv_blocks: int)
 
 
 def blockwise_attention_backward(q, k, v, o, do, lse, idx, lens, bs_q: int, bs_k: int, sm_scale: float,
-                                 key_valid: Optional[torch.Tensor] = None):
+                                 key_valid: Optional[torch.Tensor] = None, q_blocks=None, kv_blocks=None):
     """Restatement of the reference backward's numerics (bsa:341-461; kernels vmask:288-360, 428-462, wrappers
     vmask:630-642, 943-945):
       M2 = lse * RCP_LN2 (fp32); k_s = k * (sm_scale * RCP_LN2) in k's dtype (one rounding, bsa:369-370);
@@ -371,6 +371,9 @@ def blockwise_attention_backward(q, k, v, o, do, lse, idx, lens, bs_q: int, bs_k
     dQ walks a row's blocks in list order, dK / dV walk the query blocks of a KV block in ascending order
     (bsa:389-392); fp32 summation order inside a product is free.  Padded keys (extension) have p = 0.  Lists name
     a block at most once (a selection does); the reference gives a repeated block no consistent meaning.
+    q_blocks / kv_blocks (optional, for problems too large to evaluate in full): only the dQ rows of these query
+    blocks and the dK / dV rows of these KV blocks are computed, each from all of its pairs; every other row of
+    the result stays zero.
     Returns (dq, dk, dv) in the input dtype."""
     B, H, Sq, D = q.shape
     Sk = k.shape[2]
@@ -383,7 +386,13 @@ def blockwise_attention_backward(q, k, v, o, do, lse, idx, lens, bs_q: int, bs_k
     dq = torch.zeros(B, H, Sq, D, dtype=torch.float32)
     dk = torch.zeros(B, H, Sk, D, dtype=torch.float32)
     dv = torch.zeros(B, H, Sk, D, dtype=torch.float32)
-    inv, inv_n = inverse_block_lists(idx, lens, nbk)
+    q_todo = range(nbq) if q_blocks is None else sorted(set(int(m) for m in q_blocks))
+    kv_todo = range(nbk) if kv_blocks is None else sorted(set(int(j) for j in kv_blocks))
+
+    def selectors(b, h, j):
+        """Query blocks of (b, h) whose list names KV block j, ascending (bsa:152-165 for one column)."""
+        live = torch.arange(idx.shape[-1]).unsqueeze(0) < lens[b, h].long().unsqueeze(1)
+        return torch.nonzero(((idx[b, h] == j) & live).any(dim=1)).flatten().tolist()
 
     def pair(b, h, m, j):
         qs = q[b, h, m * bs_q:(m + 1) * bs_q]
@@ -400,14 +409,13 @@ def blockwise_attention_backward(q, k, v, o, do, lse, idx, lens, bs_q: int, bs_k
 
     for b in range(B):
         for h in range(H):
-            for m in range(nbq):                                            # dQ: list order (vmask:469-499)
+            for m in q_todo:                                                # dQ: list order (vmask:469-499)
                 for i in range(int(lens[b, h, m])):
                     j = int(idx[b, h, m, i])
                     qs, ks, dos, p, ds = pair(b, h, m, j)
                     dq[b, h, m * bs_q:(m + 1) * bs_q] += ds.float() @ ks.float()
-            for j in range(nbk):                                            # dK, dV: ascending query blocks (vmask:327-356)
-                for i in range(int(inv_n[b, h, j])):
-                    m = int(inv[b, h, j, i])
+            for j in kv_todo:                                               # dK, dV: ascending query blocks (vmask:327-356)
+                for m in selectors(b, h, j):
                     qs, ks, dos, p, ds = pair(b, h, m, j)
                     dv[b, h, j * bs_k:(j + 1) * bs_k] += p.float().t() @ dos.float()
                     dk[b, h, j * bs_k:(j + 1) * bs_k] += ds.float().t() @ qs.float()

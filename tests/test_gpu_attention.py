@@ -22,11 +22,24 @@ def I():
     return bsa_interface
 
 
+KERNEL = {"name": None}
+
+
+@pytest.fixture(autouse=True, params=["fragment", "lds"])
+def attention_kernel(request):
+    """Every test that goes through run() is made with both attention kernels of the blocked-order boundary: the
+    operator's fragment-order kernel (bsa_fwd_fragment) and the LDS-tiled one (bsa_fwd).  fp32 has one kernel."""
+    KERNEL["name"] = request.param
+    yield request.param
+    KERNEL["name"] = None
+
+
 def run(q, k, v, idx, lens, bs_q=64, bs_k=64, scale=None, valid_bits=None):
     scale = 1 / math.sqrt(q.shape[-1]) if scale is None else scale
     tv = None if valid_bits is None else torch.from_numpy(valid_bits.view(np.int64)).cuda()
+    kern = None if q.dtype == torch.float32 else KERNEL["name"]
     o, lse = I().attn_fwd_bsa_varlen(q.cuda(), k.cuda(), v.cuda(), scale, idx.cuda(), lens.cuda(), bs_q, bs_k,
-                                     tile_valid=tv)
+                                     tile_valid=tv, kernel=kern)
     torch.cuda.synchronize()
     return o.cpu(), lse.cpu()
 
@@ -189,7 +202,8 @@ def test_480p_two_heads_sampled_rows():
 def test_thw_attention_equals_permute_attend_unpermute(latent, chunk):
     """attn_fwd_bsa_thw reads q/k/v and writes o/lse in (T,H,W) order; the blocked-order kernel between
     a permute and an unpermute (bsa_interface.py:650-659) must give the same result, also for lists
-    of different lengths (an empty one included) in arbitrary order.  The two routes run different kernels
+    of different lengths (an empty one included) in arbitrary order.  With the LDS-tiled kernel on the blocked-order
+    route the two routes run different kernels
     (one online softmax over 32-key steps on fragment-order K/V against two 32-key halves per tile merged at the
     end), so P is rounded to bf16 relative to different running maxima and the sums run in different orders: the results
     agree to a couple of bf16 ulps of the value rows (max-abs 1.6e-2, mean-abs 1e-3), like either against the oracle."""
@@ -208,13 +222,17 @@ def test_thw_attention_equals_permute_attend_unpermute(latent, chunk):
     kp, _, valid = bi._permute(k, latent, chunk, want_valid=True)
     vp, _, _ = bi._permute(v, latent, chunk)
     padded = any(a % c for a, c in zip(latent, chunk))
-    op, lse_p = bi.attn_fwd_bsa_varlen(qp, kp, vp, 0.11, idx, lens, bs, bs, tile_valid=valid if padded else None)
+    op, lse_p = bi.attn_fwd_bsa_varlen(qp, kp, vp, 0.11, idx, lens, bs, bs, tile_valid=valid if padded else None,
+                                       kernel=KERNEL["name"])
     grid = O.block_grid(latent, chunk)
     want = bi.rearrange_3d_block_to_THW(op, *grid, *chunk, 128, latent_shape=latent)
     want_lse = O.rearrange_3d_block_to_thw(lse_p.cpu().unsqueeze(-1), latent, chunk)[..., 0]
     got, lse = bi.attn_fwd_bsa_thw(q, k, v, latent, latent, chunk, chunk, idx, lens, sm_scale=0.11, return_lse=True)
     d = (got.float() - want.float()).abs()
     assert d.max() <= 1.6e-2 and d.mean() <= 1e-3, (float(d.max()), float(d.mean()))
+    if KERNEL["name"] == "fragment":
+        # the same kernel on both routes, reading q and writing o through a row table on one of them: the same bits
+        assert torch.equal(got, want) and torch.equal(lse.cpu(), want_lse)
     # rows of empty lists and their lse are exact on both routes
     assert torch.equal(got == 0, want == 0)
     assert torch.allclose(lse.cpu(), want_lse, atol=1e-4, rtol=1e-5)

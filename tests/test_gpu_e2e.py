@@ -192,6 +192,58 @@ def test_720p_full_shape_sampled():
     assert torch.equal(o, o2)
 
 
+def gpu_qkv(seed, heads, tokens):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return tuple(torch.randn(1, heads, tokens, 128, generator=g, device="cuda").bfloat16() for _ in range(3))
+
+
+def all_heads_properties(o, v_rows):
+    assert torch.isfinite(o.float()).all()
+    # a convex combination of value rows cannot leave their range, in any head
+    assert bool((o.float().abs().amax(dim=(0, 2, 3)) <= v_rows.float().abs().amax(dim=(0, 2, 3))).all())
+
+
+def test_480p_all_heads():
+    """benchmark configuration 2 at full size (32 heads, 37 440 tokens, 624 blocks, 39 kept): 19 968 work items are
+    19 full rounds of 1 024 and one of 512, and a head's 624 items never fill a round, so every round crosses a head
+    boundary.  All heads: finiteness, range, determinism; heads on both sides of round boundaries: the oracle on
+    sampled query blocks (the last block of a head and the first of the next lie in one round)."""
+    latent = (24, 30, 52)
+    q, k, v = gpu_qkv(1, 32, 37440)
+    o, idx, lens, score = I()._bsa_3d(q, k, v, latent, latent, 0.9375, (4, 4, 4), (4, 4, 4), True)
+    assert idx.shape == (1, 32, 624, 39) and torch.all(lens == 39)
+    all_heads_properties(o, v)
+    # item 1023 | 1024 is block 399 | 400 of head 1; item 19 455 | 19 456 (the half round begins) is block 111 | 112 of head 31
+    check_against_oracle(q.cpu(), k.cpu(), v.cpu(), latent, latent, 0.9375, o, idx, lens, score,
+                         q_blocks=[0, 111, 112, 399, 400, 623], heads=[0, 1, 31])
+    assert torch.equal(o, I().flash_attn_bsa_3d(q, k, v, latent, latent, sparsity=0.9375, **CH))
+
+
+def test_long_video_continuation_all_heads():
+    """benchmark configuration 4 at full size (32 heads, grid 48x30x52, 12 conditioning frames): both operator calls of
+    attention.py:124-135 into one output buffer - 32 x 312 work items of 39 tiles, then 32 x 936 of 156."""
+    T, Hh, W, cond = 48, 30, 52, 12
+    S, n = T * Hh * W, cond * Hh * W
+    q, k, v = gpu_qkv(3, 32, S)
+    out = torch.empty(1, S, 32, 128, dtype=torch.bfloat16, device="cuda").permute(0, 2, 1, 3)
+    bi = I()
+    call = lambda: (bi._bsa_3d(q[:, :, :n], k[:, :, :n], v[:, :, :n], (cond, Hh, W), (cond, Hh, W), 0.875, (4, 4, 4), (4, 4, 4), True,
+                               out=out[:, :, :n]),
+                    bi._bsa_3d(q[:, :, n:], k, v, (T - cond, Hh, W), (T, Hh, W), 0.875, (4, 4, 4), (4, 4, 4), True, out=out[:, :, n:]))
+    (_, idx_c, lens_c, score_c), (_, idx_n, lens_n, score_n) = call()
+    assert idx_c.shape == (1, 32, 312, 39) and idx_n.shape == (1, 32, 936, 156)
+    all_heads_properties(out, v)
+    first = out.clone()
+    heads = [0, 3, 31]               # item 1023 | 1024 of the conditioning call: block 87 | 88 of head 3; of the noise call: block 87 | 88 of head 1
+    qc, kc, vc = q.cpu(), k.cpu(), v.cpu()
+    check_against_oracle(qc[:, :, :n], kc[:, :, :n], vc[:, :, :n], (cond, Hh, W), (cond, Hh, W), 0.875,
+                         out[:, :, :n], idx_c, lens_c, score_c, q_blocks=[0, 87, 88, 311], heads=heads)
+    check_against_oracle(qc[:, :, n:], kc, vc, (T - cond, Hh, W), (T, Hh, W), 0.875,
+                         out[:, :, n:], idx_n, lens_n, score_n, q_blocks=[0, 87, 88, 935], heads=[1, 31])
+    call()
+    assert torch.equal(out, first)
+
+
 @pytest.mark.parametrize("sparsity", [None, 0.75])
 def test_operator_with_cdf_selection(sparsity):
     """flash_attn_bsa_3d with cdf_threshold (bsa_interface.py:268-277, 555): rows keep different numbers of

@@ -99,3 +99,25 @@ def test_finite_differences_on_a_tiny_case():
             args_m = {"q": (tm, k, v), "k": (q, tm, v), "v": (q, k, tm)}[which]
             fd = float((loss(*args_p) - loss(*args_m)) / (2 * eps))
             assert abs(float(grad[pos]) - fd) <= 2e-4 * max(1.0, abs(fd)), (which, pos, float(grad[pos]), fd)
+
+
+def test_block_subsets_equal_the_rows_of_the_full_evaluation():
+    """q_blocks / kv_blocks: the named rows bit for bit as in the full evaluation (same pairs, same order), every other
+    row zero; the query blocks of a KV block found column by column are those of inverse_block_lists."""
+    sm = 1 / math.sqrt(128)
+    q, k, v, do, idx, lens = case(6, 2, 7, 9, 4, torch.bfloat16)
+    mask = O.block_mask_from_indices(idx, lens, 9)
+    o32, lse = O.masked_dense_attention(q, k, v, mask, 64, 64, sm)
+    o = o32.bfloat16()
+    full = O.blockwise_attention_backward(q, k, v, o, do, lse, idx, lens, 64, 64, sm)
+    qb, kb = [0, 5, 6], [2, 8]
+    part = O.blockwise_attention_backward(q, k, v, o, do, lse, idx, lens, 64, 64, sm, q_blocks=qb, kv_blocks=kb)
+    rows = lambda blocks, n: torch.isin(torch.arange(n * 64) // 64, torch.tensor(blocks))
+    rq, rk = rows(qb, 7), rows(kb, 9)
+    assert torch.equal(part[0][:, :, rq], full[0][:, :, rq]) and torch.all(part[0][:, :, ~rq] == 0)
+    for got, want in ((part[1], full[1]), (part[2], full[2])):
+        assert torch.equal(got[:, :, rk], want[:, :, rk]) and torch.all(got[:, :, ~rk] == 0)
+    assert float(full[1][:, :, rk].abs().max()) > 0              # the sampled KV blocks were selected by someone
+    # an empty subset computes nothing
+    none = O.blockwise_attention_backward(q, k, v, o, do, lse, idx, lens, 64, 64, sm, q_blocks=[], kv_blocks=[])
+    assert all(torch.all(t == 0) for t in none)
