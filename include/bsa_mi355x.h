@@ -183,10 +183,10 @@ int bsa_fwd(const void* q, const void* k, const void* v, const int32_t* idx, con
  * rewritten once per call into the order its matrix instructions consume them): the same boundary -
  * attn_fwd_bsa_varlen_triton (bsa:290-341), kernel vmask:172-285 - the same arguments, results within the
  * rounding of another summation order, plus a workspace of bsa_fwd_fragment_workspace_bytes() bytes
- * (two copies of k's size), 256-byte aligned.  Padded key slots may hold anything finite: they are masked
+ * (two copies of k's size and two small tables), 256-byte aligned.  Padded key slots may hold anything finite: they are masked
  * by tile_valid.  idx_stride <= 4096.
  */
-size_t bsa_fwd_fragment_workspace_bytes(int B, int Hn, int64_t Sk, int D, int dtype);
+size_t bsa_fwd_fragment_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int D, int dtype);
 int bsa_fwd_fragment(const void* q, const void* k, const void* v, const int32_t* idx, const int32_t* lens,
                      const uint64_t* tile_valid, void* o, float* lse,
                      int B, int Hn, int64_t Sq, int64_t Sk, int D, int bs_q, int bs_k, int idx_stride,

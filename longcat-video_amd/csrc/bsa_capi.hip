@@ -248,13 +248,25 @@ static int check_fwd_fragment(const void* q, const void* k, const void* v, const
     return BSA_OK;
 }
 
-size_t bsa_fwd_fragment_workspace_bytes(int B, int Hn, int64_t Sk, int D, int dtype) {
-    if ((dtype != BSA_BF16 && dtype != BSA_F16) || D != 128 || B <= 0 || Hn <= 0 || Sk <= 0 || Sk % 64 != 0) {
-        set_error(BSA_ERR_UNSUPPORTED, "fwd_fragment: bf16 / fp16, head dim 128, Sk a positive multiple of 64");
+namespace {
+struct FragmentWs { size_t kv, norms, fallback, total; };
+FragmentWs fragment_ws(int B, int Hn, int64_t Sq, int64_t Sk, int D) {
+    auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
+    FragmentWs w;
+    w.kv = up((size_t)B * Hn * (size_t)Sk * D * 2);
+    w.norms = up(frag_key_norm_floats(B, Hn, Sk / 64) * sizeof(float));
+    w.fallback = up(frag_fallback_ints((int64_t)B * Hn * (Sq / 64)) * sizeof(int32_t));
+    w.total = 2 * w.kv + w.norms + w.fallback;       // K, V, key norms, the list of items left to the second kernel
+    return w;
+}
+}  // namespace
+
+size_t bsa_fwd_fragment_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int D, int dtype) {
+    if ((dtype != BSA_BF16 && dtype != BSA_F16) || D != 128 || B <= 0 || Hn <= 0 || Sq <= 0 || Sq % 64 != 0 || Sk <= 0 || Sk % 64 != 0) {
+        set_error(BSA_ERR_UNSUPPORTED, "fwd_fragment: bf16 / fp16, head dim 128, Sq and Sk positive multiples of 64");
         return 0;
     }
-    const size_t one = ((size_t)B * Hn * (size_t)Sk * D * 2 + 255) & ~(size_t)255;
-    return 2 * one;
+    return fragment_ws(B, Hn, Sq, Sk, D).total;
 }
 
 int bsa_fwd_fragment(const void* q, const void* k, const void* v, const int32_t* idx, const int32_t* lens,
@@ -266,20 +278,23 @@ int bsa_fwd_fragment(const void* q, const void* k, const void* v, const int32_t*
     if (!(sm_scale > 0.f) || !std::isfinite(sm_scale)) return set_error(BSA_ERR_BAD_ARG, "fwd_fragment: sm_scale must be positive and finite");
     if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return set_error(BSA_ERR_BAD_ARG, "fwd_fragment: q/k/v/o must be 16-byte aligned, the workspace 256-byte aligned");
-    const size_t need = bsa_fwd_fragment_workspace_bytes(B, Hn, Sk, D, dtype);
+    const FragmentWs fw = fragment_ws(B, Hn, Sq, Sk, D);
+    const size_t need = fw.total;
     if (workspace_bytes < need) return set_error(BSA_ERR_WORKSPACE, "fwd_fragment: workspace of %zu bytes, %zu needed", workspace_bytes, need);
     // a blocked-order tensor is a (Sk / 64, 8, 8) grid cut into (1, 8, 8) chunks: tile i = rows 64 i .. 64 i + 63
     const Grid3 g = make_grid((int)(Sk / 64), 8, 8, 1, 8, 8);
     const int64_t kv_st[3] = {(int64_t)Hn * Sk * D, Sk * D, D};
     const int64_t q_st[3] = {(int64_t)Hn * Sq * D, Sq * D, D};
     char* kf = static_cast<char*>(workspace);
-    char* vf = kf + need / 2;
+    char* vf = kf + fw.kv;
+    float* knorm = reinterpret_cast<float*>(vf + fw.kv);
+    int32_t* fallback = reinterpret_cast<int32_t*>(vf + fw.kv + fw.norms);
     hipStream_t st = (hipStream_t)stream;
-    hipError_t e = launch_frag(k, kv_st, kf, B, Hn, g, dtype, false, st);
+    hipError_t e = launch_frag(k, kv_st, kf, B, Hn, g, dtype, false, st, nullptr, nullptr, nullptr, knorm);
     if (e == hipSuccess) e = launch_frag(v, kv_st, vf, B, Hn, g, dtype, true, st);
     if (e == hipSuccess)
         e = launch_fwd_frag(q, kf, vf, idx, lens, tile_valid, o, lse, B, Hn, Sq, Sk, bs_q, bs_k, idx_stride, sm_scale, dtype, st,
-                            nullptr, q_st, q_st, Sq);
+                            nullptr, q_st, q_st, Sq, nullptr, nullptr, knorm, fallback);
     return e == hipSuccess ? BSA_OK : hip_fail(e, "fwd_fragment");
 }
 
@@ -333,7 +348,7 @@ struct Plan {
     bool cdf;
     bool direct_qo, direct_kv;
     bool frag;            // k and v are rewritten in fragment order for fwd_frag_kernel (bsa_fwd_frag.hip)
-    size_t off_qp, off_kp, off_vp, off_op, off_qc, off_kc, off_score, off_idx, off_idx_sorted, off_lens, off_valid, off_qrows, off_ktiles, off_order, off_queue, total;
+    size_t off_qp, off_kp, off_vp, off_op, off_qc, off_kc, off_score, off_idx, off_idx_sorted, off_lens, off_valid, off_qrows, off_ktiles, off_order, off_queue, off_knorm, off_fallback, total;
 };
 inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
@@ -388,6 +403,8 @@ int make_plan(const bsa_3d_params* p, Plan* pl, bool compact = false) {
     // lists of unequal length (the CDF rule): work items by descending length, and the counter they are drawn with
     pl->off_order = take(pl->cdf && pl->direct_qo ? bh * (size_t)(pl->Sqp / 64) * sizeof(int32_t) : 0);
     pl->off_queue = take(pl->cdf && pl->direct_qo ? 2 * sizeof(uint32_t) : 0);    // the counter and the choice of schedule
+    pl->off_knorm = take(pl->frag ? frag_key_norm_floats(p->B, p->Hn, pl->Skp / 64) * sizeof(float) : 0);   // key norms per head and tile
+    pl->off_fallback = take(pl->frag ? frag_fallback_ints((int64_t)bh * (pl->Sqp / 64)) * sizeof(int32_t) : 0);
     pl->total = off;
     return BSA_OK;
 }
@@ -405,6 +422,8 @@ struct Ws {
     int32_t *idx, *idx_sorted, *lens, *qrows, *order;
     uint32_t *ktiles, *queue;
     uint64_t* valid;
+    float* knorm;
+    int32_t* fallback;
 };
 int carve(const Plan& pl, void* workspace, size_t workspace_bytes, const char* who, Ws* w) {
     if (!workspace) return set_error(BSA_ERR_BAD_ARG, "%s: workspace is null", who);
@@ -422,6 +441,8 @@ int carve(const Plan& pl, void* workspace, size_t workspace_bytes, const char* w
     w->ktiles = pl.direct_kv ? reinterpret_cast<uint32_t*>(ws + pl.off_ktiles) : nullptr;
     w->order = pl.cdf && pl.direct_qo ? reinterpret_cast<int32_t*>(ws + pl.off_order) : nullptr;
     w->queue = pl.cdf && pl.direct_qo ? reinterpret_cast<uint32_t*>(ws + pl.off_queue) : nullptr;
+    w->knorm = pl.frag ? reinterpret_cast<float*>(ws + pl.off_knorm) : nullptr;
+    w->fallback = pl.frag ? reinterpret_cast<int32_t*>(ws + pl.off_fallback) : nullptr;
     return BSA_OK;
 }
 bool kv_padded(const bsa_3d_params* p) { return (p->Tk % p->tk) || (p->Hk % p->hk) || (p->Wk % p->wk); }
@@ -457,7 +478,7 @@ hipError_t prepare_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, cons
         // 64-slot chunks: one pass over k gives its fragment order, its chunk means and the validity words
         if (pl.gk.chunk() == 64) {
             e = launch_frag(k, k_strides, w.kp, p->B, p->Hn, pl.gk, p->dtype, false, st, pool ? w.kc : nullptr,
-                            padded_k ? w.valid : nullptr, trk);
+                            padded_k ? w.valid : nullptr, trk, w.knorm);
             if (e != hipSuccess) return e;
             return launch_frag(v, v_strides, w.vp, p->B, p->Hn, pl.gk, p->dtype, true, st);
         }
@@ -469,7 +490,7 @@ hipError_t prepare_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, cons
                 e = launch_permute(k, k_strides, nullptr, nullptr, w.valid, 1, 1, pl.gk, p->D, p->dtype, st);
             if (e != hipSuccess) return e;
         }
-        e = launch_frag(k, k_strides, w.kp, p->B, p->Hn, pl.gk, p->dtype, false, st);
+        e = launch_frag(k, k_strides, w.kp, p->B, p->Hn, pl.gk, p->dtype, false, st, nullptr, nullptr, nullptr, w.knorm);
         if (e != hipSuccess) return e;
         return launch_frag(v, v_strides, w.vp, p->B, p->Hn, pl.gk, p->dtype, true, st);
     }
@@ -489,7 +510,7 @@ hipError_t attention_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, co
     if (pl.frag)
         return launch_fwd_frag(q, w.kp, w.vp, idx, lens, kv_padded(p) ? w.valid : nullptr, o, lse, p->B, p->Hn, pl.Sqp, pl.Skp,
                                pl.gq.chunk(), pl.gk.chunk(), idx_stride, p->sm_scale, p->dtype, st, w.qrows, q_strides, o_strides,
-                               (int64_t)p->Tq * p->Hq * p->Wq, by_length ? w.order : nullptr, by_length ? w.queue : nullptr);
+                               (int64_t)p->Tq * p->Hq * p->Wq, by_length ? w.order : nullptr, by_length ? w.queue : nullptr, w.knorm, w.fallback);
     FwdLayout L;
     L.q_rows = w.qrows;
     L.k_tiles = w.ktiles;

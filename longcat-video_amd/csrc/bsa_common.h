@@ -146,6 +146,10 @@ void launch_schedule_choice(const int32_t* lens, int nbq, int tiles_per_block, i
 // the bits launch_permute's pooling gives) and the tile validity words; both optional.  dst may be null: the pass
 // then only reads (chunk means of q).
 // tr (optional, transpose = false only): per-head RMSNorm and / or 3-D RoPE of every row on its way through the pass.
+// key_norm (optional, transpose = false only, frag_key_norm_floats() floats): its first B*Hn entries receive the largest
+// Euclidean norm of a row of every (batch, head) as the pass writes it (a part in a thousand above), the rest is
+// the per-tile norms they are reduced from; launch_fwd_frag takes the first part to bound q . k.
+size_t frag_key_norm_floats(int B, int Hn, int64_t tiles);
 struct RowTransform {
     const void* norm_w;      // 128 norm weights in the storage type; null: no norm
     const float* tab;        // rotation table (the layout bsa_norm_rope reads); null: no rotation
@@ -157,14 +161,18 @@ struct RowTransform {
 };
 hipError_t launch_frag(const void* src, const int64_t strides[3], void* dst, int B, int Hn, const Grid3& g, int dtype,
                        bool transpose, hipStream_t st, void* pooled = nullptr, uint64_t* tile_valid = nullptr,
-                       const RowTransform* tr = nullptr);
+                       const RowTransform* tr = nullptr, float* key_norm = nullptr);
 // The attention kernel on fragment-order K and V.  q_rows (optional): token row of every blocked-order query
 // slot, -1 for padding; q_st / o_st: element strides {batch, head, row}; lse_rows: rows per (batch, head) of lse.
 hipError_t launch_fwd_frag(const void* q, const void* kf, const void* vf, const int32_t* idx, const int32_t* lens,
                            const uint64_t* tile_valid, void* o, float* lse, int B, int Hn, int64_t Sq, int64_t Sk,
                            int bs_q, int bs_k, int idx_stride, float sm_scale, int dtype, hipStream_t st,
                            const int32_t* q_rows, const int64_t q_st[3], const int64_t o_st[3], int64_t lse_rows,
-                           const int32_t* order = nullptr, uint32_t* queue = nullptr);
+                           const int32_t* order = nullptr, uint32_t* queue = nullptr, const float* key_norm = nullptr,
+                           int32_t* fallback = nullptr);
+// fallback (optional, frag_fallback_ints(B * Hn * Sq / 64) int32): with it and key_norm the rounds run the kernel that
+// takes no row maxima and list here the items whose logits it cannot bound; a last launch computes those.
+size_t frag_fallback_ints(int64_t items);
 
 
 // Backward of the blocked-order attention (bsa_bwd.hip), bf16 / fp16.  workspace: bwd_workspace_bytes() bytes.

@@ -44,6 +44,11 @@ __device__ inline void load_to_lds_16(const void* sbase, uint32_t voff, uint32_t
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
 }
+// The same with 4 bytes per lane: the LDS address is m0 + 4*lane.
+__device__ inline void load_to_lds_4(const void* sbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                 :: "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
 __device__ inline uint32_t lds_address(const void* p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
 }
@@ -58,6 +63,12 @@ __device__ inline s16x4 lds_read_tr16(const void* p) {
 // operands.  The compiler does not see that such a statement is an MFMA and adds no wait states behind it:
 // the code keeps every VALU access to these accumulators at least eight MFMAs (256 clocks) behind the MFMA
 // that writes them, or puts explicit s_nop there.
+// The register allocator sees such a statement as an ordinary instruction that is complete when issued.  If the
+// result were dead behind the last statement of a chain (a timing build that compiles the consumer out, say), the
+// allocator could hand the registers to something else - an address, a loaded value - while the MFMA, whose
+// passes run for another 32 clocks and more, still writes them: the new value is overwritten, and an overwritten
+// address is a memory fault.  mfma_chain_end() (below) costs no instruction and ties the accumulators as live up
+// to the place where it stands; every chain is closed with one, placed where the distance rule above holds.
 // kAgprB: the B operand (the Q fragment) lives in an AGPR.  The queries 32 .. 63 of a work item are kept there,
 // the queries 0 .. 31 in VGPRs, which balances the two register files (VGPR: S^T, P^T, the K ring, half of Q;
 // AGPR: the output accumulators, the V ring, the other half of Q).
@@ -81,6 +92,11 @@ __device__ inline void mfma_s(f32x16& acc, f16x8 a, f16x8 b) {
         else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
     }
 }
+
+// Marks the end of a chain of assembly MFMAs into `acc`: from here on the accumulators may be read, written or
+// reused.  Emits nothing; it only keeps `acc` allocated, and unchanged, between the chain's last MFMA and this
+// point, which the caller places at least eight MFMAs (or the equivalent s_nop) behind that MFMA.
+__device__ __forceinline__ void mfma_chain_end(f32x16& acc) { asm volatile("" : "+v"(acc)); }
 
 }  // namespace mfma
 }  // namespace bsa

@@ -50,7 +50,7 @@ SIGNATURES = {
     "bsa_score_cdf": (_i, [_p, _p, _p, _p, _p, _p] + [_i] * 5 + [_f, _f, _i, _i, _i, _p]),
     "bsa_cdf_from_score": (_i, [_p, _p, _p, _p] + [_i] * 4 + [_f, _f, _i, _i, _i, _p]),
     "bsa_fwd": (_i, [_p] * 8 + [_i, _i, _i64, _i64, _i, _i, _i, _i, _f, _i, _p]),
-    "bsa_fwd_fragment_workspace_bytes": (C.c_size_t, [_i, _i, _i64, _i, _i]),
+    "bsa_fwd_fragment_workspace_bytes": (C.c_size_t, [_i, _i, _i64, _i64, _i, _i]),
     "bsa_fwd_fragment": (_i, [_p] * 8 + [_i, _i, _i64, _i64, _i, _i, _i, _i, _f, _i, _p, C.c_size_t, _p]),
     "bsa_bwd_workspace_bytes": (C.c_size_t, [_i, _i, _i64, _i64, _i, _i, _i, _i, _i]),
     "bsa_bwd": (_i, [_p] * 12 + [_i, _i, _i64, _i64, _i, _i, _i, _i, _f, _i, _p, C.c_size_t, _p]),

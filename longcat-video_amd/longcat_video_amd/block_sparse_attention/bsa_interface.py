@@ -332,7 +332,7 @@ def attn_fwd_bsa_varlen(q, k, v, sm_scale, block_indices, block_indices_lens, ch
     lib = _capi.load()
     with torch.cuda.device(q.device):
         if kernel == "fragment":
-            need = lib.bsa_fwd_fragment_workspace_bytes(B, H, Sk, D, _code(q))
+            need = lib.bsa_fwd_fragment_workspace_bytes(B, H, Sq, Sk, D, _code(q))
             if need == 0:
                 raise NotImplementedError("bsa_fwd_fragment: " + _capi.last_error())
             ws = _workspace(need, q.device)
