@@ -35,8 +35,10 @@ WORKLOADS = {
     "c3": ((24, 45, 80), 0.9375, 2, True, "720p layer: 32 heads x 128, grid 24x45x80 (86400 tokens), density 1/16"),
 }
 ATTENTION_KERNEL = "fwd_frag_kernel<bf16> (all launches of one layer)"
-# what the attention kernel's traffic depends on: the kernel itself and the visiting order of the lists it walks
-ATTENTION_SOURCES = [os.path.join(ROOT, "longcat-video_amd", "csrc", f) for f in ("bsa_fwd_frag.hip", "bsa_select.hip")]
+# what the attention kernel's traffic depends on: the kernel and its helpers, the visiting order of the lists it walks,
+# and the layer that decides rounds per launch and whether the visiting order runs
+ATTENTION_SOURCES = [os.path.join(ROOT, "longcat-video_amd", "csrc", f)
+                     for f in ("bsa_fwd_frag.hip", "bsa_select.hip", "bsa_mfma.h", "bsa_common.h", "bsa_capi.hip")]
 
 
 def source_sha16(paths=ATTENTION_SOURCES):
@@ -69,6 +71,7 @@ def recorded_traffic(workload, summaries="bsa_operator_%s_*.md", sources=ATTENTI
 
 CHUNK = (4, 4, 4)
 HEADS, D = 32, 128
+DRAWN = {"host": "drawn in fp32 by torch's CPU generator (seeded) and moved to the GPU", "device": "drawn in fp32 by the GPU's generator (seeded)"}
 
 
 def kv_blocks(latent):
@@ -80,12 +83,18 @@ def operator_lists(I, idx_score_order, lens, latent_k):
     return I.visit_order(idx_score_order.sort(dim=-1).values.int().contiguous(), lens, kv_blocks(latent_k))
 
 
-def make_inputs(torch, latent, seed, rms):
+def make_inputs(torch, latent, seed, rms, where="device"):
+    """q, k, v ~ N(0, 1) in fp32 from one seeded generator, q and k optionally RMS-normalised per head, cast to bf16.
+    where = "host": drawn by torch's CPU generator (the same numbers on every machine) and moved to the GPU;
+    "device": drawn by the GPU's generator (seconds faster; used for the side figures)."""
     S = latent[0] * latent[1] * latent[2]
-    g = torch.Generator(device="cuda").manual_seed(seed)
+    g = torch.Generator(device="cuda" if where == "device" else "cpu").manual_seed(seed)
     out = []
     for i in range(3):
-        x = torch.randn(1, HEADS, S, D, generator=g, device="cuda")
+        if where == "device":
+            x = torch.randn(1, HEADS, S, D, generator=g, device="cuda")
+        else:
+            x = torch.randn(1, HEADS, S, D, generator=g).cuda()
         if rms and i < 2:
             x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6)
         out.append(x.bfloat16())
@@ -201,13 +210,13 @@ def attention_roofline(flop, ms, workload, coherent=False):
             "traffic": None if coherent else recorded_traffic(workload), "ms": round(ms, 4)}
 
 
-def run_c4(torch, args):
-    """benchmark configuration 4: long-video continuation, grid 48x30x52 with 12 conditioning frames.  Two operator
-    calls per layer as in attention.py:124-135, writing into one output buffer."""
+def measure_c4(torch, steps, warmup, settle, where):
+    """Both operator calls of configuration 4 (attention.py:124-135) into one output buffer: ms per layer of the operator
+    and of its attention kernel alone (the operator's own lists; its output is asserted to be reproduced)."""
     from longcat_video_amd.block_sparse_attention import bsa_interface as I
     T, Hh, W, cond = 48, 30, 52, 12
     S, n = T * Hh * W, cond * Hh * W
-    q, k, v = make_inputs(torch, (T, Hh, W), 3, False)
+    q, k, v = make_inputs(torch, (T, Hh, W), 3, False, where)
     out = torch.empty(1, S, HEADS, D, dtype=torch.bfloat16, device="cuda").permute(0, 2, 1, 3)
     calls = [((q[:, :, :n], k[:, :, :n], v[:, :, :n]), (cond, Hh, W), (cond, Hh, W), out[:, :, :n]),
              ((q[:, :, n:], k, v), (T - cond, Hh, W), (T, Hh, W), out[:, :, n:])]
@@ -215,14 +224,14 @@ def run_c4(torch, args):
     def step():
         for (a, b, c), lq, lk, o in calls:
             I._bsa_3d(a, b, c, lq, lk, 0.875, CHUNK, CHUNK, out=o)
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms = (time.perf_counter() - t0) * 1e3 / steps
     want = out.clone()
     # the attention kernel of both calls on its own, with the operator's lists
     ms_attn = 0.0
@@ -230,16 +239,72 @@ def run_c4(torch, args):
         _, idx, lens, _ = I._bsa_3d(a, b, c, lq, lk, 0.875, CHUNK, CHUNK, want_selection=True)
         idx = operator_lists(I, idx, lens, lk)
         attend = I.ThwAttention(b, c, lq, lk, CHUNK, CHUNK)
-        ms_attn += time_events(torch, lambda: attend(a, idx, lens, out=o), max(args.steps, 20), 5, settle_s=args.settle)
+        ms_attn += time_events(torch, lambda: attend(a, idx, lens, out=o), max(steps, 20), 5, settle_s=settle)
         del attend
     assert torch.equal(out, want), "the separately timed attention kernel must reproduce the operator's output"
+    pairs = HEADS * (312 * 39 + 936 * 156)
+    return ms, ms_attn, pairs, (T, Hh, W, cond, S, n)
+
+
+def measure_operator(torch, workload, steps, warmup, settle, where, coherent=False):
+    """One of the single-call workloads: ms per layer of the whole operator over exactly `steps` timed calls, and of its
+    attention kernel alone exactly as the operator runs it (same lists in the same visiting order, same (T, H, W)
+    addressing, workspace prepared outside the timed region; its output is asserted equal to the operator's)."""
+    from longcat_video_amd.block_sparse_attention import bsa_interface as I
+    latent, sparsity, seed, rms, desc = WORKLOADS[workload]
+    q, k, v = make_coherent_inputs(torch, latent, seed) if coherent else make_inputs(torch, latent, seed, rms, where)
+    prm = dict(sparsity=sparsity, chunk_3d_shape_q=list(CHUNK), chunk_3d_shape_k=list(CHUNK))
+    for _ in range(warmup):
+        I.flash_attn_bsa_3d(q, k, v, latent, latent, **prm)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        o = I.flash_attn_bsa_3d(q, k, v, latent, latent, **prm)
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / steps
+    _, idx_score, lens, _ = I._bsa_3d(q, k, v, latent, latent, sparsity, CHUNK, CHUNK, want_selection=True)
+    idx = operator_lists(I, idx_score, lens, latent)
+    del idx_score
+    attend = I.ThwAttention(k, v, latent, latent, CHUNK, CHUNK)
+    o_buf = torch.empty_like(q)
+    ms_attn = time_events(torch, lambda: attend(q, idx, lens, out=o_buf), max(steps, 20), max(warmup, 5), settle_s=settle)
+    assert torch.equal(o_buf, o), "the separately timed attention kernel must reproduce the operator's output"
+    del attend, o_buf, o
+    return ms_step, ms_attn, idx.shape[2], idx.shape[3], (q, k, v)
+
+
+def other_configurations(torch, args):
+    """The attention kernel (and the operator around it) at the other operator configurations, for the default line:
+    a few seconds of GPU time each, inputs drawn on the device, no CPU leg."""
+    out = {}
+    ms_step, ms_attn, nbq, k_sel, qkv = measure_operator(torch, "c2", 10, 3, args.settle, "device")
+    del qkv
+    flop = HEADS * nbq * k_sel * 4 * 64 * 64 * D
+    out["c2"] = {"workload": WORKLOADS["c2"][4], "operator_ms": round(ms_step, 4), "attention_ms": round(ms_attn, 4),
+                 "attention_tflops": round(flop / ms_attn / 1e9, 1), "attention_frac_of_bf16_peak": round(flop / ms_attn / 1e9 / PEAK_BF16_TFLOPS, 4),
+                 "block_pairs": HEADS * nbq * k_sel}
+    torch.cuda.empty_cache()
+    ms, ms_attn, pairs, _ = measure_c4(torch, 5, 2, args.settle, "device")
+    flop = pairs * 4 * 64 * 64 * D
+    out["c4"] = {"workload": "32 heads x 128, grid 48x30x52 (74880 tokens), 12 conditioning frames, density 1/8, two operator calls",
+                 "operator_ms": round(ms, 4), "attention_ms": round(ms_attn, 4), "attention_tflops": round(flop / ms_attn / 1e9, 1),
+                 "attention_frac_of_bf16_peak": round(flop / ms_attn / 1e9 / PEAK_BF16_TFLOPS, 4), "block_pairs": pairs}
+    torch.cuda.empty_cache()
+    return out
+
+
+def run_c4(torch, args):
+    """benchmark configuration 4: long-video continuation, grid 48x30x52 with 12 conditioning frames.  Two operator
+    calls per layer as in attention.py:124-135, writing into one output buffer."""
+    from longcat_video_amd.block_sparse_attention import bsa_interface as I
+    ms, ms_attn, pairs, (T, Hh, W, cond, S, n) = measure_c4(torch, args.steps, args.warmup, args.settle, args.inputs)
     pairs = HEADS * (312 * 39 + 936 * 156)
     flop = pairs * 4 * 64 * 64 * D
     result = {
         "metric": "BSA fwd ms/layer + sparse TFLOPS, long-video continuation (cond/noise split)", "value": round(flop / ms / 1e9, 2),
         "unit": "TFLOP/s (sparse-actual, both operator calls)", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic N(0,1) q/k/v, seeded on the GPU",
+        "data": "synthetic N(0,1) q/k/v, " + DRAWN[args.inputs],
         "config": {"workload": "c4: 32 heads x 128, grid 48x30x52 (74880 tokens), 12 conditioning frames, density 1/8",
                    "block_pairs": pairs},
         "pct_of_bf16_peak_whole_operator": round(100 * flop / ms / 1e9 / PEAK_BF16_TFLOPS, 2),
@@ -269,7 +334,7 @@ def run_bwd(torch, args):
     scaled k, bit matrix, seven fragment-order passes, dQ kernel, dK/dV kernel); the forward is not in it."""
     from longcat_video_amd.block_sparse_attention import bsa_interface as I
     latent, sparsity, seed, rms, desc = WORKLOADS["c3"]
-    q, k, v = make_inputs(torch, latent, seed, rms)
+    q, k, v = make_inputs(torch, latent, seed, rms, args.inputs)
     qp, kp, vp = (I._permute(t, latent, CHUNK)[0] for t in (q, k, v))
     del q, k, v
     sm = 1 / math.sqrt(D)
@@ -295,7 +360,7 @@ def run_bwd(torch, args):
         "metric": "BSA bwd ms/layer + TFLOPS at 720p 86.4k tokens (blocked order)", "value": round(tflops, 2),
         "unit": "TFLOP/s (seven 64x64x128 products per selected block pair)", "n_gpus": 1, "steps": steps, "warmup": min(args.warmup, 2),
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic N(0,1) q/k/v with per-head RMS-normalised q/k and N(0,1) output gradient, seeded on the GPU",
+        "data": "synthetic N(0,1) q/k/v with per-head RMS-normalised q/k, " + DRAWN[args.inputs] + "; N(0,1) output gradient drawn on the GPU",
         "config": {"workload": "bwd: backward of the c3 layer in blocked order, 32 heads x 128, 1440 x 1440 blocks of 64, 90 per row",
                    "block_pairs": pairs},
         "roofline": {"kernel": "bwd_dq_lds_kernel<bf16> + bwd_dkdv_kernel<bf16> (with the passes before them)", "bound": "mfma",
@@ -318,6 +383,22 @@ def run_bwd(torch, args):
                                        64, 64, sm)
         sec = time.perf_counter() - t0
         layer_s = sec * pairs / (nq * idx.shape[3])
+        # the checker's other job in this leg: the timed call's own gradients against the oracle on sampled blocks of
+        # the first head (all pairs of three query blocks; every query block that selected two KV blocks)
+        one = lambda t: t[:, :1].cpu()
+        nb = idx.shape[2]
+        counts = torch.bincount(idx[0, 0].flatten().long(), minlength=nb).cpu()
+        qb, kb = [0, nb // 2, nb - 1], [int(counts.argmax()), int(counts.argmin())]
+        wq, wk, wv = O.blockwise_attention_backward(one(qp), one(kp), one(vp), one(o), one(do), one(lse), one(idx).long(), one(lens),
+                                                    64, 64, sm, q_blocks=qb, kv_blocks=kb)
+        rows = lambda blocks: torch.cat([torch.arange(64 * b, 64 * b + 64) for b in blocks])
+        worst = 0.0
+        for got, want, r in ((dq, wq, rows(qb)), (dk, wk, rows(kb)), (dv, wv, rows(kb))):
+            g, w = one(got)[:, :, r].float(), want[:, :, r].float()
+            err = float((g - w).abs().max()) / max(float(w.abs().max()), 1e-30)
+            assert err <= 4 * 2.0 ** -7, "sampled gradient blocks differ from the oracle (%.3g of the largest entry)" % err
+            worst = max(worst, err)
+        result["sampled_parity"] = {"query_blocks": qb, "kv_blocks": kb, "max_error_over_largest_entry": round(worst, 6), "bound": 4 * 2.0 ** -7}
         result["cpu_baseline"] = {
             "value": round(flop / layer_s / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port", "ms_per_layer": round(layer_s * 1e3, 1),
             "sample": "1 of %d heads, inputs drawn on the host from the same distribution (a separate draw): the oracle's backward "
@@ -460,6 +541,11 @@ def main():
                     help="seconds of warm-up, and at least as many of timing, for the kernel-alone measurements (0: fixed "
                          "call counts, for runs under a profiler whose per-dispatch averages must weigh every call alike)")
     ap.add_argument("--no-gemm-tuning", action="store_true", help="c5: leave the GEMM algorithm choice to hipBLASLt's first proposal")
+    ap.add_argument("--inputs", default="host", choices=["host", "device"],
+                    help="where q, k, v of the timed workload are drawn: torch's CPU generator (the same numbers on every "
+                         "machine; half a minute at 720p) or the GPU's")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="c3: leave out the attention-kernel figures of c2 and c4 that the default line carries beside its own")
     ap.add_argument("--data", default="random", choices=["random", "coherent"],
                     help="random (the benchmark's definition) or spatially coherent q/k (c2, c3 only; no CPU baseline)")
     args = ap.parse_args()
@@ -481,32 +567,9 @@ def main():
         return run_bwd(torch, args)
     latent, sparsity, seed, rms, desc = WORKLOADS[args.workload]
     coherent = args.data == "coherent"
-    q, k, v = make_coherent_inputs(torch, latent, seed) if coherent else make_inputs(torch, latent, seed, rms)
-    prm = dict(sparsity=sparsity, chunk_3d_shape_q=list(CHUNK), chunk_3d_shape_k=list(CHUNK))
-
-    # ---- whole operator: warm-up, then exactly K timed steps between synchronisations ----
-    for _ in range(args.warmup):
-        I.flash_attn_bsa_3d(q, k, v, latent, latent, **prm)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        o = I.flash_attn_bsa_3d(q, k, v, latent, latent, **prm)
-    torch.cuda.synchronize()
-    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
-
-    # ---- per-kernel timing with events on the launch stream ----
-    # the attention kernel exactly as the operator runs it: same lists in the same visiting order, same
-    # THW-order addressing, workspace prepared once outside the timed region
-    _, idx_score, lens, _ = I._bsa_3d(q, k, v, latent, latent, sparsity, CHUNK, CHUNK, want_selection=True)
-    idx = operator_lists(I, idx_score, lens, latent)
-    del idx_score
-    nbq, k_sel = idx.shape[2], idx.shape[3]
+    # ---- whole operator: warm-up, then exactly K timed steps between synchronisations; then the attention kernel alone
+    ms_step, ms_attn, nbq, k_sel, (q, k, v) = measure_operator(torch, args.workload, args.steps, args.warmup, args.settle, args.inputs, coherent)
     ksteps, kwarm = max(args.steps, 20), max(args.warmup, 5)      # kernels alone: enough calls for a steady clock
-    attend = I.ThwAttention(k, v, latent, latent, CHUNK, CHUNK)
-    o_buf = torch.empty_like(q)
-    ms_attn = time_events(torch, lambda: attend(q, idx, lens, out=o_buf), ksteps, kwarm, settle_s=args.settle)
-    assert torch.equal(o_buf, o), "the separately timed attention kernel must reproduce the operator's output"
-    del attend, o_buf
     # the other entry points on their own (the permutes are no longer part of the operator for bf16)
     qp, q_cmp, _ = I._permute(q, latent, CHUNK, want_pooled=True)
     _, k_cmp, _ = I._permute(k, latent, CHUNK, want_pooled=True)
@@ -535,7 +598,7 @@ def main():
         "dtype": "bf16",
         "data": ("synthetic, spatially coherent q = k (smooth in the grid position + noise, RMS-normalised), random v, seeded on the GPU"
                  if coherent else
-                 "synthetic N(0,1) q/k/v%s, seeded on the GPU" % (" with per-head RMS-normalised q/k" if rms else "")),
+                 "synthetic N(0,1) q/k/v%s, %s" % (" with per-head RMS-normalised q/k" if rms else "", DRAWN[args.inputs])),
         "config": {"workload": "%s: %s" % (args.workload, desc), "chunk": list(CHUNK), "kv_blocks": nbk, "k_sel": k_sel,
                    "block_pairs": pairs, "padded_tokens": Sp},
         "ms_per_layer": round(ms_step, 4),
@@ -547,7 +610,10 @@ def main():
         "permute_gbs": round(permute_bytes / (ms_permute * 1e-3) / 1e9, 1),
         "roofline": attention_roofline(flop, ms_attn, args.workload, coherent),
     }
-    del o
+    del q, k, v, qp, q_cmp, k_cmp
+    torch.cuda.empty_cache()
+    if args.workload == "c3" and not coherent and not args.no_other_configs:
+        result["other_configs"] = other_configurations(torch, args)
     if not args.no_cpu_baseline and not coherent:
         result["cpu_baseline"] = cpu_baseline(torch, latent, sparsity, seed, rms, args.cpu_seconds)
     print(json.dumps(result))

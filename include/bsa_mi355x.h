@@ -37,7 +37,8 @@ typedef enum bsa_status {
     BSA_ERR_UNSUPPORTED = -2,    /* dtype / head_dim / chunk size not built */
     BSA_ERR_SHAPE = -3,          /* sizes inconsistent with each other */
     BSA_ERR_WORKSPACE = -4,      /* workspace smaller than bsa_workspace_bytes() */
-    BSA_ERR_HIP = -5             /* a HIP call failed; text in bsa_last_error() */
+    BSA_ERR_HIP = -5,            /* a HIP call failed; text in bsa_last_error() */
+    BSA_ERR_BUSY = -6            /* bsa_fwd_3d_static: the built-in scratch buffer is still in use by a call on another stream */
 } bsa_status;
 
 typedef enum bsa_dtype {
@@ -268,8 +269,11 @@ int bsa_bwd(const void* q, const void* k, const void* v, const void* o, const vo
  *   - The call itself makes no hipMalloc / hipFree and calls no allocating library routine.  The first call
  *     on a device looks up the buffer's address (hipGetSymbolAddress); make that call outside graph capture.
  *   - All calls on one GPU share the one buffer, which keeps the previous call's contents; nothing in it
- *     needs to start at zero.  Calls that overlap in time on one GPU (different streams, different threads)
- *     race on it and give wrong results: serialise them, or use bsa_fwd_3d with one workspace per stream.
+ *     needs to start at zero.  Calls that overlap in time on one GPU would race on it: serialise them, or use
+ *     bsa_fwd_3d with one workspace per stream.  A call made while the previous call on the same GPU, enqueued
+ *     on ANOTHER stream, has not finished is refused with BSA_ERR_BUSY and launches nothing (an event recorded
+ *     behind every call is queried; calls on one stream run in order and are never refused).  Under stream
+ *     capture nothing is recorded or queried: replays of graphs that hold such calls are the caller's to order.
  */
 #define BSA_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
 int bsa_fwd_3d_static(const bsa_3d_params* p,
@@ -356,8 +360,9 @@ int bsa_norm_rope(const void* src, const int64_t src_strides[3], void* dst, cons
 
 /* out[M,N] = x[M,K] . w[N,K]^T (+ bias[N]) (+ residual[M,N]), bf16 in/out, fp32 accumulate, on MFMA
  * through hipBLASLt.  Replaces the nn.Linear calls attention.py:111 and :142.  `workspace`: at least
- * 64 MiB of device memory (BSA_ERR_WORKSPACE otherwise); its contents do not matter.  Creates one
- * process-wide hipBLASLt handle on first use. */
+ * 64 MiB of device memory (BSA_ERR_WORKSPACE otherwise); its contents do not matter.  Every calling thread
+ * uses a hipBLASLt handle of its own per device; a thread that ends hands its handles to the next thread that
+ * needs one, so their number stays at the largest number of threads that called at one time. */
 int bsa_linear_bf16(const void* x, const void* w, const void* bias, const void* residual, void* out,
                     int64_t M, int N, int K, void* workspace, size_t workspace_bytes, void* stream);
 
@@ -415,7 +420,7 @@ int bsa_fwd_3d_qknorm(const bsa_3d_params* p, const bsa_qk_norm* n, const void* 
 /* The engine's own GEMM for the two projections of the attention module (attention.py:111 and :142):
  * out[M,N] = x[M,K] . w[N,K]^T (+ bias[N]) (+ residual[M,N]), bf16 in/out, fp32 accumulation on MFMA, one
  * rounding at the end.  Row strides in elements (ldx, ldw >= K; ldo, ldr >= N; multiples of 8).  N must be a
- * multiple of 128 and K of 32; x, w, out, residual 16-byte aligned.  Needs no workspace and allocates nothing. */
+ * multiple of 128 and K of 64; x, w, out, residual 16-byte aligned.  Needs no workspace and allocates nothing. */
 int bsa_gemm_bf16(const void* x, int64_t ldx, const void* w, int64_t ldw, const void* bias, const void* residual,
                   int64_t ldr, void* out, int64_t ldo, int64_t M, int N, int K, void* stream);
 

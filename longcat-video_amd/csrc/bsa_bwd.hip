@@ -26,6 +26,8 @@
 // the reference.
 #include "bsa_mfma.h"
 
+#include <atomic>
+
 namespace bsa {
 namespace {
 
@@ -634,6 +636,11 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
 
 }  // namespace
 
+constexpr size_t kBwdLdsLimit = 160 * 1024;
+// LDS of the dK / dV kernel for nbq query blocks: its stages, then the list of a KV block's query blocks
+size_t bwd_dkdv_lds_bytes(int nbq) { return (size_t)kBwdStages * kBwdStage + (size_t)nbq * sizeof(int32_t); }
+int bwd_max_query_blocks() { return (int)((kBwdLdsLimit - (size_t)kBwdStages * kBwdStage) / sizeof(int32_t)); }
+
 // Workspace of the backward, in bytes: k_s in blocked order, delta and M2, the bit matrix, the lists in the dQ kernel's visiting
 // order, per KV block its number of query blocks, the KV tiles of every head by that number.
 size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride) {
@@ -689,21 +696,28 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
 
     const dim3 block(64);
     // the dK / dV kernel's LDS: four stages of half a Q tile, half a dO tile and the queries' M2 / delta, then a KV block's query blocks
-    const size_t lds = (size_t)kBwdStages * kBwdStage + (size_t)nbq * sizeof(int32_t);
-    if (lds > 160 * 1024) return hipErrorInvalidValue;
+    const size_t lds = bwd_dkdv_lds_bytes(nbq);
+    if (lds > kBwdLdsLimit) return hipErrorInvalidValue;          // the C-ABI layer has rejected such a shape already
     const bool masked = tile_valid != nullptr;
-    const void* dkdv = dtype == BSA_BF16
-                           ? (masked ? reinterpret_cast<const void*>(bwd_dkdv_kernel<__bf16, true>) : reinterpret_cast<const void*>(bwd_dkdv_kernel<__bf16, false>))
-                           : (masked ? reinterpret_cast<const void*>(bwd_dkdv_kernel<_Float16, true>)
-                                     : reinterpret_cast<const void*>(bwd_dkdv_kernel<_Float16, false>));
-    if ((e = hipFuncSetAttribute(dkdv, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess) return e;
+    // Per device, once: the four dK / dV instantiations may use all of the LDS, and the number of compute units.
+    static std::atomic<int> device_cus[64];
+    int dev = 0;
+    if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+    if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+    int cus = device_cus[dev].load(std::memory_order_acquire);
+    if (cus == 0) {
+        const void* kernels[4] = {reinterpret_cast<const void*>(bwd_dkdv_kernel<__bf16, true>), reinterpret_cast<const void*>(bwd_dkdv_kernel<__bf16, false>),
+                                  reinterpret_cast<const void*>(bwd_dkdv_kernel<_Float16, true>), reinterpret_cast<const void*>(bwd_dkdv_kernel<_Float16, false>)};
+        for (const void* kf : kernels)
+            if ((e = hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBwdLdsLimit)) != hipSuccess) return e;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        device_cus[dev].store(cus, std::memory_order_release);   // threads racing here set the same attributes
+    }
     const dim3 grid_k((unsigned)(bh * (Sk / kTile)));
     // dQ: rounds of as many wavefronts as the device runs at once (one per SIMD), two rounds per launch.  The dK / dV
     // kernel runs as one grid, longest list first: its lists (the query blocks of a KV block) differ in length, and
     // rounds that wait for the longest list cost more than they bring.
-    int cus = 256, dev = 0;
-    if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    const int round = 4 * (cus > 0 ? cus : 256), span = 2 * round;
+    const int round = 4 * cus, span = 2 * round;
     const int total_q = (int)(bh * (Sq / kTile)), total_k = (int)(bh * (Sk / kTile));
     if (dtype == BSA_BF16) {
         for (int first = 0; first < total_q; first += span) {

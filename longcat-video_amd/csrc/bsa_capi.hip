@@ -3,6 +3,7 @@
 #include "bsa_common.h"
 
 #include <atomic>
+#include <mutex>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -310,6 +311,9 @@ static int check_bwd_shape(int B, int Hn, int64_t Sq, int64_t Sk, int D, int bs_
         return set_error(BSA_ERR_SHAPE, "bwd: Sq=%lld / Sk=%lld are not multiples of the chunk sizes %d / %d", (long long)Sq, (long long)Sk, bs_q, bs_k);
     if ((Sq / 32) * (int64_t)B * Hn > 0x7fffffffLL || (Sk / 32) * (int64_t)B * Hn > 0x7fffffffLL)
         return set_error(BSA_ERR_UNSUPPORTED, "bwd: problem too large (32-bit work item indices)");
+    if (Sq / bs_q > bwd_max_query_blocks())
+        return set_error(BSA_ERR_UNSUPPORTED, "bwd: %lld query blocks exceed the %d whose list the dK / dV kernel can hold in LDS",
+                         (long long)(Sq / bs_q), bwd_max_query_blocks());
     return BSA_OK;
 }
 
@@ -659,6 +663,15 @@ constexpr size_t kStaticScratchBytes = BSA_STATIC_SCRATCH_BYTES;
 __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 constexpr int kMaxDevices = 64;
 std::atomic<void*> g_scratch_ptr[kMaxDevices];
+// Per device: an event recorded behind the last call that used the buffer, and the stream of that call.  A call on
+// another stream while that event is pending would race on the buffer and is refused.
+struct StaticUse {
+    std::mutex mu;
+    hipEvent_t done = nullptr;
+    hipStream_t stream = nullptr;
+    bool pending = false;
+};
+StaticUse g_static_use[kMaxDevices];
 
 int static_scratch(void** out) {
     int dev = -1;
@@ -724,10 +737,39 @@ int bsa_fwd_3d_static(const bsa_3d_params* p, const void* q, const int64_t q_str
                          "use bsa_fwd_3d with a workspace of bsa_workspace_bytes()", pl.total, kStaticScratchBytes);
     void* ws = nullptr;
     BSA_TRY(static_scratch(&ws));
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return set_error(BSA_ERR_HIP, "fwd_3d_static: hipGetDevice");
+    StaticUse& use = g_static_use[dev];
+    std::lock_guard<std::mutex> lock(use.mu);          // two host threads enqueue one after the other
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing((hipStream_t)stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone;
+    if (!capturing) {
+        if (use.done == nullptr && hipEventCreateWithFlags(&use.done, hipEventDisableTiming) != hipSuccess) {
+            use.done = nullptr;
+            return set_error(BSA_ERR_HIP, "fwd_3d_static: hipEventCreateWithFlags");
+        }
+        if (use.pending && use.stream != (hipStream_t)stream) {
+            const hipError_t q_state = hipEventQuery(use.done);
+            (void)hipGetLastError();                   // "not ready" is an answer, not a failure to be found later
+            if (q_state == hipErrorNotReady)
+                return set_error(BSA_ERR_BUSY, "fwd_3d_static: the built-in scratch buffer is in use by a call on another stream; "
+                                 "wait for it, or use bsa_fwd_3d with a workspace per stream");
+        }
+    }
     // Nothing in the buffer has to start at zero: every piece is written by the kernel sequence before it is
     // read (the work counter of the queue schedule is cleared by a fill kernel inside launch_fwd).
-    return fwd_3d_impl(pl, p, q, q_strides, k, k_strides, v, v_strides, o, o_strides, ws, kStaticScratchBytes, idx_out,
-                       lens_out, score_out, stream);
+    const int rc = fwd_3d_impl(pl, p, q, q_strides, k, k_strides, v, v_strides, o, o_strides, ws, kStaticScratchBytes, idx_out,
+                               lens_out, score_out, stream);
+    if (!capturing && rc == BSA_OK) {
+        if (hipEventRecord(use.done, (hipStream_t)stream) == hipSuccess) {
+            use.pending = true;
+            use.stream = (hipStream_t)stream;
+        } else {
+            (void)hipGetLastError();
+            use.pending = false;
+        }
+    }
+    return rc;
 }
 
 }  // extern "C"

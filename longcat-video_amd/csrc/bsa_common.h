@@ -177,6 +177,7 @@ size_t frag_fallback_ints(int64_t items);
 
 // Backward of the blocked-order attention (bsa_bwd.hip), bf16 / fp16.  workspace: bwd_workspace_bytes() bytes.
 size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride);
+int bwd_max_query_blocks();      // the dK / dV kernel stages a KV block's query blocks in LDS: Sq / bs_q may not exceed this
 hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
                       const int32_t* idx, const int32_t* lens, const uint64_t* tile_valid, void* dq, void* dk, void* dv,
                       int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride, float sm_scale, int dtype,

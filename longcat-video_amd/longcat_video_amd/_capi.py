@@ -14,6 +14,7 @@ BSA_ERR_UNSUPPORTED = -2
 BSA_ERR_SHAPE = -3
 BSA_ERR_WORKSPACE = -4
 BSA_ERR_HIP = -5
+BSA_ERR_BUSY = -6
 
 BSA_BF16, BSA_F16, BSA_F32 = 0, 1, 2
 BSA_STATIC_SCRATCH_BYTES = 64 << 20
@@ -117,4 +118,4 @@ def check(status: int, what: str = "") -> None:
         raise ValueError(msg)
     if status == BSA_ERR_UNSUPPORTED:
         raise NotImplementedError(msg)
-    raise RuntimeError(msg)
+    raise RuntimeError(msg)          # workspace, HIP and busy errors

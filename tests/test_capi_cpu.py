@@ -97,6 +97,31 @@ def test_fwd_rejects_bad_arguments():
     assert call(p=[None] + ptrs[1:]) == _capi.BSA_ERR_BAD_ARG
 
 
+def test_fwd_fragment_and_bwd_shape_limits():
+    """The blocked-order entry on the fragment-order kernel and the backward reject what they cannot run before any
+    launch (no GPU is touched: every check comes before the first HIP call)."""
+    lib = _capi.load()
+    need = lib.bsa_fwd_fragment_workspace_bytes(1, 2, 640, 1280, 128, _capi.BSA_BF16)
+    assert need >= 2 * 2 * 1280 * 128 * 2 and need % 256 == 0                      # K and V in fragment order, two tables
+    assert lib.bsa_fwd_fragment_workspace_bytes(1, 2, 640, 1280, 128, _capi.BSA_F32) == 0
+    assert lib.bsa_fwd_fragment_workspace_bytes(1, 2, 640, 1290, 128, _capi.BSA_BF16) == 0
+    ptrs = [FAKE] * 5 + [None, FAKE, None]
+
+    def call(Sq=640, Sk=1280, D=128, bs_q=64, bs_k=64, stride=3, dtype=_capi.BSA_BF16, ws=FAKE, ws_bytes=1 << 30):
+        return lib.bsa_fwd_fragment(*ptrs, 1, 2, Sq, Sk, D, bs_q, bs_k, stride, 0.088, dtype, ws, ws_bytes, None)
+
+    assert call(dtype=_capi.BSA_F32) == _capi.BSA_ERR_UNSUPPORTED
+    assert call(D=64) == _capi.BSA_ERR_UNSUPPORTED
+    assert call(Sq=650) == _capi.BSA_ERR_SHAPE
+    assert call(stride=5000) == _capi.BSA_ERR_UNSUPPORTED and "4096" in _capi.last_error()
+    assert call(ws=None) == _capi.BSA_ERR_BAD_ARG
+    assert call(ws_bytes=need - 1) == _capi.BSA_ERR_WORKSPACE
+    # the backward stages a KV block's query blocks in LDS: more query blocks than fit are refused, with the number
+    assert lib.bsa_bwd_workspace_bytes(1, 1, 64 * 23552, 64, 128, 64, 64, 1, _capi.BSA_BF16) > 0
+    assert lib.bsa_bwd_workspace_bytes(1, 1, 64 * 23553, 64, 128, 64, 64, 1, _capi.BSA_BF16) == 0
+    assert "23552" in _capi.last_error()
+
+
 def test_fwd_3d_plan_and_workspace():
     lib = _capi.load()
     prm = _capi.Bsa3dParams(1, 32, 128, _capi.BSA_BF16, 24, 45, 80, 24, 45, 80, 4, 4, 4, 4, 4, 4, 90, 0.0883883)

@@ -75,3 +75,80 @@ def test_a_problem_beyond_the_buffer_is_rejected_before_any_launch():
     assert rc == _capi.BSA_ERR_WORKSPACE
     assert "scratch" in _capi.last_error()
     torch.cuda.synchronize()
+
+
+def _direct_call(lib, prm, q, k, v, o, stream):
+    """bsa_fwd_3d_static through the C-ABI with tensors that exist already: the Python side allocates nothing either."""
+    from longcat_video_amd import _capi
+    st = lambda t: _capi.strides3(t.stride()[:3])
+    return lib.bsa_fwd_3d_static(C.byref(prm), q.data_ptr(), st(q), k.data_ptr(), st(k), v.data_ptr(), st(v), o.data_ptr(), st(o),
+                                 None, None, None, C.c_void_p(stream.cuda_stream))
+
+
+def _problem(seed, heads, latent, k_sel):
+    from longcat_video_amd import _capi
+    S = int(np.prod(latent))
+    q, k, v = (t.cuda() for t in seeded_qkv(seed, 1, heads, S, S, 128, torch.bfloat16))
+    prm = _capi.Bsa3dParams(1, heads, 128, _capi.BSA_BF16, *latent, *latent, 4, 4, 4, 4, 4, 4, k_sel, 128 ** -0.5, 0.0)
+    return prm, q, k, v, torch.empty_like(q)
+
+
+def test_a_call_leaves_the_free_device_memory_as_it_was():
+    """What the entry point is for: after one warm call (which looks up the buffer's address) a call through the
+    C-ABI with existing tensors changes neither the driver's free memory nor what torch's allocator holds."""
+    from longcat_video_amd import _capi
+    lib = _capi.load()
+    prm, q, k, v, o = _problem(96, 2, (5, 9, 13), 6)
+    stream = torch.cuda.current_stream()
+    assert _direct_call(lib, prm, q, k, v, o, stream) == _capi.BSA_OK       # warm: symbol lookup, event creation
+    torch.cuda.synchronize()
+    want = o.clone()
+    o.zero_()
+    free_before, reserved_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
+    for _ in range(3):
+        assert _direct_call(lib, prm, q, k, v, o, stream) == _capi.BSA_OK
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before and torch.cuda.memory_reserved() == reserved_before
+    assert torch.equal(o, want)
+
+
+def test_a_captured_call_replays():
+    """Under stream capture the call records kernels only (no allocation, no memset node); every replay, with eager
+    work and synchronisations between them, gives the eager result."""
+    from longcat_video_amd import _capi
+    lib = _capi.load()
+    prm, q, k, v, o = _problem(97, 2, (4, 8, 12), 6)
+    assert _direct_call(lib, prm, q, k, v, o, torch.cuda.current_stream()) == _capi.BSA_OK
+    torch.cuda.synchronize()
+    want = o.clone()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph, stream=side):
+        assert _direct_call(lib, prm, q, k, v, o, torch.cuda.current_stream()) == _capi.BSA_OK
+    for r in range(3):
+        o.fill_(float(r))
+        (q.float().sum() + r).item()                     # eager work and a synchronisation between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(o, want), r
+
+
+def test_a_call_while_another_stream_still_uses_the_buffer_is_refused():
+    """Two streams: the second call arrives while the first one's kernels run and must come back with BSA_ERR_BUSY,
+    having launched nothing; once the first has finished, the same call goes through.  One stream never refuses."""
+    from longcat_video_amd import _capi
+    lib = _capi.load()
+    prm, q, k, v, o = _problem(98, 6, (24, 45, 80), 90)                      # the largest 720p share that fits: ~2 ms
+    o2 = torch.full_like(o, 7.0)
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    assert _direct_call(lib, prm, q, k, v, o, a) == _capi.BSA_OK
+    assert _direct_call(lib, prm, q, k, v, o, a) == _capi.BSA_OK             # same stream: in order, never refused
+    rc = _direct_call(lib, prm, q, k, v, o2, b)
+    assert rc == _capi.BSA_ERR_BUSY and "another stream" in _capi.last_error()
+    torch.cuda.synchronize()
+    assert bool((o2 == 7.0).all())                                           # nothing ran
+    assert _direct_call(lib, prm, q, k, v, o2, b) == _capi.BSA_OK
+    torch.cuda.synchronize()
+    assert torch.equal(o2, o)
