@@ -336,7 +336,35 @@ def run_bwd(torch, args):
     latent, sparsity, seed, rms, desc = WORKLOADS["c3"]
     q, k, v = make_inputs(torch, latent, seed, rms, args.inputs)
     qp, kp, vp = (I._permute(t, latent, CHUNK)[0] for t in (q, k, v))
-    del q, k, v
+    # ---- first the operator as a training step sees it: flash_attn_bsa_3d on inputs that require a gradient (the
+    # forward of every other call, which also keeps lse and the lists it walked) and autograd's backward through it
+    # (permutes into blocked order, bsa_bwd, permutes back)
+    prm = dict(sparsity=sparsity, chunk_3d_shape_q=list(CHUNK), chunk_3d_shape_k=list(CHUNK))
+    for t in (q, k, v):
+        t.requires_grad_(True)
+    d_o = torch.randn(q.shape, generator=torch.Generator(device="cuda").manual_seed(seed + 100), device="cuda").bfloat16()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    ms_tf, ms_tb = [], []
+    for rep in range(3):
+        for t in (q, k, v):
+            t.grad = None
+        ev[0].record()
+        o_t = I.flash_attn_bsa_3d(q, k, v, latent, latent, **prm)
+        ev[1].record()
+        o_t.backward(d_o)
+        ev[2].record()
+        torch.cuda.synchronize()
+        ms_tf.append(ev[0].elapsed_time(ev[1]))
+        ms_tb.append(ev[1].elapsed_time(ev[2]))
+    with torch.no_grad():
+        assert torch.equal(o_t, I.flash_attn_bsa_3d(q, k, v, latent, latent, **prm)), "one forward with and without grad"
+    assert all(bool(torch.isfinite(t.grad.float()).all()) for t in (q, k, v))
+    through_autograd = {"forward_with_grad_ms": round(min(ms_tf), 4), "backward_ms": round(min(ms_tb), 4),
+                        "note": "flash_attn_bsa_3d in (T,H,W) order on inputs that require a gradient; best of 3"}
+    for t in (q, k, v):
+        t.grad = None
+    del q, k, v, o_t, d_o
+    torch.cuda.empty_cache()
     sm = 1 / math.sqrt(D)
     idx, lens = I._select_blocked(qp, kp, 64, 64, sparsity, None)
     o, lse = I.attn_fwd_bsa_varlen(qp, kp, vp, sm, idx, lens, 64, 64)
@@ -363,6 +391,7 @@ def run_bwd(torch, args):
         "data": "synthetic N(0,1) q/k/v with per-head RMS-normalised q/k, " + DRAWN[args.inputs] + "; N(0,1) output gradient drawn on the GPU",
         "config": {"workload": "bwd: backward of the c3 layer in blocked order, 32 heads x 128, 1440 x 1440 blocks of 64, 90 per row",
                    "block_pairs": pairs},
+        "through_autograd": through_autograd,
         "roofline": {"kernel": "bwd_dq_lds_kernel<bf16> + bwd_dkdv_kernel<bf16> (with the passes before them)", "bound": "mfma",
                      "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / PEAK_BF16_TFLOPS, 4),

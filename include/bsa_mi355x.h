@@ -231,6 +231,22 @@ int bsa_fwd_3d(const bsa_3d_params* p,
                int32_t* idx_out, int32_t* lens_out, void* score_out, void* stream);
 
 /*
+ * bsa_fwd_3d for a caller that will ask for gradients: the same kernels and the same output bit for bit
+ * (_attention_bsa.forward runs one kernel with and without grad and keeps lse, bsa:538-568), plus what the
+ * backward needs: lse_out [B, Hn, Tq*Hq*Wq] fp32 in token order (natural log; -inf for a query without keys),
+ * walk_out int32 [B, Hn, nbq, width] - every query block's selected KV blocks in the order the kernel visited them,
+ * block numbers counted in the padded chunk grid (width as idx_out of bsa_fwd_3d) - and lens_out int32 [B, Hn, nbq].
+ * bf16 / fp16.
+ */
+int bsa_fwd_3d_lse(const bsa_3d_params* p,
+                   const void* q, const int64_t q_strides[3],
+                   const void* k, const int64_t k_strides[3],
+                   const void* v, const int64_t v_strides[3],
+                   void* o, const int64_t o_strides[3],
+                   float* lse_out, int32_t* walk_out, int32_t* lens_out,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Backward of bsa_fwd: gradients of the block-sparse attention with respect to q, k and v.
  * Replaces attn_bwd_bsa_varlen_triton (bsa:341-461) and the kernels _attn_bwd_preprocess (common.py:94-111),
  * _attn_bwd_dkdv_bsa_varlen_wrapper (vmask:505-642) and _attn_bwd_dq_bsa_varlen(_align)_wrapper (vmask:665-945),

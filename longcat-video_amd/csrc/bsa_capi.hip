@@ -591,7 +591,7 @@ int fwd_3d_impl(const Plan& pl, const bsa_3d_params* p, const void* q, const int
                 const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
                 const int64_t o_strides[3], void* workspace, size_t workspace_bytes, int32_t* idx_out,
                 int32_t* lens_out, void* score_out, void* stream, const bsa_qk_norm* qkn = nullptr, void* q_normed = nullptr,
-                const int64_t* qn_strides = nullptr) {
+                const int64_t* qn_strides = nullptr, float* lse_out = nullptr, int32_t* walk_out = nullptr) {
     Ws w;
     if (!q || !k || !v || !o || !workspace) return set_error(BSA_ERR_BAD_ARG, "fwd_3d: null pointer");
     BSA_TRY(carve(pl, workspace, workspace_bytes, "fwd_3d", &w));
@@ -640,7 +640,7 @@ int fwd_3d_impl(const Plan& pl, const bsa_3d_params* p, const void* q, const int
         if (pl.cdf)
             BSA_HIP(launch_order_by_length(w.lens, w.order, p->B * p->Hn, pl.nbq, pl.gq.chunk() / 64, pl.sel_width, st), "order by length");
         BSA_HIP(attention_thw(pl, p, w, q, q_strides, k, k_strides, v, v_strides, o, o_strides, w.idx_sorted, w.lens, pl.sel_width,
-                              nullptr, st, pl.cdf), "attention");
+                              lse_out, st, pl.cdf), "attention");
     } else {
         BSA_HIP(launch_fwd(w.qp, w.kp, w.vp, w.idx_sorted, w.lens, padded_k ? w.valid : nullptr, w.op, nullptr, p->B, p->Hn, pl.Sqp, pl.Skp,
                            pl.gq.chunk(), pl.gk.chunk(), pl.sel_width, p->sm_scale, p->dtype, st), "attention");
@@ -649,6 +649,8 @@ int fwd_3d_impl(const Plan& pl, const bsa_3d_params* p, const void* q, const int
     const size_t bh = (size_t)p->B * p->Hn;
     if (idx_out && pl.sel_width > 0)
         BSA_HIP(hipMemcpyAsync(idx_out, w.idx, bh * pl.nbq * pl.sel_width * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy idx");
+    if (walk_out && pl.sel_width > 0)
+        BSA_HIP(hipMemcpyAsync(walk_out, w.idx_sorted, bh * pl.nbq * pl.sel_width * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy walk order");
     if (lens_out) BSA_HIP(hipMemcpyAsync(lens_out, w.lens, bh * pl.nbq * sizeof(int32_t), hipMemcpyDeviceToDevice, st), "copy lens");
     if (score_out) BSA_HIP(hipMemcpyAsync(score_out, w.score, bh * pl.nbq * (size_t)pl.nbk * pl.es, hipMemcpyDeviceToDevice, st), "copy score");
 #undef BSA_HIP
@@ -700,6 +702,18 @@ int bsa_fwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3]
     BSA_TRY(make_plan(p, &pl));
     return fwd_3d_impl(pl, p, q, q_strides, k, k_strides, v, v_strides, o, o_strides, workspace, workspace_bytes, idx_out,
                        lens_out, score_out, stream);
+}
+
+int bsa_fwd_3d_lse(const bsa_3d_params* p, const void* q, const int64_t q_strides[3], const void* k,
+                   const int64_t k_strides[3], const void* v, const int64_t v_strides[3], void* o,
+                   const int64_t o_strides[3], float* lse_out, int32_t* walk_out, int32_t* lens_out, void* workspace,
+                   size_t workspace_bytes, void* stream) {
+    Plan pl;
+    BSA_TRY(make_plan(p, &pl));
+    if (!pl.direct_qo) return set_error(BSA_ERR_UNSUPPORTED, "fwd_3d_lse: bf16 and fp16 only (the backward is built for them)");
+    if (!lse_out || !walk_out || !lens_out) return set_error(BSA_ERR_BAD_ARG, "fwd_3d_lse: lse_out, walk_out and lens_out are required");
+    return fwd_3d_impl(pl, p, q, q_strides, k, k_strides, v, v_strides, o, o_strides, workspace, workspace_bytes, nullptr,
+                       lens_out, nullptr, stream, nullptr, nullptr, nullptr, lse_out, walk_out);
 }
 
 int bsa_fwd_3d_qknorm(const bsa_3d_params* p, const bsa_qk_norm* n, const void* q, const int64_t q_strides[3],

@@ -58,6 +58,8 @@ SIGNATURES = {
     "bsa_workspace_bytes": (C.c_size_t, [C.POINTER(Bsa3dParams)]),
     "bsa_fwd_3d": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
                         _p, C.c_size_t, _p, _p, _p, _p]),
+    "bsa_fwd_3d_lse": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
+                            _p, _p, _p, _p, C.c_size_t, _p]),
     "bsa_fwd_3d_qknorm": (_i, [C.POINTER(Bsa3dParams), C.POINTER(BsaQkNorm), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
                                _p, _strides, _p, C.c_size_t, _p, _p, _p, _p]),
     "bsa_fwd_3d_static": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,

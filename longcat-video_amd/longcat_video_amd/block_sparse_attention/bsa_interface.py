@@ -442,14 +442,15 @@ def flash_attn_bsa(q, k, v, chunk_size_q, chunk_size_k, sparsity, cdf_threshold,
 # R9: the operator
 # ---------------------------------------------------------------------------
 def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k, want_selection=False, out=None,
-            cdf_threshold=None, static_scratch=False, qk_norm=None):
+            cdf_threshold=None, static_scratch=False, qk_norm=None, for_backward=False):
     """`out`: optional [B,H,Sq,D] view (any B/H/S strides, contiguous D) to write into.  `sparsity` may be
     None when `cdf_threshold` is given (bsa_interface.py:268-277).  `static_scratch`: run through
     bsa_fwd_3d_static, which keeps its scratch memory in a buffer built into the library instead of a
     workspace tensor (problems beyond that buffer raise; calls on one GPU must not overlap).
     `qk_norm` = (q_weight, k_weight, rope_table, table_T, t_offset_q, t_offset_k, eps): q and k are the raw
     projections and are normalised per head and rotated inside the operator's own passes (bsa_fwd_3d_qknorm;
-    bf16 / fp16 and 64-token chunks only)."""
+    bf16 / fp16 and 64-token chunks only).  `for_backward`: the same kernels through bsa_fwd_3d_lse; returns
+    (o, lists in the kernel's visiting order, lens, lse in token order) for the backward."""
     _need_gpu(q, k, v)
     B, H, Sq, D = q.shape
     Tq, Hq, Wq = (int(x) for x in latent_shape_q)
@@ -483,6 +484,16 @@ def _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k,
         idx = torch.empty(B, H, nbq, width, dtype=torch.int32, device=q.device)
         lens = torch.empty(B, H, nbq, dtype=torch.int32, device=q.device)
         score = torch.empty(B, H, nbq, nbk, dtype=q.dtype, device=q.device)
+    if for_backward:
+        walk = torch.empty(B, H, nbq, max(width, 1), dtype=torch.int32, device=q.device)[..., :width]
+        lens = torch.empty(B, H, nbq, dtype=torch.int32, device=q.device)
+        lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device)
+        with torch.cuda.device(q.device):
+            _capi.check(lib.bsa_fwd_3d_lse(
+                C.byref(prm), _ptr(q), _capi.strides3(q.stride()[:3]), _ptr(k), _capi.strides3(k.stride()[:3]),
+                _ptr(v), _capi.strides3(v.stride()[:3]), _ptr(o), _capi.strides3(o.stride()[:3]),
+                _ptr(lse), _ptr(walk), _ptr(lens), _ptr(ws), need, _stream(q)), "flash_attn_bsa_3d (with lse)")
+        return o, walk, lens, lse
     with torch.cuda.device(q.device):
         if qk_norm is not None:
             qw, kw, tab, table_T, t_off_q, t_off_k, eps = qk_norm
@@ -568,33 +579,58 @@ def attn_fwd_bsa_thw(q, k, v, latent_shape_q, latent_shape_k, chunk_3d_shape_q, 
         q, block_indices, block_indices_lens, return_lse, out)
 
 
+_SLOT_TOKENS: dict = {}
+
+
+def _slot_tokens(latent_shape, chunk, device) -> torch.Tensor:
+    """Token index of every slot of the blocked order of a (T, H, W) grid cut into chunks (bsa_interface.py:600-604
+    on the padded grid), -1 for padding.  int64 [padded slots]; kept per (grid, chunk, device)."""
+    key = (tuple(latent_shape), tuple(chunk), str(device))
+    m = _SLOT_TOKENS.get(key)
+    if m is None:
+        (T, Hh, W), (t, h, w) = latent_shape, chunk
+        Nt, Nh, Nw = -(-T // t), -(-Hh // h), -(-W // w)
+        ar = lambda n: torch.arange(n, device=device)
+        tt = (ar(Nt).view(Nt, 1, 1, 1, 1, 1) * t + ar(t).view(1, 1, 1, t, 1, 1)).expand(Nt, Nh, Nw, t, h, w)
+        hh = (ar(Nh).view(1, Nh, 1, 1, 1, 1) * h + ar(h).view(1, 1, 1, 1, h, 1)).expand(Nt, Nh, Nw, t, h, w)
+        ww = (ar(Nw).view(1, 1, Nw, 1, 1, 1) * w + ar(w).view(1, 1, 1, 1, 1, w)).expand(Nt, Nh, Nw, t, h, w)
+        tok = (tt * Hh + hh) * W + ww
+        m = torch.where((tt < T) & (hh < Hh) & (ww < W), tok, torch.full_like(tok, -1)).reshape(-1).contiguous()
+        _SLOT_TOKENS[key] = m
+    return m
+
+
 class _Bsa3dWithGrad(torch.autograd.Function):
-    """The operator for inputs that require a gradient: bsa_interface.py:646-660 as written there - permute,
-    ``_attention_bsa`` on blocked-order tensors, unpermute - with the permutes' own gradients (each is the other's)."""
+    """The operator for inputs that require a gradient.  The forward is the forward of every other call - the same
+    kernels on the same lists, the same bits (bsa_interface.py:538-568 runs one kernel with and without grad) - and
+    keeps the log-sum-exp and the lists it walked.  The backward moves q, k, v, o and dO into the blocked order in
+    which bsa_bwd takes them (bsa_interface.py:650-652; the permutes are each other's gradient) and the three
+    gradients back."""
 
     @staticmethod
     def forward(ctx, q, k, v, latent_shape_q, latent_shape_k, sparsity, cdf_threshold, chunk_q, chunk_k):
-        D = q.shape[-1]
-        bs_q, bs_k = int(math.prod(chunk_q)), int(math.prod(chunk_k))
-        qp, _, _ = _permute(q, latent_shape_q, chunk_q)
-        kp, _, valid = _permute(k, latent_shape_k, chunk_k, want_valid=True)
-        vp, _, _ = _permute(v, latent_shape_k, chunk_k)
-        padded_k = kp.shape[2] != k.shape[2]
-        idx, lens = _select_blocked(qp, kp, bs_q, bs_k, sparsity, cdf_threshold)
-        sm_scale = 1 / D ** 0.5
-        op, lse = attn_fwd_bsa_varlen(qp, kp, vp, sm_scale, idx, lens, bs_q, bs_k, sparsity, valid if padded_k else None)
-        ctx.save_for_backward(qp, kp, vp, op, lse, idx, lens, valid)
-        ctx.args = (tuple(latent_shape_q), tuple(latent_shape_k), tuple(chunk_q), tuple(chunk_k), sm_scale, padded_k)
-        return _unpermute(op, latent_shape_q, chunk_q)
+        o, walk, lens, lse = _bsa_3d(q, k, v, latent_shape_q, latent_shape_k, sparsity, chunk_q, chunk_k,
+                                     cdf_threshold=cdf_threshold, for_backward=True)
+        ctx.save_for_backward(q, k, v, o, lse, walk, lens)
+        ctx.args = (tuple(latent_shape_q), tuple(latent_shape_k), tuple(chunk_q), tuple(chunk_k), 1 / q.shape[-1] ** 0.5)
+        return o
 
     @staticmethod
     def backward(ctx, do):
-        qp, kp, vp, op, lse, idx, lens, valid = ctx.saved_tensors
-        latent_q, latent_k, chunk_q, chunk_k, sm_scale, padded_k = ctx.args
+        q, k, v, o, lse, walk, lens = ctx.saved_tensors
+        latent_q, latent_k, chunk_q, chunk_k, sm_scale = ctx.args
         bs_q, bs_k = int(math.prod(chunk_q)), int(math.prod(chunk_k))
+        qp, _, _ = _permute(q, latent_q, chunk_q)
+        kp, _, valid = _permute(k, latent_k, chunk_k, want_valid=True)
+        vp, _, _ = _permute(v, latent_k, chunk_k)
+        op, _, _ = _permute(o, latent_q, chunk_q)
         dop, _, _ = _permute(do, latent_q, chunk_q)                      # padded slots get a zero gradient
+        padded_k = kp.shape[2] != k.shape[2]
+        # lse in blocked order; a padded query slot has no keys as far as the backward is concerned (its p is 0)
+        slots = _slot_tokens(latent_q, chunk_q, q.device)
+        lse_p = torch.where(slots >= 0, lse[..., slots.clamp(min=0)], torch.full((), float("-inf"), device=q.device))
         dqp, dkp, dvp = (torch.empty_like(t) for t in (qp, kp, vp))
-        attn_bwd_bsa_varlen(dop, qp, kp, vp, op, dqp, dkp, dvp, sm_scale, lse, idx, lens, bs_q, bs_k, None,
+        attn_bwd_bsa_varlen(dop, qp, kp, vp, op, dqp, dkp, dvp, sm_scale, lse_p, walk, lens, bs_q, bs_k, None,
                             valid if padded_k else None)
         return (_unpermute(dqp, latent_q, chunk_q), _unpermute(dkp, latent_k, chunk_k), _unpermute(dvp, latent_k, chunk_k),
                 None, None, None, None, None, None)

@@ -131,7 +131,7 @@ def test_autograd_through_the_blocked_order_operator():
         assert torch.equal(bi.flash_attn_bsa(q, k, v, 64, 64, 0.75, None, sm), o)
 
 
-@pytest.mark.parametrize("shape", [(8, 8, 16), (6, 10, 14)])
+@pytest.mark.parametrize("shape", [(8, 8, 16), (6, 10, 14), (9, 13, 22)])
 def test_autograd_through_the_operator_on_a_grid(shape):
     """flash_attn_bsa_3d with inputs that require a gradient, on a grid with and without padded chunks: gradients in
     (T, H, W) order against autograd through fp32 attention with the token-level mask of the GPU's own selection."""
@@ -145,8 +145,7 @@ def test_autograd_through_the_operator_on_a_grid(shape):
     o.backward(do)
     with torch.no_grad():
         o_plain = bi.flash_attn_bsa_3d(q, k, v, shape, shape, sparsity=0.5, chunk_3d_shape_q=list(chunk), chunk_3d_shape_k=list(chunk))
-    d = (o.detach().float() - o_plain.float()).abs()
-    assert float(d.max()) <= 1.6e-2 and float(d.mean()) <= 1e-3           # two attention kernels, one selection
+    assert torch.equal(o.detach(), o_plain)                                # one forward kernel with and without grad (bsa:538-568)
     # the oracle in blocked order on the GPU's selection
     qp, kp, vp, dop = (O.rearrange_thw_to_3d_block(t.detach().cpu(), shape, chunk) for t in (q, k, v, do))
     idx, lens = bi._select_blocked(qp.cuda(), kp.cuda(), 64, 64, 0.5, None)
