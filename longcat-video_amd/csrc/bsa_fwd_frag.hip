@@ -924,7 +924,11 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
 
 }  // namespace
 
+// Rounds per launch: two (three and four measure the same at 90 tiles per list, from six on the items drift apart and the
+// L2 hit rate falls); three for short lists, whose launches are otherwise over before the clock has settled.
 constexpr int kRoundsPerLaunch = 2;
+constexpr int kRoundsPerLaunchShort = 3;     // lists of at most kShortList tiles
+constexpr int kShortList = 64;
 
 // Workgroups (of one wavefront) the device runs at once with this kernel: one per SIMD.
 static int resident_wavefronts() {
@@ -1006,7 +1010,7 @@ hipError_t launch_fwd_frag(const void* q, const void* kf, const void* vf, const 
     if (bounded) hipLaunchKernelGGL(frag_zero_kernel, dim3(1), dim3(64), 0, st, fb_count, 1);
     // kRoundsPerLaunch rounds per launch, every workgroup running one item of each: the items of a round start
     // together and keep in step (with many more rounds per launch they drift apart and the L2 hit rate falls).
-    const int span = kRoundsPerLaunch * resident;
+    const int span = (idx_stride * (bs_k / kTile) <= kShortList ? kRoundsPerLaunchShort : kRoundsPerLaunch) * resident;
     for (int first = 0; first < total;) {
         int end = first + span < total ? first + span : total;
         const int bh0 = first / per_head;

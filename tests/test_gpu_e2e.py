@@ -431,3 +431,40 @@ def test_cdf_lists_of_unequal_length_schedule(spread):
     for m in blocks:
         d = (got_p[:, :, 64 * m:64 * m + 64].float() - want_o[:, :, 64 * m:64 * m + 64]).abs()
         assert d.max() <= MAX_ABS and d.mean() <= MEAN_ABS
+
+
+def test_keys_beyond_one_buffer_span():
+    """6 batches x 32 heads at the 720p grid: K in fragment order is 4.5 GB, more than the 4 GB one buffer resource of the
+    attention kernel spans, so the launches are cut at head boundaries and each addresses K and V from its own first
+    head.  The last batch must come out as when it is given alone (another kernel variant: the tolerance between two
+    summation orders), and equal to the oracle on sampled blocks."""
+    latent = (24, 45, 80)
+    B, H, S = 6, 32, 86400
+    g = torch.Generator(device="cuda").manual_seed(11)
+    q, k, v = (torch.randn(B, H, S, 128, generator=g, device="cuda").bfloat16() for _ in range(3))
+    bi = I()
+    o = bi.flash_attn_bsa_3d(q, k, v, latent, latent, sparsity=0.9375, **CH)
+    assert torch.isfinite(o.float()).all()
+    for b in (0, B - 1):
+        one, idx, lens, score = bi._bsa_3d(q[b:b + 1], k[b:b + 1], v[b:b + 1], latent, latent, 0.9375, (4, 4, 4), (4, 4, 4), True)
+        d = (o[b:b + 1].float() - one.float()).abs()
+        assert float(d.max()) <= 1.6e-2 and float(d.mean()) <= 1e-3, (b, float(d.max()), float(d.mean()))
+    check_against_oracle(q[B - 1:].cpu(), k[B - 1:].cpu(), v[B - 1:].cpu(), latent, latent, 0.9375, o[B - 1:], idx, lens, score,
+                         q_blocks=[0, 733, 1439], heads=[0, 31])
+
+
+def test_query_rows_too_far_apart_for_32_bit_offsets():
+    """q as a view whose token rows lie 1.2 MB apart (4.9 GB from first to last): the LDS DMA that prepares the next
+    work item's Q rows cannot address them, so every item fetches its own; the result must not change."""
+    latent = (4, 32, 32)
+    S = 4096
+    g = torch.Generator(device="cuda").manual_seed(12)
+    qc, k, v = (torch.randn(1, 1, S, 128, generator=g, device="cuda").bfloat16() for _ in range(3))
+    wide = torch.empty(1, 1, S, 600000, dtype=torch.bfloat16, device="cuda")        # 4096 rows x 1.2 MB
+    q = wide[..., :128]
+    q.copy_(qc)
+    assert q.stride(2) * 2 * S > 2 ** 32 and not q.is_contiguous()
+    bi = I()
+    got = bi.flash_attn_bsa_3d(q, k, v, latent, latent, sparsity=0.75, **CH)
+    want = bi.flash_attn_bsa_3d(qc, k, v, latent, latent, sparsity=0.75, **CH)
+    assert torch.equal(got, want)
