@@ -246,7 +246,41 @@ def measure_c4(torch, steps, warmup, settle, where):
     return ms, ms_attn, pairs, (T, Hh, W, cond, S, n)
 
 
-def measure_operator(torch, workload, steps, warmup, settle, where, coherent=False):
+def sample_clocks(torch, fn, seconds=3.0):
+    """Runs fn back to back for `seconds` while a thread asks `rocm-smi` (a child process) for the shader clock and the
+    board power every 0.3 s: what the kernel settles at once the power controller has acted."""
+    import re
+    import subprocess
+    import threading
+    samples, stop = [], threading.Event()
+
+    def sampler():
+        while not stop.is_set():
+            try:
+                text = subprocess.run(["rocm-smi", "--showclocks", "--showpower"], capture_output=True, text=True, timeout=10).stdout
+                sclk = re.findall(r"sclk clock level: \d+: \((\d+)Mhz\)", text)
+                watt = re.findall(r"Power[^\n]*\(W\)[^\n]*?:\s*([\d.]+)", text)
+                samples.append((int(sclk[0]) if sclk else None, float(watt[0]) if watt else None))
+            except Exception:
+                samples.append((None, None))
+            stop.wait(0.3)
+    th = threading.Thread(target=sampler)
+    t0, calls = time.perf_counter(), 0
+    th.start()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
+        calls += 8
+    ms = (time.perf_counter() - t0) * 1e3 / calls
+    stop.set()
+    th.join()
+    samples = samples[1:] or samples                # the first reading may precede the load
+    return {"ms_per_call_in_this_loop": round(ms, 4), "sclk_mhz": [a for a, _ in samples], "power_w": [b for _, b in samples],
+            "nominal_sclk_mhz": 2400, "how": "rocm-smi --showclocks --showpower every 0.3 s while the attention kernel runs back to back"}
+
+
+def measure_operator(torch, workload, steps, warmup, settle, where, coherent=False, clocks=None):
     """One of the single-call workloads: ms per layer of the whole operator over exactly `steps` timed calls, and of its
     attention kernel alone exactly as the operator runs it (same lists in the same visiting order, same (T, H, W)
     addressing, workspace prepared outside the timed region; its output is asserted equal to the operator's)."""
@@ -269,6 +303,8 @@ def measure_operator(torch, workload, steps, warmup, settle, where, coherent=Fal
     o_buf = torch.empty_like(q)
     ms_attn = time_events(torch, lambda: attend(q, idx, lens, out=o_buf), max(steps, 20), max(warmup, 5), settle_s=settle)
     assert torch.equal(o_buf, o), "the separately timed attention kernel must reproduce the operator's output"
+    if clocks is not None:
+        clocks.update(sample_clocks(torch, lambda: attend(q, idx, lens, out=o_buf)))
     del attend, o_buf, o
     return ms_step, ms_attn, idx.shape[2], idx.shape[3], (q, k, v)
 
@@ -575,6 +611,9 @@ def main():
                          "machine; half a minute at 720p) or the GPU's")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="c3: leave out the attention-kernel figures of c2 and c4 that the default line carries beside its own")
+    ap.add_argument("--clocks", action="store_true",
+                    help="c2, c3: also run the attention kernel back to back for three seconds and report the shader clock and "
+                         "board power that rocm-smi shows meanwhile")
     ap.add_argument("--data", default="random", choices=["random", "coherent"],
                     help="random (the benchmark's definition) or spatially coherent q/k (c2, c3 only; no CPU baseline)")
     args = ap.parse_args()
@@ -597,7 +636,8 @@ def main():
     latent, sparsity, seed, rms, desc = WORKLOADS[args.workload]
     coherent = args.data == "coherent"
     # ---- whole operator: warm-up, then exactly K timed steps between synchronisations; then the attention kernel alone
-    ms_step, ms_attn, nbq, k_sel, (q, k, v) = measure_operator(torch, args.workload, args.steps, args.warmup, args.settle, args.inputs, coherent)
+    clocks = {} if args.clocks else None
+    ms_step, ms_attn, nbq, k_sel, (q, k, v) = measure_operator(torch, args.workload, args.steps, args.warmup, args.settle, args.inputs, coherent, clocks)
     ksteps, kwarm = max(args.steps, 20), max(args.warmup, 5)      # kernels alone: enough calls for a steady clock
     # the other entry points on their own (the permutes are no longer part of the operator for bf16)
     qp, q_cmp, _ = I._permute(q, latent, CHUNK, want_pooled=True)
@@ -639,6 +679,8 @@ def main():
         "permute_gbs": round(permute_bytes / (ms_permute * 1e-3) / 1e9, 1),
         "roofline": attention_roofline(flop, ms_attn, args.workload, coherent),
     }
+    if clocks:
+        result["clocks_under_the_attention_kernel"] = clocks
     del q, k, v, qp, q_cmp, k_cmp
     torch.cuda.empty_cache()
     if args.workload == "c3" and not coherent and not args.no_other_configs:

@@ -323,6 +323,8 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
         __builtin_amdgcn_sched_barrier(0);
         take_transposed(hp + 1);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        // the chains into (ns, ndp) end here, sixteen MFMAs behind their last one
+        mfma_chain_end(ns[0]); mfma_chain_end(ns[1]); mfma_chain_end(ndp[0]); mfma_chain_end(ndp[1]);
     };
     if (nhalves > 0) {
         f32x16 sa[2], dpa[2], sb[2], dpb[2];
@@ -333,6 +335,7 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
         products(0, sa, dpa, [&]() {}, [&](int) {});
         take_transposed(0);
         asm volatile("s_nop 15\n\ts_nop 7\n\ts_waitcnt lgkmcnt(0)" ::: "memory");
+        mfma_chain_end(sa[0]); mfma_chain_end(sa[1]); mfma_chain_end(dpa[0]); mfma_chain_end(dpa[1]);
         for (int hp = 0; hp < nhalves; hp += 2) {                                // halves come in pairs
             step(hp, sa, dpa, sb, dpb);
             step(hp + 1, sb, dpb, sa, dpa);
@@ -568,6 +571,8 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
         products_and_exponentials(hp, s, dp, s_next, dp_next, [&]() { issue(hp + 3, (hp + 3) & 3); });
         __builtin_amdgcn_sched_barrier(0);
         gradients(hp, s, dp);
+        // the chains into (s_next, dp_next) end here, sixteen MFMAs behind their last one
+        mfma_chain_end(s_next); mfma_chain_end(dp_next);
         if (hp + 3 < nhalves) {
             if (wave == 0) asm volatile("s_waitcnt vmcnt(9) lgkmcnt(0)" ::: "memory");
             else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
@@ -609,6 +614,7 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
                 mfma_s<false, false>(dp0, *reinterpret_cast<const V8*>(dn + roff[c]), vreg[c]);
             }
             asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+            mfma_chain_end(s0); mfma_chain_end(dp0);
         }
         for (int hp = 0; hp < nhalves; hp += 2) {                                // halves come in pairs
             step(hp, s0, dp0, s1, dp1);

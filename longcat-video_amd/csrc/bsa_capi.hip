@@ -474,8 +474,10 @@ hipError_t prepare_thw(const Plan& pl, const bsa_3d_params* p, const Ws& w, cons
         e = launch_permute(q, q_strides, nullptr, nullptr, nullptr, 1, 1, pl.gq, p->D, p->dtype, st, false, w.qrows, nullptr);
     if (e != hipSuccess) return e;
     if (pool && pl.frag && pl.gq.chunk() == 64) {
-        // chunk means of q from the fragment pass run without a destination: the same sums, a faster read
-        e = launch_frag(q, q_strides, nullptr, p->B, p->Hn, pl.gq, p->dtype, false, st, w.qc, nullptr, trq);
+        // chunk means of q from a read-only pass (the same sums); with a row transform, from the fragment pass run
+        // without a destination, which applies it
+        if (trq == nullptr && p->D == 128) e = launch_pool_tiles(q, q_strides, w.qrows, w.qc, p->B, p->Hn, pl.gq, p->dtype, st);
+        else e = launch_frag(q, q_strides, nullptr, p->B, p->Hn, pl.gq, p->dtype, false, st, w.qc, nullptr, trq);
         if (e != hipSuccess) return e;
     }
     if (pl.frag) {

@@ -103,6 +103,11 @@ hipError_t launch_permute(const void* src, const int64_t strides[3], void* dst, 
                           hipStream_t st, bool edge_only = false, int32_t* row_table = nullptr,
                           uint32_t* tile_table = nullptr, const void* src2 = nullptr,
                           const int64_t* strides2 = nullptr, void* dst2 = nullptr);
+// Chunk means of a 16-bit tensor with 64-slot chunks and D = 128, nothing else: the bits of launch_permute's pooling
+// from a read-only pass.  row_table: the token of every slot of one (batch, head), -1 for padding, as launch_permute
+// writes it.
+hipError_t launch_pool_tiles(const void* src, const int64_t strides[3], const int32_t* row_table, void* pooled, int B, int Hn,
+                             const Grid3& g, int dtype, hipStream_t st);
 hipError_t launch_unpermute(const void* src, void* dst, const int64_t strides[3], int B, int Hn,
                             const Grid3& g, int D, int dtype, hipStream_t st);
 hipError_t launch_mean_pool(const void* x, void* out, int B, int Hn, int64_t S, int block, int D,

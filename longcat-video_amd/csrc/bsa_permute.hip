@@ -183,6 +183,90 @@ __global__ __launch_bounds__(kThreads) void mean_pool_kernel(const T* __restrict
     finish_pool<T>(acc, red, out + ((int64_t)bh * nb + blk) * D, cpr, c, rg, RG, 1.0f / block);
 }
 
+// Chunk means only, for 64-slot chunks of 16-bit rows of 128 elements: one wavefront per chunk, no LDS, no
+// barrier, all of a lane's sixteen 16-byte loads in flight at once (the read-only pass over q of the operator).
+// Rows come through the row table (token of every slot, -1 = padding: a zero row).  The sums are taken in
+// permute_kernel's order - a thread's rows rg, rg + 16, rg + 32, rg + 48 first, then the sixteen partial sums
+// of a column in ascending rg, starting from zero - so the means carry the same bits.  Lane = (c16, r4): 16-byte
+// piece c16 of the rows rg = 4 r4 .. 4 r4 + 3.
+template <bool kBf16>
+__global__ __launch_bounds__(256) void pool_tiles_kernel(const uint16_t* __restrict__ src, int64_t sB, int64_t sH, int64_t sS,
+                                                         const int32_t* __restrict__ row_table, uint16_t* __restrict__ pooled,
+                                                         int tiles, int Hn, int64_t total, int head_fastest) {
+    const int lane = threadIdx.x & 63;
+    const int64_t id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (id >= total) return;
+    int tile_id, bh;
+    if (head_fastest) {
+        const int64_t per_batch = (int64_t)tiles * Hn;
+        const int b = (int)(id / per_batch), rest = (int)(id - b * per_batch);
+        tile_id = rest / Hn;
+        bh = b * Hn + (rest - tile_id * Hn);
+    } else {
+        bh = (int)(id / tiles);
+        tile_id = (int)(id - (int64_t)bh * tiles);
+    }
+    const uint16_t* sbase = src + (int64_t)(bh / Hn) * sB + (int64_t)(bh % Hn) * sH;
+    const int c16 = lane & 15, r4 = lane >> 4;
+    // the table entries first, then every row unconditionally (a padded slot reads token 0 and is cleared afterwards):
+    // sixteen independent loads per lane, no branch between them
+    int32_t token[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) token[u][i] = row_table[tile_id * 64 + 4 * r4 + u + 16 * i];
+    uint4 xs[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            xs[u][i] = *reinterpret_cast<const uint4*>(sbase + (int64_t)max(token[u][i], 0) * sS + c16 * 8);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (token[u][i] < 0) xs[u][i] = make_uint4(0, 0, 0, 0);
+    float part[4][8];                       // this lane's rows rg = 4 r4 + u: rg, rg + 16, rg + 32, rg + 48 in that order
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) part[u][e] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w[4] = {xs[u][i].x, xs[u][i].y, xs[u][i].z, xs[u][i].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float lo, hi;
+                if (kBf16) { lo = __uint_as_float(w[e] << 16); hi = __uint_as_float(w[e] & 0xffff0000u); }
+                else { lo = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[e] & 0xffffu)); hi = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[e] >> 16)); }
+                part[u][2 * e] += lo;
+                part[u][2 * e + 1] += hi;
+            }
+        }
+    }
+    // the sixteen partial sums of a column in ascending rg: four per lane, handed from r4 to r4 + 1
+    float sum[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum[e] = 0.f;
+#pragma unroll
+    for (int stage = 0; stage < 4; ++stage) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float below = stage == 0 ? 0.f : __shfl_up(sum[e], 16);
+            if (r4 == stage) sum[e] = (((below + part[0][e]) + part[1][e]) + part[2][e]) + part[3][e];
+        }
+    }
+    if (r4 == 3) {
+        uint16_t out[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float mean = sum[e] * (1.0f / 64.0f);
+            out[e] = kBf16 ? __builtin_bit_cast(uint16_t, (__bf16)mean) : __builtin_bit_cast(uint16_t, (_Float16)mean);
+        }
+        *reinterpret_cast<uint4*>(pooled + ((int64_t)bh * tiles + tile_id) * 128 + c16 * 8) = *reinterpret_cast<const uint4*>(out);
+    }
+}
+
 inline size_t red_bytes(int D, int esize) {
     const int cpr = D / (16 / esize);
     return (size_t)(kThreads / cpr) * D * sizeof(float);
@@ -212,6 +296,21 @@ hipError_t launch_permute(const void* src, const int64_t st3[3], void* dst, void
     else if (dtype == BSA_F16) { BSA_LAUNCH(_Float16) }
     else { BSA_LAUNCH(float) }
 #undef BSA_LAUNCH
+    return hipGetLastError();
+}
+
+hipError_t launch_pool_tiles(const void* src, const int64_t st3[3], const int32_t* row_table, void* pooled, int B, int Hn,
+                             const Grid3& g, int dtype, hipStream_t st) {
+    if (g.chunk() != 64 || (dtype != BSA_BF16 && dtype != BSA_F16) || row_table == nullptr) return hipErrorInvalidValue;
+    const int64_t total = (int64_t)g.blocks() * B * Hn;
+    const dim3 grid((unsigned)((total + 3) / 4)), block(256);
+    const int head_fastest = st3[1] < st3[2] ? 1 : 0;
+    if (dtype == BSA_BF16)
+        hipLaunchKernelGGL(pool_tiles_kernel<true>, grid, block, 0, st, (const uint16_t*)src, st3[0], st3[1], st3[2], row_table,
+                           (uint16_t*)pooled, g.blocks(), Hn, total, head_fastest);
+    else
+        hipLaunchKernelGGL(pool_tiles_kernel<false>, grid, block, 0, st, (const uint16_t*)src, st3[0], st3[1], st3[2], row_table,
+                           (uint16_t*)pooled, g.blocks(), Hn, total, head_fastest);
     return hipGetLastError();
 }
 

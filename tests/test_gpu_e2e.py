@@ -140,6 +140,30 @@ def test_strided_inputs_from_a_qkv_projection():
     assert torch.equal(dq.cpu(), q)      # inputs are not modified
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("token_major", [False, True])
+def test_the_operator_scores_equal_the_standalone_route(dtype, token_major):
+    """The operator takes q's chunk means in a read-only pass of its own and k's in the pass that writes the fragment
+    order; permute + pool + score through the separate entry points (bsa_interface.py:547-548, 650-652 as
+    the reference runs them) must give the same score bits and the same selection, on a grid with padding on two
+    axes, for head-major tensors and for the token-major views a QKV projection leaves."""
+    latent, B, H = (6, 10, 13), 2, 3
+    S = latent[0] * latent[1] * latent[2]
+    g = torch.Generator().manual_seed(71)
+    if token_major:
+        qkv = torch.randn(B, S, 3, H, 128, generator=g).to(dtype).cuda()
+        q, k, v = qkv.permute(2, 0, 3, 1, 4).unbind(0)
+    else:
+        q, k, v = (torch.randn(B, H, S, 128, generator=g).to(dtype).cuda() for _ in range(3))
+    bi = I()
+    o, idx, lens, score = bi._bsa_3d(q, k, v, latent, latent, 0.75, (4, 4, 4), (4, 4, 4), True)
+    _, q_cmp, _ = bi._permute(q, latent, (4, 4, 4), want_pooled=True)
+    _, k_cmp, _ = bi._permute(k, latent, (4, 4, 4), want_pooled=True)
+    idx2, lens2, score2 = bi._score_topk(q_cmp, k_cmp, idx.shape[-1])
+    assert torch.equal(score.view(torch.int16), score2.view(torch.int16))
+    assert torch.equal(idx, idx2) and torch.equal(lens, lens2)
+
+
 def test_480p_two_heads():
     latent = (24, 30, 52)
     q, k, v = seeded_qkv(1, 1, 2, 37440, 37440, 128, torch.bfloat16)
