@@ -268,6 +268,32 @@ int bsa_bwd(const void* q, const void* k, const void* v, const void* o, const vo
             void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Backward of bsa_fwd_3d_lse on the operator's own tensors: what _attention_bsa.backward (bsa:570-596) computes
+ * for the q, k, v that flash_attn_bsa_3d rearranged (bsa:650-652, whose gradient is the inverse rearrangement), with
+ * every tensor left in (T, H, W) token order.  Same arithmetic and rounding points as bsa_bwd.
+ *   q, o, d_o, dq [B, Hn, Tq*Hq*Wq, D] and k, v, dk, dv [B, Hn, Tk*Hk*Wk, D]: element strides as in bsa_fwd_3d,
+ *   bf16 / fp16, D == 128, 16-byte aligned; lse [B, Hn, Tq*Hq*Wq] fp32 contiguous and idx [B, Hn, nbq, idx_stride],
+ *   lens [B, Hn, nbq] as bsa_fwd_3d_lse returned them (blocks counted in the padded chunk grids).  p->k_sel and
+ *   p->cdf_threshold are not read.  Padded keys give and get no gradient; dq, dk, dv are written at every token.
+ *   workspace: bsa_bwd_3d_workspace_bytes() bytes, 256-byte aligned: blocked-order copies of q, v and d_o (the kernels
+ *   stream their tiles as they lie in memory), the row tables of both grids, and bsa_bwd's workspace.  o, d_o, lse
+ *   and k are read through the row tables by the passes that take delta and the scaled k, and the kernels store the
+ *   gradient rows at their tokens: five of the eight rearrangements a caller of bsa_bwd would run are not made.
+ */
+size_t bsa_bwd_3d_workspace_bytes(const bsa_3d_params* p, int idx_stride);
+int bsa_bwd_3d(const bsa_3d_params* p,
+               const void* q, const int64_t q_strides[3],
+               const void* k, const int64_t k_strides[3],
+               const void* v, const int64_t v_strides[3],
+               const void* o, const int64_t o_strides[3],
+               const void* d_o, const int64_t do_strides[3],
+               const float* lse, const int32_t* idx, const int32_t* lens, int idx_stride,
+               void* dq, const int64_t dq_strides[3],
+               void* dk, const int64_t dk_strides[3],
+               void* dv, const int64_t dv_strides[3],
+               void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * bsa_fwd_3d without a workspace argument and without any allocation.  It has no counterpart in the
  * reference; it is for callers that cannot allocate device memory around the call: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  What bsa_fwd_3d carves from its workspace

@@ -76,6 +76,78 @@ __global__ __launch_bounds__(256) void bwd_scale_kernel(const T* __restrict__ k,
     *reinterpret_cast<V8*>(ks + i * 8) = x;
 }
 
+// Where a gradient row goes when the caller's tensors are in token order: the token of every blocked-order slot of one
+// (batch, head) (-1: padding, nothing is stored) and the element strides of the destination.  rows null: blocked order.
+struct BwdStore {
+    const int32_t* rows;
+    int64_t sB, sH, sS;
+    int Hn;
+};
+template <typename T>
+__device__ __forceinline__ T* store_row(T* blocked, const BwdStore& w, int64_t bh, int64_t rows_per_bh, int64_t slot) {
+    if (w.rows == nullptr) return blocked + (bh * rows_per_bh + slot) * kD;
+    const int32_t token = w.rows[slot];
+    if (token < 0) return nullptr;
+    return blocked + (bh / w.Hn) * w.sB + (bh % w.Hn) * w.sH + (int64_t)token * w.sS;
+}
+
+// bwd_rows_kernel for o, dO and lse in token order (element strides oS / dS per token, lse [B * Hn][tokens]): the
+// same delta and m2 per blocked-order slot, and dO copied into blocked order on the way (padded slots: a zero row,
+// delta 0, m2 -inf, so that their p is 0).  One 16-lane group per slot.
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_rows_thw_kernel(const T* __restrict__ o, int64_t oB, int64_t oH, int64_t oS,
+                                                           const T* __restrict__ dout, int64_t dB, int64_t dH, int64_t dS,
+                                                           const float* __restrict__ lse, const int32_t* __restrict__ rows,
+                                                           int64_t tokens, int Hn, int64_t slots, T* __restrict__ dout_blocked,
+                                                           float* __restrict__ delta, float* __restrict__ m2, int64_t total) {
+    typedef typename Vec8<T>::type V8;
+    const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int c = threadIdx.x & 15;
+    if (row >= total) return;                                    // whole 16-lane groups leave together
+    const int64_t bh = row / slots;
+    const int32_t token = rows[row - bh * slots];
+    float s = 0.f;
+    V8 b;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] = (T)0.f;
+    if (token >= 0) {
+        const int64_t at = (bh / Hn), hd = (bh % Hn);
+        const V8 a = *reinterpret_cast<const V8*>(o + at * oB + hd * oH + (int64_t)token * oS + c * 8);
+        b = *reinterpret_cast<const V8*>(dout + at * dB + hd * dH + (int64_t)token * dS + c * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s += (float)a[e] * (float)b[e];
+    }
+    *reinterpret_cast<V8*>(dout_blocked + row * kD + c * 8) = b;
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off);
+    if (c == 0) {
+        delta[row] = -s;
+        const float l = token >= 0 ? lse[bh * tokens + token] : -INFINITY;
+        m2[row] = l == -INFINITY ? -INFINITY : -(l * kRcpLn2);
+    }
+}
+
+// bwd_scale_kernel for k in token order: k_s in blocked order, padded slots zero.  One 16-lane group per slot.
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_scale_thw_kernel(const T* __restrict__ k, int64_t kB, int64_t kH, int64_t kS,
+                                                            const int32_t* __restrict__ rows, int Hn, int64_t slots,
+                                                            T* __restrict__ ks, float c, int64_t total) {
+    typedef typename Vec8<T>::type V8;
+    const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    if (row >= total) return;
+    const int64_t bh = row / slots;
+    const int32_t token = rows[row - bh * slots];
+    V8 x;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = (T)0.f;
+    if (token >= 0) {
+        x = *reinterpret_cast<const V8*>(k + (bh / Hn) * kB + (bh % Hn) * kH + (int64_t)token * kS + (threadIdx.x & 15) * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * c);
+    }
+    *reinterpret_cast<V8*>(ks + row * kD + (threadIdx.x & 15) * 8) = x;
+}
+
 __global__ void bwd_zero_kernel(uint32_t* p, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0u;
@@ -148,8 +220,8 @@ __device__ inline void mfma_from_v(f32x16& acc, f16x8 a, f16x8 b, const f32x16& 
 constexpr int kDqStage = 2 * kBwdHalfTileBytes;              // K_s rows and V rows of 32 keys
 constexpr int kDqRingLds = 2 * kDqStage;
 
-// kMasked: the caller has a validity word per KV tile (padding keys exist); without one the test of every P element
-// is compiled out - three of its seven instructions, in a kernel whose time is its instruction issue.
+// kMasked: the caller has a validity word per KV tile (padding keys exist); they cost nothing per P element (see
+// start_block below), only the look-up of the word per half tile.
 template <typename T, bool kMasked>
 __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q, const T* __restrict__ dout,
                                                         const T* __restrict__ ks, const T* __restrict__ v,
@@ -157,7 +229,7 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
                                                         const int32_t* __restrict__ idx, const int32_t* __restrict__ lens,
                                                         const uint64_t* __restrict__ tile_valid, T* __restrict__ dq,
                                                         int64_t Sq, int64_t Sk, int bs_q, int bs_k, int stride, int item_begin,
-                                                        int item_end, int round) {
+                                                        int item_end, int round, BwdStore dq_to) {
     typedef typename Vec8<T>::type V8;
     extern __shared__ __attribute__((aligned(1024))) char dq_ring[];
     const int lane = threadIdx.x, lr = lane & 31, lh = lane >> 5;
@@ -254,15 +326,29 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
         }
     };
     // accumulator i <-> key 8 (i / 4) + 4 lh + i % 4 of the half, query lr (+ 32)
-    auto exponentials = [&](f32x16 (&s)[2], f32x16 (&dp)[2], uint32_t hv, int qq, int i0, int count) {
+    auto exponentials = [&](f32x16 (&s)[2], f32x16 (&dp)[2], int qq, int i0, int count) {
 #pragma unroll
         for (int i = i0; i < i0 + count; ++i) {
-            float p = __builtin_amdgcn_exp2f(s[qq][i]);              // s holds S^T - M2
-            if (kMasked) {
-                const int key = 8 * (i / 4) + 4 * lh + (i % 4);
-                if (!((hv >> key) & 1u)) p = 0.f;
-            }
+            const float p = __builtin_amdgcn_exp2f(s[qq][i]);        // s holds S^T - M2, -inf for a padded key
             s[qq][i] = p * (dp[qq][i] + d_row[qq]);
+        }
+    };
+    // Padded keys: the chain of a half tile that holds any starts from -inf in their accumulators instead of -M2, so
+    // their p is exp2(-inf) = 0 and the exponentials test nothing.  Such half tiles are the few at the upper edges of
+    // the grid; the start block is rebuilt only when the validity of the half in hand differs from all-valid or the
+    // one before did.
+    bool start_masked = false;
+    auto start_block = [&](uint32_t hv) {
+        if (!kMasked) return;
+        const bool edge = hv != ~0u;
+        if (!edge && !start_masked) return;
+        start_masked = edge;
+        const uint32_t mine = hv >> (4 * lh);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const bool ok = (mine >> (8 * (i / 4) + (i % 4))) & 1u;
+            neg_m[0][i] = ok ? m_row[0] : -INFINITY;
+            neg_m[1][i] = ok ? m_row[1] : -INFINITY;
         }
     };
     // S^T and dP^T of half hp (both query halves) into (s, dp); between its groups of four MFMAs the exponentials of
@@ -306,18 +392,20 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
             }
         }
     };
-    auto valid_half = [&](int hp) -> uint32_t {
+    auto valid_half = [&](int hp) -> uint32_t {                   // the same in every lane
         if (!kMasked) return ~0u;
         const uint64_t w = tile_valid[tile_at(min(hp, nhalves - 1) >> 1)];
-        return (uint32_t)(w >> (32 * (hp & 1)));
+        return (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(w >> (32 * (hp & 1))));
     };
+    uint32_t hv_ahead = ~0u;
     // (s, dp): this half, products done; (ns, ndp): the next half
     auto step = [&](int hp, f32x16 (&s)[2], f32x16 (&dp)[2], f32x16 (&ns)[2], f32x16 (&ndp)[2]) {
-        const uint32_t hv = valid_half(hp);
+        start_block(hv_ahead);                   // validity of half hp + 1, asked for a step ago
+        hv_ahead = valid_half(hp + 2);
         // The next half's rows must have landed; the stage that this half was read from (rows and transposed
         // fragments are in registers) takes half hp + 2.
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        products(hp + 1, ns, ndp, [&]() { issue(hp + 2); }, [&](int c) { exponentials(s, dp, hv, c >> 2, 4 * (c & 3), 4); });
+        products(hp + 1, ns, ndp, [&]() { issue(hp + 2); }, [&](int c) { exponentials(s, dp, c >> 2, 4 * (c & 3), 4); });
         __builtin_amdgcn_sched_barrier(0);
         gradients(s);
         __builtin_amdgcn_sched_barrier(0);
@@ -332,6 +420,8 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
         issue(0);
         issue(1);
         asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        start_block(valid_half(0));
+        hv_ahead = valid_half(1);
         products(0, sa, dpa, [&]() {}, [&](int) {});
         take_transposed(0);
         asm volatile("s_nop 15\n\ts_nop 7\n\ts_waitcnt lgkmcnt(0)" ::: "memory");
@@ -344,7 +434,8 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
     // accumulator i of d tile t <-> d = 32 t + 8 (i / 4) + 4 lh + i % 4, query lr (+ 32)
 #pragma unroll
     for (int qq = 0; qq < 2; ++qq) {
-        T* out = dq + (bh * Sq + qrow0 + 32 * qq + lr) * kD;
+        T* out = store_row(dq, dq_to, bh, Sq, qrow0 + 32 * qq + lr);
+        if (out == nullptr) continue;                            // a padded slot of a token-order destination
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -384,7 +475,8 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
                                                        const uint32_t* __restrict__ bits,
                                                        const uint64_t* __restrict__ tile_valid, T* __restrict__ dk,
                                                        T* __restrict__ dv, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int words,
-                                                       float dk_scale, const int32_t* __restrict__ order, int n_items, int round) {
+                                                       float dk_scale, const int32_t* __restrict__ order, int n_items, int round,
+                                                       BwdStore dk_to, BwdStore dv_to) {
     typedef typename Vec8<T>::type V8;
     extern __shared__ __attribute__((aligned(1024))) char bwd_lds[];
     const int lane = threadIdx.x & 63, lr = lane & 31, lh = lane >> 5;
@@ -623,20 +715,23 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
     }
     // accumulator i of d tile t <-> d = 32 t + 8 (i / 4) + 4 lh + i % 4, key lr
     {
-        const int64_t row = bh * Sk + krow0 + 32 * wave + lr;
+        T* out_k = store_row(dk, dk_to, bh, Sk, krow0 + 32 * wave + lr);
+        T* out_v = store_row(dv, dv_to, bh, Sk, krow0 + 32 * wave + lr);
+        if (out_k != nullptr && out_v != nullptr) {              // both or neither: one row table serves dk and dv
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                T xk[4], xv[4];
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    T xk[4], xv[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    xk[j] = (T)(acc_dk[t][4 * g4 + j] * dk_scale);
-                    xv[j] = (T)acc_dv[t][4 * g4 + j];
+                    for (int j = 0; j < 4; ++j) {
+                        xk[j] = (T)(acc_dk[t][4 * g4 + j] * dk_scale);
+                        xv[j] = (T)acc_dv[t][4 * g4 + j];
+                    }
+                    *reinterpret_cast<uint2*>(out_k + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(xk);
+                    *reinterpret_cast<uint2*>(out_v + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(xv);
                 }
-                *reinterpret_cast<uint2*>(dk + row * kD + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(xk);
-                *reinterpret_cast<uint2*>(dv + row * kD + 32 * t + 8 * g4 + 4 * lh) = *reinterpret_cast<const uint2*>(xv);
-            }
+        }
     }
 }
 
@@ -660,7 +755,7 @@ size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int 
 hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
                       const int32_t* idx, const int32_t* lens, const uint64_t* tile_valid, void* dq, void* dk, void* dv,
                       int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride, float sm_scale, int dtype,
-                      void* workspace, hipStream_t st) {
+                      void* workspace, hipStream_t st, const BwdThw* thw) {
     const size_t bh = (size_t)B * Hn;
     auto up = [](size_t x) { return (x + 255) / 256 * 256; };
     char* ws = static_cast<char*>(workspace);
@@ -677,7 +772,30 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
 
     const int64_t qrows = (int64_t)bh * Sq, krows = (int64_t)bh * Sk;
     const float c = sm_scale * kRcpLn2;
-    if (dtype == BSA_BF16) {
+    BwdStore dq_to = {nullptr, 0, 0, 0, Hn}, dk_to = dq_to, dv_to = dq_to;
+    if (thw != nullptr) {
+        // o, dO, lse and k in token order: the two passes read them through the row tables, and dO comes out in
+        // blocked order for the kernels; q and v are the caller's blocked-order copies
+        dq_to = {thw->q_rows, thw->dq_st[0], thw->dq_st[1], thw->dq_st[2], Hn};
+        dk_to = {thw->k_rows, thw->dk_st[0], thw->dk_st[1], thw->dk_st[2], Hn};
+        dv_to = {thw->k_rows, thw->dv_st[0], thw->dv_st[1], thw->dv_st[2], Hn};
+        dq = thw->dq; dk = thw->dk; dv = thw->dv;
+        dout = thw->dout_blocked;
+        const dim3 gq((unsigned)((qrows + 15) / 16)), gk((unsigned)((krows + 15) / 16)), blk(256);
+        if (dtype == BSA_BF16) {
+            hipLaunchKernelGGL((bwd_rows_thw_kernel<__bf16>), gq, blk, 0, st, (const __bf16*)thw->o, thw->o_st[0], thw->o_st[1], thw->o_st[2],
+                               (const __bf16*)thw->dout, thw->do_st[0], thw->do_st[1], thw->do_st[2], thw->lse, thw->q_rows, thw->q_tokens, Hn,
+                               Sq, (__bf16*)thw->dout_blocked, delta, m2, qrows);
+            hipLaunchKernelGGL((bwd_scale_thw_kernel<__bf16>), gk, blk, 0, st, (const __bf16*)thw->k, thw->k_st[0], thw->k_st[1], thw->k_st[2],
+                               thw->k_rows, Hn, Sk, (__bf16*)ks, c, krows);
+        } else {
+            hipLaunchKernelGGL((bwd_rows_thw_kernel<_Float16>), gq, blk, 0, st, (const _Float16*)thw->o, thw->o_st[0], thw->o_st[1], thw->o_st[2],
+                               (const _Float16*)thw->dout, thw->do_st[0], thw->do_st[1], thw->do_st[2], thw->lse, thw->q_rows, thw->q_tokens, Hn,
+                               Sq, (_Float16*)thw->dout_blocked, delta, m2, qrows);
+            hipLaunchKernelGGL((bwd_scale_thw_kernel<_Float16>), gk, blk, 0, st, (const _Float16*)thw->k, thw->k_st[0], thw->k_st[1], thw->k_st[2],
+                               thw->k_rows, Hn, Sk, (_Float16*)ks, c, krows);
+        }
+    } else if (dtype == BSA_BF16) {
         hipLaunchKernelGGL((bwd_rows_kernel<__bf16>), dim3((unsigned)((qrows + 15) / 16)), dim3(256), 0, st, (const __bf16*)o,
                            (const __bf16*)dout, lse, delta, m2, qrows);
         hipLaunchKernelGGL((bwd_scale_kernel<__bf16>), dim3((unsigned)((krows * 16 + 255) / 256)), dim3(256), 0, st,
@@ -731,40 +849,40 @@ hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o
             if (tile_valid != nullptr)
                 hipLaunchKernelGGL((bwd_dq_lds_kernel<__bf16, true>), dim3(end - first), block, kDqRingLds, st, (const __bf16*)q,
                                    (const __bf16*)dout, (const __bf16*)ks, (const __bf16*)v, m2, delta, paced, lens, tile_valid, (__bf16*)dq, Sq, Sk,
-                                   bs_q, bs_k, idx_stride, first, end, round);
+                                   bs_q, bs_k, idx_stride, first, end, round, dq_to);
             else
                 hipLaunchKernelGGL((bwd_dq_lds_kernel<__bf16, false>), dim3(end - first), block, kDqRingLds, st, (const __bf16*)q,
                                    (const __bf16*)dout, (const __bf16*)ks, (const __bf16*)v, m2, delta, paced, lens, tile_valid, (__bf16*)dq, Sq, Sk,
-                                   bs_q, bs_k, idx_stride, first, end, round);
+                                   bs_q, bs_k, idx_stride, first, end, round, dq_to);
         }
         if (masked)
             hipLaunchKernelGGL((bwd_dkdv_kernel<__bf16, true>), grid_k, dim3(128), lds, st, (const __bf16*)q, (const __bf16*)dout,
                                (const __bf16*)ks, (const __bf16*)v, m2, delta, bits, tile_valid, (__bf16*)dk, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words,
-                               sm_scale, order, total_k, round);
+                               sm_scale, order, total_k, round, dk_to, dv_to);
         else
             hipLaunchKernelGGL((bwd_dkdv_kernel<__bf16, false>), grid_k, dim3(128), lds, st, (const __bf16*)q, (const __bf16*)dout,
                                (const __bf16*)ks, (const __bf16*)v, m2, delta, bits, tile_valid, (__bf16*)dk, (__bf16*)dv, Sq, Sk, bs_q, bs_k, words,
-                               sm_scale, order, total_k, round);
+                               sm_scale, order, total_k, round, dk_to, dv_to);
     } else {
         for (int first = 0; first < total_q; first += span) {
             const int end = first + span < total_q ? first + span : total_q;
             if (tile_valid != nullptr)
                 hipLaunchKernelGGL((bwd_dq_lds_kernel<_Float16, true>), dim3(end - first), block, kDqRingLds, st, (const _Float16*)q,
                                    (const _Float16*)dout, (const _Float16*)ks, (const _Float16*)v, m2, delta, paced, lens, tile_valid, (_Float16*)dq,
-                                   Sq, Sk, bs_q, bs_k, idx_stride, first, end, round);
+                                   Sq, Sk, bs_q, bs_k, idx_stride, first, end, round, dq_to);
             else
                 hipLaunchKernelGGL((bwd_dq_lds_kernel<_Float16, false>), dim3(end - first), block, kDqRingLds, st, (const _Float16*)q,
                                    (const _Float16*)dout, (const _Float16*)ks, (const _Float16*)v, m2, delta, paced, lens, tile_valid, (_Float16*)dq,
-                                   Sq, Sk, bs_q, bs_k, idx_stride, first, end, round);
+                                   Sq, Sk, bs_q, bs_k, idx_stride, first, end, round, dq_to);
         }
         if (masked)
             hipLaunchKernelGGL((bwd_dkdv_kernel<_Float16, true>), grid_k, dim3(128), lds, st, (const _Float16*)q, (const _Float16*)dout,
                                (const _Float16*)ks, (const _Float16*)v, m2, delta, bits, tile_valid, (_Float16*)dk, (_Float16*)dv, Sq, Sk, bs_q,
-                               bs_k, words, sm_scale, order, total_k, round);
+                               bs_k, words, sm_scale, order, total_k, round, dk_to, dv_to);
         else
             hipLaunchKernelGGL((bwd_dkdv_kernel<_Float16, false>), grid_k, dim3(128), lds, st, (const _Float16*)q, (const _Float16*)dout,
                                (const _Float16*)ks, (const _Float16*)v, m2, delta, bits, tile_valid, (_Float16*)dk, (_Float16*)dv, Sq, Sk, bs_q,
-                               bs_k, words, sm_scale, order, total_k, round);
+                               bs_k, words, sm_scale, order, total_k, round, dk_to, dv_to);
     }
     return hipGetLastError();
 }

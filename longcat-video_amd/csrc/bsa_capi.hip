@@ -788,4 +788,92 @@ int bsa_fwd_3d_static(const bsa_3d_params* p, const void* q, const int64_t q_str
     return rc;
 }
 
+// ---- backward of the operator on token-order tensors ------------------------
+namespace {
+struct Bwd3dPlan {
+    Grid3 gq, gk;
+    int64_t Sqp, Skp;
+    size_t off_qp, off_vp, off_dop, off_qrows, off_krows, off_valid, off_bwd, total;
+};
+int make_bwd3d_plan(const bsa_3d_params* p, int idx_stride, Bwd3dPlan* pl) {
+    if (!p) return set_error(BSA_ERR_BAD_ARG, "params are null");
+    BSA_TRY(check_row(p->D, p->dtype));
+    BSA_TRY(check_grid(p->B, p->Hn, p->Tq, p->Hq, p->Wq, p->tq, p->hq, p->wq));
+    BSA_TRY(check_grid(p->B, p->Hn, p->Tk, p->Hk, p->Wk, p->tk, p->hk, p->wk));
+    pl->gq = make_grid(p->Tq, p->Hq, p->Wq, p->tq, p->hq, p->wq);
+    pl->gk = make_grid(p->Tk, p->Hk, p->Wk, p->tk, p->hk, p->wk);
+    pl->Sqp = (int64_t)pl->gq.blocks() * pl->gq.chunk();
+    pl->Skp = (int64_t)pl->gk.blocks() * pl->gk.chunk();
+    BSA_TRY(check_bwd_shape(p->B, p->Hn, pl->Sqp, pl->Skp, p->D, pl->gq.chunk(), pl->gk.chunk(), p->dtype));
+    if (idx_stride <= 0 || idx_stride > 4096) return set_error(BSA_ERR_BAD_ARG, "bwd_3d: idx_stride=%d outside [1, 4096]", idx_stride);
+    if (!(p->sm_scale > 0.f) || !std::isfinite(p->sm_scale)) return set_error(BSA_ERR_BAD_ARG, "bwd_3d: sm_scale must be positive and finite");
+    const size_t bh = (size_t)p->B * p->Hn, row = (size_t)p->D * dtype_size(p->dtype);
+    size_t off = 0;
+    auto take = [&](size_t bytes) { const size_t o = off; off += up256(bytes); return o; };
+    pl->off_qp = take(bh * pl->Sqp * row);
+    pl->off_vp = take(bh * pl->Skp * row);
+    pl->off_dop = take(bh * pl->Sqp * row);
+    pl->off_qrows = take((size_t)pl->Sqp * sizeof(int32_t));
+    pl->off_krows = take((size_t)pl->Skp * sizeof(int32_t));
+    pl->off_valid = take((size_t)(pl->Skp / 64) * sizeof(uint64_t));
+    pl->off_bwd = take(bwd_workspace_bytes(p->B, p->Hn, pl->Sqp, pl->Skp, pl->gq.chunk(), pl->gk.chunk(), idx_stride));
+    pl->total = off;
+    return BSA_OK;
+}
+}  // namespace
+
+size_t bsa_bwd_3d_workspace_bytes(const bsa_3d_params* p, int idx_stride) {
+    Bwd3dPlan pl;
+    if (make_bwd3d_plan(p, idx_stride, &pl) != BSA_OK) return 0;
+    return pl.total;
+}
+
+int bsa_bwd_3d(const bsa_3d_params* p, const void* q, const int64_t q_strides[3], const void* k, const int64_t k_strides[3],
+               const void* v, const int64_t v_strides[3], const void* o, const int64_t o_strides[3], const void* d_o,
+               const int64_t do_strides[3], const float* lse, const int32_t* idx, const int32_t* lens, int idx_stride,
+               void* dq, const int64_t dq_strides[3], void* dk, const int64_t dk_strides[3], void* dv,
+               const int64_t dv_strides[3], void* workspace, size_t workspace_bytes, void* stream) {
+    Bwd3dPlan pl;
+    BSA_TRY(make_bwd3d_plan(p, idx_stride, &pl));
+    if (!lse || !idx || !lens) return set_error(BSA_ERR_BAD_ARG, "bwd_3d: lse, idx or lens is null");
+    BSA_TRY(check_tensor(q, q_strides, p, "q"));
+    BSA_TRY(check_tensor(k, k_strides, p, "k"));
+    BSA_TRY(check_tensor(v, v_strides, p, "v"));
+    BSA_TRY(check_tensor(o, o_strides, p, "o"));
+    BSA_TRY(check_tensor(d_o, do_strides, p, "d_o"));
+    BSA_TRY(check_tensor(dq, dq_strides, p, "dq"));
+    BSA_TRY(check_tensor(dk, dk_strides, p, "dk"));
+    BSA_TRY(check_tensor(dv, dv_strides, p, "dv"));
+    if (!workspace) return set_error(BSA_ERR_BAD_ARG, "bwd_3d: workspace is null");
+    if (workspace_bytes < pl.total) return set_error(BSA_ERR_WORKSPACE, "bwd_3d: workspace of %zu bytes, %zu needed", workspace_bytes, pl.total);
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return set_error(BSA_ERR_BAD_ARG, "bwd_3d: workspace must be 256-byte aligned");
+    char* ws = static_cast<char*>(workspace);
+    hipStream_t st = (hipStream_t)stream;
+    int32_t* q_rows = reinterpret_cast<int32_t*>(ws + pl.off_qrows);
+    int32_t* k_rows = reinterpret_cast<int32_t*>(ws + pl.off_krows);
+    uint64_t* valid = reinterpret_cast<uint64_t*>(ws + pl.off_valid);
+    // q and v in blocked order (the kernels stream their tiles as they lie in memory); the passes write the row tables
+    // of both grids and the validity words of the keys on the way
+    hipError_t e = launch_permute(q, q_strides, ws + pl.off_qp, nullptr, nullptr, p->B, p->Hn, pl.gq, p->D, p->dtype, st, false, q_rows);
+    if (e != hipSuccess) return hip_fail(e, "bwd_3d: permute q");
+    e = launch_permute(v, v_strides, ws + pl.off_vp, nullptr, valid, p->B, p->Hn, pl.gk, p->D, p->dtype, st, false, k_rows);
+    if (e != hipSuccess) return hip_fail(e, "bwd_3d: permute v");
+    BwdThw t;
+    t.q_rows = q_rows;
+    t.k_rows = k_rows;
+    t.q_tokens = (int64_t)p->Tq * p->Hq * p->Wq;
+    t.k_tokens = (int64_t)p->Tk * p->Hk * p->Wk;
+    t.o = o; t.dout = d_o; t.lse = lse; t.k = k;
+    t.dout_blocked = ws + pl.off_dop;
+    t.dq = dq; t.dk = dk; t.dv = dv;
+    for (int i = 0; i < 3; ++i) {
+        t.o_st[i] = o_strides[i]; t.do_st[i] = do_strides[i]; t.k_st[i] = k_strides[i];
+        t.dq_st[i] = dq_strides[i]; t.dk_st[i] = dk_strides[i]; t.dv_st[i] = dv_strides[i];
+    }
+    e = launch_bwd(ws + pl.off_qp, nullptr, ws + pl.off_vp, nullptr, nullptr, nullptr, idx, lens, kv_padded(p) ? valid : nullptr, nullptr,
+                   nullptr, nullptr, p->B, p->Hn, pl.Sqp, pl.Skp, pl.gq.chunk(), pl.gk.chunk(), idx_stride, p->sm_scale, p->dtype,
+                   ws + pl.off_bwd, st, &t);
+    return e == hipSuccess ? BSA_OK : hip_fail(e, "bwd_3d launch");
+}
+
 }  // extern "C"

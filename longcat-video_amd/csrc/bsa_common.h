@@ -183,9 +183,26 @@ size_t frag_fallback_ints(int64_t items);
 // Backward of the blocked-order attention (bsa_bwd.hip), bf16 / fp16.  workspace: bwd_workspace_bytes() bytes.
 size_t bwd_workspace_bytes(int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride);
 int bwd_max_query_blocks();      // the dK / dV kernel stages a KV block's query blocks in LDS: Sq / bs_q may not exceed this
+// With `thw` the caller's o, dO, lse, k and the three gradients are in token order: the passes that take delta and k_s
+// read them through the row tables (token of every blocked-order slot of one (batch, head), -1 = padding) and the
+// kernels store the gradient rows at their tokens.  q and v are then blocked-order copies (launch_permute), and the
+// arguments k, o, dout, lse, dq, dk, dv of launch_bwd are not used.  Strides count elements.
+struct BwdThw {
+    const int32_t* q_rows;
+    const int32_t* k_rows;
+    int64_t q_tokens, k_tokens;       // real tokens per (batch, head)
+    const void* o; int64_t o_st[3];
+    const void* dout; int64_t do_st[3];
+    const float* lse;                 // [B * Hn][q_tokens]
+    const void* k; int64_t k_st[3];
+    void* dout_blocked;               // B * Hn * Sq rows of 128 elements
+    void* dq; int64_t dq_st[3];
+    void* dk; int64_t dk_st[3];
+    void* dv; int64_t dv_st[3];
+};
 hipError_t launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* dout, const float* lse,
                       const int32_t* idx, const int32_t* lens, const uint64_t* tile_valid, void* dq, void* dk, void* dv,
                       int B, int Hn, int64_t Sq, int64_t Sk, int bs_q, int bs_k, int idx_stride, float sm_scale, int dtype,
-                      void* workspace, hipStream_t st);
+                      void* workspace, hipStream_t st, const BwdThw* thw = nullptr);
 
 }  // namespace bsa

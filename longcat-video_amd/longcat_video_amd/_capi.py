@@ -55,6 +55,8 @@ SIGNATURES = {
     "bsa_fwd_fragment": (_i, [_p] * 8 + [_i, _i, _i64, _i64, _i, _i, _i, _i, _f, _i, _p, C.c_size_t, _p]),
     "bsa_bwd_workspace_bytes": (C.c_size_t, [_i, _i, _i64, _i64, _i, _i, _i, _i, _i]),
     "bsa_bwd": (_i, [_p] * 12 + [_i, _i, _i64, _i64, _i, _i, _i, _i, _f, _i, _p, C.c_size_t, _p]),
+    "bsa_bwd_3d_workspace_bytes": (C.c_size_t, [C.POINTER(Bsa3dParams), _i]),
+    "bsa_bwd_3d": (_i, [C.POINTER(Bsa3dParams)] + [_p, _strides] * 5 + [_p, _p, _p, _i] + [_p, _strides] * 3 + [_p, C.c_size_t, _p]),
     "bsa_workspace_bytes": (C.c_size_t, [C.POINTER(Bsa3dParams)]),
     "bsa_fwd_3d": (_i, [C.POINTER(Bsa3dParams), _p, _strides, _p, _strides, _p, _strides, _p, _strides,
                         _p, C.c_size_t, _p, _p, _p, _p]),

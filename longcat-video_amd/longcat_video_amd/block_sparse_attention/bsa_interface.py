@@ -603,9 +603,7 @@ def _slot_tokens(latent_shape, chunk, device) -> torch.Tensor:
 class _Bsa3dWithGrad(torch.autograd.Function):
     """The operator for inputs that require a gradient.  The forward is the forward of every other call - the same
     kernels on the same lists, the same bits (bsa_interface.py:538-568 runs one kernel with and without grad) - and
-    keeps the log-sum-exp and the lists it walked.  The backward moves q, k, v, o and dO into the blocked order in
-    which bsa_bwd takes them (bsa_interface.py:650-652; the permutes are each other's gradient) and the three
-    gradients back."""
+    keeps the log-sum-exp and the lists it walked.  The backward (bsa_bwd_3d) takes and returns token-order tensors."""
 
     @staticmethod
     def forward(ctx, q, k, v, latent_shape_q, latent_shape_k, sparsity, cdf_threshold, chunk_q, chunk_k):
@@ -619,21 +617,50 @@ class _Bsa3dWithGrad(torch.autograd.Function):
     def backward(ctx, do):
         q, k, v, o, lse, walk, lens = ctx.saved_tensors
         latent_q, latent_k, chunk_q, chunk_k, sm_scale = ctx.args
-        bs_q, bs_k = int(math.prod(chunk_q)), int(math.prod(chunk_k))
-        qp, _, _ = _permute(q, latent_q, chunk_q)
-        kp, _, valid = _permute(k, latent_k, chunk_k, want_valid=True)
-        vp, _, _ = _permute(v, latent_k, chunk_k)
-        op, _, _ = _permute(o, latent_q, chunk_q)
-        dop, _, _ = _permute(do, latent_q, chunk_q)                      # padded slots get a zero gradient
-        padded_k = kp.shape[2] != k.shape[2]
-        # lse in blocked order; a padded query slot has no keys as far as the backward is concerned (its p is 0)
-        slots = _slot_tokens(latent_q, chunk_q, q.device)
-        lse_p = torch.where(slots >= 0, lse[..., slots.clamp(min=0)], torch.full((), float("-inf"), device=q.device))
-        dqp, dkp, dvp = (torch.empty_like(t) for t in (qp, kp, vp))
-        attn_bwd_bsa_varlen(dop, qp, kp, vp, op, dqp, dkp, dvp, sm_scale, lse_p, walk, lens, bs_q, bs_k, None,
-                            valid if padded_k else None)
-        return (_unpermute(dqp, latent_q, chunk_q), _unpermute(dkp, latent_k, chunk_k), _unpermute(dvp, latent_k, chunk_k),
-                None, None, None, None, None, None)
+        return _bsa_3d_backward(do, q, k, v, o, lse, walk, lens, latent_q, latent_k, chunk_q, chunk_k, sm_scale) + (None,) * 6
+
+
+def _bsa_3d_backward(do, q, k, v, o, lse, walk, lens, latent_q, latent_k, chunk_q, chunk_k, sm_scale):
+    """bsa_bwd_3d: dq, dk, dv in token order from token-order tensors (bsa_interface.py:570-596 between the
+    rearrangements of :650-652 and :659, of which only those of q and v are made, inside the call)."""
+    _need_gpu(do, q, k, v, o)
+    B, H, Sq, D = q.shape
+    lib = _capi.load()
+    q, k, v, o, do = (_rows_ok(t) for t in (q, k, v, o, do))
+    prm = _capi.Bsa3dParams(B, H, D, _code(q), *latent_q, *latent_k, *chunk_q, *chunk_k, 0, float(sm_scale), 0.0)
+    width = walk.shape[3]
+    need = lib.bsa_bwd_3d_workspace_bytes(C.byref(prm), width)
+    if need == 0:        # the call itself names what is wrong with the shape
+        _capi.check(lib.bsa_bwd_3d(C.byref(prm), *([None] * 10), None, None, None, width, *([None] * 6), None, 0, None), "bsa_bwd_3d")
+        raise RuntimeError("bsa_bwd_3d: no workspace size for this problem")
+    ws = _workspace(need, q.device)
+    dq, dk, dv = (torch.empty(t.shape, dtype=t.dtype, device=t.device) for t in (q, k, v))
+    lse, walk, lens = lse.contiguous(), walk.contiguous(), lens.contiguous()
+    st = lambda t: _capi.strides3(t.stride()[:3])
+    with torch.cuda.device(q.device):
+        _capi.check(lib.bsa_bwd_3d(C.byref(prm), _ptr(q), st(q), _ptr(k), st(k), _ptr(v), st(v), _ptr(o), st(o), _ptr(do), st(do),
+                                   _ptr(lse), _ptr(walk), _ptr(lens), width, _ptr(dq), st(dq), _ptr(dk), st(dk), _ptr(dv), st(dv),
+                                   _ptr(ws), need, _stream(q)), "bsa_bwd_3d")
+    return dq, dk, dv
+
+
+def _bsa_3d_backward_by_rearranging(do, q, k, v, o, lse, walk, lens, latent_q, latent_k, chunk_q, chunk_k, sm_scale):
+    """The same gradients the way a caller of the blocked-order entry points gets them: five rearrangements in
+    (bsa_interface.py:650-652 and their like for o and dO), bsa_bwd, three out.  Kept for the tests."""
+    bs_q, bs_k = int(math.prod(chunk_q)), int(math.prod(chunk_k))
+    qp, _, _ = _permute(q, latent_q, chunk_q)
+    kp, _, valid = _permute(k, latent_k, chunk_k, want_valid=True)
+    vp, _, _ = _permute(v, latent_k, chunk_k)
+    op, _, _ = _permute(o, latent_q, chunk_q)
+    dop, _, _ = _permute(do, latent_q, chunk_q)                      # padded slots get a zero gradient
+    padded_k = kp.shape[2] != k.shape[2]
+    # lse in blocked order; a padded query slot has no keys as far as the backward is concerned (its p is 0)
+    slots = _slot_tokens(latent_q, chunk_q, q.device)
+    lse_p = torch.where(slots >= 0, lse[..., slots.clamp(min=0)], torch.full((), float("-inf"), device=q.device))
+    dqp, dkp, dvp = (torch.empty_like(t) for t in (qp, kp, vp))
+    attn_bwd_bsa_varlen(dop, qp, kp, vp, op, dqp, dkp, dvp, sm_scale, lse_p, walk, lens, bs_q, bs_k, None,
+                        valid if padded_k else None)
+    return _unpermute(dqp, latent_q, chunk_q), _unpermute(dkp, latent_k, chunk_k), _unpermute(dvp, latent_k, chunk_k)
 
 
 def _unpermute(xp, latent_shape, chunk):

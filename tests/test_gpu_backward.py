@@ -160,6 +160,41 @@ def test_autograd_through_the_operator_on_a_grid(shape):
         assert float(err.mean()) <= 2.0 ** -6 * float(w_thw.abs().mean())
 
 
+@pytest.mark.parametrize("dtype,lq,lk,chunk_q,chunk_k,token_major", [
+    (torch.bfloat16, (8, 8, 16), (8, 8, 16), (4, 4, 4), (4, 4, 4), False),      # no padding
+    (torch.bfloat16, (6, 10, 13), (6, 10, 13), (4, 4, 4), (4, 4, 4), True),     # padding on all axes, views of a projection
+    (torch.float16, (5, 9, 14), (5, 9, 14), (4, 4, 4), (4, 4, 4), False),
+    (torch.bfloat16, (4, 8, 12), (8, 8, 12), (4, 4, 4), (4, 4, 8), False),      # fewer queries than keys, 128-token key chunks
+    (torch.bfloat16, (7, 9, 17), (7, 9, 17), (4, 4, 8), (4, 4, 8), True),
+])
+def test_the_token_order_backward_equals_the_rearranging_route(dtype, lq, lk, chunk_q, chunk_k, token_major):
+    """bsa_bwd_3d reads o, dO, lse and k through the row tables and stores the gradients at their tokens; five
+    rearrangements (bsa_interface.py:650-652 and their like), bsa_bwd and three rearrangements back run the same kernels on
+    the same values, so the two must agree bit for bit - on padded grids, strided views, two batches."""
+    bi = I()
+    B, H = 2, 3
+    Sq, Sk = int(np.prod(lq)), int(np.prod(lk))
+    g = torch.Generator().manual_seed(11)
+    if token_major and Sq == Sk:
+        qkv = torch.randn(B, Sq, 3, H, 128, generator=g).to(dtype).cuda()
+        q, k, v = qkv.permute(2, 0, 3, 1, 4).unbind(0)
+    else:
+        q = torch.randn(B, H, Sq, 128, generator=g).to(dtype).cuda()
+        k, v = (torch.randn(B, H, Sk, 128, generator=g).to(dtype).cuda() for _ in range(2))
+    do = torch.randn(B, Sq, H, 128, generator=g).to(dtype).cuda().transpose(1, 2)          # a view, as a reshape upstream leaves it
+    o, walk, lens, lse = bi._bsa_3d(q, k, v, lq, lk, 0.5, chunk_q, chunk_k, for_backward=True)
+    args = (do, q, k, v, o, lse, walk, lens, lq, lk, chunk_q, chunk_k, 1 / math.sqrt(128))
+    got = bi._bsa_3d_backward(*args)
+    want = bi._bsa_3d_backward_by_rearranging(*args)
+    for a, b, name in zip(got, want, ("dq", "dk", "dv")):
+        assert a.shape == b.shape and a.is_contiguous()
+        assert torch.isfinite(a.float()).all(), name
+        assert torch.equal(a, b), (name, float((a.float() - b.float()).abs().max()))
+    again = bi._bsa_3d_backward(*args)
+    for a, b in zip(got, again):
+        assert torch.equal(a, b)
+
+
 def test_argument_checks():
     from longcat_video_amd import _capi
     lib = _capi.load()
@@ -176,3 +211,16 @@ def test_argument_checks():
     assert lib.bsa_bwd(*args, 1, 1, 64, 64, 96, 64, 64, 1, 0.1, _capi.BSA_BF16, p(ws), 1 << 20, None) == _capi.BSA_ERR_UNSUPPORTED
     args[0] = None
     assert lib.bsa_bwd(*args, 1, 1, 64, 64, 128, 64, 64, 1, 0.1, _capi.BSA_BF16, p(ws), 1 << 20, None) == _capi.BSA_ERR_BAD_ARG
+    # the token-order entry point
+    import ctypes as C
+    prm = _capi.Bsa3dParams(1, 1, 128, _capi.BSA_BF16, 4, 4, 4, 4, 4, 4, 4, 4, 4, 4, 4, 4, 0, 0.1, 0.0)
+    need = lib.bsa_bwd_3d_workspace_bytes(C.byref(prm), 1)
+    assert need > 3 * 64 * 128 * 2
+    bad = _capi.Bsa3dParams(1, 1, 128, _capi.BSA_F32, 4, 4, 4, 4, 4, 4, 4, 4, 4, 4, 4, 4, 0, 0.1, 0.0)
+    assert lib.bsa_bwd_3d_workspace_bytes(C.byref(bad), 1) == 0
+    assert lib.bsa_bwd_3d_workspace_bytes(C.byref(prm), 0) == 0
+    st = _capi.strides3((64 * 128, 64 * 128, 128))
+    call = lambda first, ws_bytes: lib.bsa_bwd_3d(C.byref(prm), first, st, p(t), st, p(t), st, p(t), st, p(t), st, p(f), p(i), p(i), 1,
+                                                  p(t), st, p(t), st, p(t), st, p(ws), ws_bytes, None)
+    assert call(p(t), 16) == _capi.BSA_ERR_WORKSPACE
+    assert call(None, 1 << 20) == _capi.BSA_ERR_BAD_ARG
