@@ -289,9 +289,11 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
         const int f = ((row << 1) & 14) | ((row >> 3) & 1);
         voff[i] = (uint32_t)(row * 256 + (((lane & 15) ^ f) << 4));
     }
+    uint32_t hv_ahead = ~0u;                     // validity of the keys of the half tile requested last
     auto issue = [&](int hp) {
         if (hp >= nhalves) return;
         const int64_t tile = (int64_t)__builtin_amdgcn_readfirstlane((int)tile_at(hp >> 1));
+        if (kMasked) hv_ahead = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(tile_valid[tile] >> (32 * (hp & 1))));
         const int64_t off = tile * kTileBytes + (hp & 1) * kBwdHalfTileBytes;
         const uint32_t dst = lds0 + (hp & 1) * kDqStage;
 #pragma unroll
@@ -392,16 +394,9 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
             }
         }
     };
-    auto valid_half = [&](int hp) -> uint32_t {                   // the same in every lane
-        if (!kMasked) return ~0u;
-        const uint64_t w = tile_valid[tile_at(min(hp, nhalves - 1) >> 1)];
-        return (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(w >> (32 * (hp & 1))));
-    };
-    uint32_t hv_ahead = ~0u;
     // (s, dp): this half, products done; (ns, ndp): the next half
     auto step = [&](int hp, f32x16 (&s)[2], f32x16 (&dp)[2], f32x16 (&ns)[2], f32x16 (&ndp)[2]) {
-        start_block(hv_ahead);                   // validity of half hp + 1, asked for a step ago
-        hv_ahead = valid_half(hp + 2);
+        start_block(hv_ahead);                   // validity of half hp + 1, looked up when its rows were requested
         // The next half's rows must have landed; the stage that this half was read from (rows and transposed
         // fragments are in registers) takes half hp + 2.
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -418,10 +413,10 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
         f32x16 sa[2], dpa[2], sb[2], dpb[2];
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // the Q / dO rows: from here on the DMA loads are counted by hand
         issue(0);
+        const uint32_t hv_first = hv_ahead;
         issue(1);
         asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-        start_block(valid_half(0));
-        hv_ahead = valid_half(1);
+        start_block(hv_first);
         products(0, sa, dpa, [&]() {}, [&](int) {});
         take_transposed(0);
         asm volatile("s_nop 15\n\ts_nop 7\n\ts_waitcnt lgkmcnt(0)" ::: "memory");
