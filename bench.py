@@ -247,8 +247,8 @@ def measure_c4(torch, steps, warmup, settle, where):
 
 
 def sample_clocks(torch, fn, seconds=3.0):
-    """Runs fn back to back for `seconds` while a thread asks `rocm-smi` (a child process) for the shader clock and the
-    board power every 0.3 s: what the kernel settles at once the power controller has acted."""
+    """Runs fn back to back for `seconds` while a thread asks `rocm-smi` (a child process) for the shader clock every
+    0.3 s: what the kernel settles at once the power controller has acted."""
     import re
     import subprocess
     import threading
@@ -257,12 +257,11 @@ def sample_clocks(torch, fn, seconds=3.0):
     def sampler():
         while not stop.is_set():
             try:
-                text = subprocess.run(["rocm-smi", "--showclocks", "--showpower"], capture_output=True, text=True, timeout=10).stdout
+                text = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=10).stdout
                 sclk = re.findall(r"sclk clock level: \d+: \((\d+)Mhz\)", text)
-                watt = re.findall(r"Power[^\n]*\(W\)[^\n]*?:\s*([\d.]+)", text)
-                samples.append((int(sclk[0]) if sclk else None, float(watt[0]) if watt else None))
+                samples.append(int(sclk[0]) if sclk else None)
             except Exception:
-                samples.append((None, None))
+                samples.append(None)
             stop.wait(0.3)
     th = threading.Thread(target=sampler)
     t0, calls = time.perf_counter(), 0
@@ -276,8 +275,8 @@ def sample_clocks(torch, fn, seconds=3.0):
     stop.set()
     th.join()
     samples = samples[1:] or samples                # the first reading may precede the load
-    return {"ms_per_call_in_this_loop": round(ms, 4), "sclk_mhz": [a for a, _ in samples], "power_w": [b for _, b in samples],
-            "nominal_sclk_mhz": 2400, "how": "rocm-smi --showclocks --showpower every 0.3 s while the attention kernel runs back to back"}
+    return {"ms_per_call_in_this_loop": round(ms, 4), "sclk_mhz": samples, "nominal_sclk_mhz": 2400,
+            "how": "rocm-smi --showclocks every 0.3 s while the attention kernel runs back to back"}
 
 
 def measure_operator(torch, workload, steps, warmup, settle, where, coherent=False, clocks=None):
@@ -612,8 +611,8 @@ def main():
     ap.add_argument("--no-other-configs", action="store_true",
                     help="c3: leave out the attention-kernel figures of c2 and c4 that the default line carries beside its own")
     ap.add_argument("--clocks", action="store_true",
-                    help="c2, c3: also run the attention kernel back to back for three seconds and report the shader clock and "
-                         "board power that rocm-smi shows meanwhile")
+                    help="c2, c3: also run the attention kernel back to back for three seconds and report the shader clock "
+                         "that rocm-smi shows meanwhile")
     ap.add_argument("--data", default="random", choices=["random", "coherent"],
                     help="random (the benchmark's definition) or spatially coherent q/k (c2, c3 only; no CPU baseline)")
     args = ap.parse_args()
