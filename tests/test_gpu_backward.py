@@ -160,6 +160,41 @@ def test_autograd_through_the_operator_on_a_grid(shape):
         assert float(err.mean()) <= 2.0 ** -6 * float(w_thw.abs().mean())
 
 
+def test_autograd_through_the_operator_with_the_cdf_rule():
+    """Lists of unequal length (bsa_interface.py:226-266 feeding :570-596) on a padded grid: gradients in (T, H, W) order
+    against autograd through fp32 attention with the token-level mask of the GPU's own selection."""
+    bi = I()
+    shape, chunk = (6, 10, 14), (4, 4, 4)
+    S = int(np.prod(shape))
+    g = torch.Generator().manual_seed(12)
+    q, k, v = (torch.randn(1, 2, S, 128, generator=g) for _ in range(3))
+    # a common direction whose weight varies over the grid: the pooled scores then differ from row to row by more than
+    # noise, and so do the numbers of blocks the rule keeps
+    pos = torch.arange(S).view(1, 1, S, 1).float()
+    q = q + 0.6 * torch.sin(pos / 37.0) * torch.ones(128)
+    k = k + 0.6 * torch.cos(pos / 53.0) * torch.ones(128)
+    q, k, v = (t.bfloat16().cuda().requires_grad_(True) for t in (q, k, v))
+    do = torch.randn(1, 2, S, 128, generator=g).bfloat16().cuda()
+    prm = dict(sparsity=0.75, cdf_threshold=0.6, chunk_3d_shape_q=list(chunk), chunk_3d_shape_k=list(chunk))
+    o = bi.flash_attn_bsa_3d(q, k, v, shape, shape, **prm)
+    o.backward(do)
+    with torch.no_grad():
+        o_plain, idx, lens, _ = bi._bsa_3d(q, k, v, shape, shape, 0.75, chunk, chunk, want_selection=True, cdf_threshold=0.6)
+    assert torch.equal(o.detach(), o_plain)
+    lens_c = lens.cpu()
+    assert int(lens_c.min()) < int(lens_c.max())                          # the rule did give lists of unequal length
+    qp, kp, vp, dop = (O.rearrange_thw_to_3d_block(t.detach().cpu(), shape, chunk) for t in (q, k, v, do))
+    nb = qp.shape[2] // 64
+    mask = O.block_mask_from_indices(idx.cpu().long().clamp(min=0), lens_c, nb)
+    valid = torch.from_numpy(O.slot_validity(shape, chunk))
+    wq, wk, wv = O.masked_dense_attention_autograd(qp, kp, vp, dop, mask, 64, 64, 1 / math.sqrt(128), key_valid=valid)
+    for t, w in zip((q, k, v), (wq, wk, wv)):
+        w_thw = O.rearrange_3d_block_to_thw(w, shape, chunk)
+        err = (t.grad.cpu().float() - w_thw).abs()
+        assert float(err.max()) <= 2.0 ** -6 * 4 * float(w_thw.abs().max()), float(err.max())
+        assert float(err.mean()) <= 2.0 ** -6 * float(w_thw.abs().mean())
+
+
 @pytest.mark.parametrize("dtype,lq,lk,chunk_q,chunk_k,token_major", [
     (torch.bfloat16, (8, 8, 16), (8, 8, 16), (4, 4, 4), (4, 4, 4), False),      # no padding
     (torch.bfloat16, (6, 10, 13), (6, 10, 13), (4, 4, 4), (4, 4, 4), True),     # padding on all axes, views of a projection
