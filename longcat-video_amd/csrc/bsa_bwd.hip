@@ -1,4 +1,7 @@
-// Block-sparse flash-attention backward for gfx950 (bf16 / fp16 MFMA), blocked-order tensors.
+// Block-sparse flash-attention backward for gfx950 (bf16 / fp16 MFMA).  The kernels work on blocked-order q, k_s, v,
+// dO; the caller's tensors are either in blocked order too (launch_bwd without `thw`) or in (T, H, W) token order, in
+// which case the two small passes read o, dO, lse and k through row tables and the kernels store every gradient row
+// at its token (BwdThw, BwdStore).
 //
 // Follows the reference's backward (bsa_interface.py:341-461; kernels flash_attn_bsa_varlen_mask.py:288-360
 // for dK/dV and :428-462 for dQ, wrappers :630-642 and :943-945) with the same rounding points:
@@ -193,7 +196,7 @@ __device__ __forceinline__ V8 pack8(const f32x16& x, int s) {
 // V rows of a half tile (32 keys x 256 B each, as they lie in memory - no fragment-order copies) go from global
 // memory straight into the wavefront's own LDS (global_load_lds_dwordx4, two stages of 16 KB: one being read, one on
 // its way, completion counted by hand), the row fragments come from there with ds_read_b128 and the transposed K_s
-// fragments with ds_read_b64_tr_b16 (slot p of row r holds 16-byte unit p ^ f(r), f(r) = ((r << 1) & 14) | ((r >> 3) & 1),
+// fragments with ds_read_b64_tr_b16 (slot p of row r holds 16-byte unit p ^ f(r), f(r) = ((r & 3) << 2) | ((r >> 2) & 3),
 // applied on the global side of the DMA, so that neither kind of read collides on a bank).  That leaves the registers
 // for two sets of S^T / dP^T accumulators, so the products of the next half are issued between the exponentials of
 // this one: the wavefront has its SIMD to itself and nothing else fills the MFMA pipe while it computes
@@ -286,7 +289,7 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int row = 4 * i + (lane >> 4);                                     // + 16 j
-        const int f = ((row << 1) & 14) | ((row >> 3) & 1);
+        const int f = ((row & 3) << 2) | ((row >> 2) & 3);
         voff[i] = (uint32_t)(row * 256 + (((lane & 15) ^ f) << 4));
     }
     uint32_t hv_ahead = ~0u;                     // validity of the keys of the half tile requested last
@@ -305,7 +308,7 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
             }
     };
     // ---- LDS -> fragments
-    const uint32_t fl = (uint32_t)(((lr << 1) & 14) | ((lr >> 3) & 1));
+    const uint32_t fl = (uint32_t)(((lr & 3) << 2) | ((lr >> 2) & 3));
     uint32_t roff[8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) roff[c] = (uint32_t)(lr * 256) + ((((uint32_t)(2 * c + lh)) ^ fl) << 4);
@@ -315,7 +318,7 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
     for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int hi = 0; hi < 2; ++hi)
-            toff[t][hi] = (uint32_t)((4 * lh + tx + 8 * hi) * 256) + ((((uint32_t)(4 * t + 2 * g1 + ty)) ^ (uint32_t)((8 * lh + 2 * tx) | hi)) << 4) +
+            toff[t][hi] = (uint32_t)((4 * lh + tx + 8 * hi) * 256) + ((((uint32_t)(4 * t + 2 * g1 + ty)) ^ (uint32_t)((4 * tx) | (lh + 2 * hi))) << 4) +
                           (uint32_t)(tz * 8);
     V8 kt[8];                                    // the transposed K_s fragments of the half whose dQ products come next
     auto take_transposed = [&](int hp) {
@@ -455,7 +458,7 @@ __global__ __launch_bounds__(64) void bwd_dq_lds_kernel(const T* __restrict__ q,
 // once instead of twice (128 MFMAs per tile pair instead of 160), and no fragment-order copy of q or dO is made.
 // The LDS side of the DMA is linear in the lane index, so the swizzle that keeps both kinds of read free of bank
 // conflicts is applied on the global side: the 16-byte slot p of row r receives unit p ^ f(r),
-// f(r) = ((r << 1) & 14) | ((r >> 3) & 1): 16 consecutive rows, and the 4 consecutive rows of a transposing read,
+// f(r) = ((r & 3) << 2) | ((r >> 2) & 3): 16 consecutive rows, and the 4 rows x 4 units of a transposing read's 32 lanes,
 // land on different banks.
 constexpr int kBwdHalfTile = kTileBytes / 2;                 // 32 query rows of Q or of dO
 constexpr int kBwdStats = 1024;                              // M2 (128 B), delta (128 B), the rest filled blindly by the 64-lane DMA
@@ -542,7 +545,7 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int row = 4 * i + (lane >> 4);                                     // + 16 j
-        const int f = ((row << 1) & 14) | ((row >> 3) & 1);
+        const int f = ((row & 3) << 2) | ((row >> 2) & 3);
         voff[i] = (uint32_t)(row * 256 + (((lane & 15) ^ f) << 4));
     }
     const uint32_t stat_gap = (uint32_t)(reinterpret_cast<const char*>(m2) - reinterpret_cast<const char*>(delta));
@@ -566,7 +569,7 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
     };
 
     // ---- LDS -> fragments
-    const uint32_t fl = (uint32_t)(((lr << 1) & 14) | ((lr >> 3) & 1));
+    const uint32_t fl = (uint32_t)(((lr & 3) << 2) | ((lr >> 2) & 3));
     uint32_t roff[8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) roff[c] = (uint32_t)(lr * 256) + ((((uint32_t)(2 * c + lh)) ^ fl) << 4);
@@ -576,7 +579,7 @@ __global__ __launch_bounds__(128) void bwd_dkdv_kernel(const T* __restrict__ q, 
     for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int hi = 0; hi < 2; ++hi)
-            toff[t][hi] = (uint32_t)((4 * lh + tx + 8 * hi) * 256) + ((((uint32_t)(4 * t + 2 * g1 + ty)) ^ (uint32_t)((8 * lh + 2 * tx) | hi)) << 4) +
+            toff[t][hi] = (uint32_t)((4 * lh + tx + 8 * hi) * 256) + ((((uint32_t)(4 * t + 2 * g1 + ty)) ^ (uint32_t)((4 * tx) | (lh + 2 * hi))) << 4) +
                           (uint32_t)(tz * 8);
     auto frag_tr_lds = [&](const char* part, int st2, int t) -> V8 {
         const char* base = part + (16 * st2) * 256;

@@ -14,7 +14,8 @@ Differences from the reference, all supersets:
     (bsa_interface.py:639-640);
   * block indices are int32 inside the engine; the helpers that the reference
     returns int64 from (torch.topk) convert on the way out;
-  * forward only: inputs that require grad are rejected while grad mode is on;
+  * gradients flow for bf16 / fp16 inputs (the reference's backward, bsa_interface.py:570-596); fp32 inputs that
+    require a gradient are rejected while grad mode is on;
   * the CDF selection rule (bsa_interface.py:226-266) keeps its weights in fp32 and its running sum in double
     for every storage type, and ``get_select_indices_from_score`` takes the ``sm_scale`` the reference forgets
     to pass on (bsa_interface.py:283, 285).
