@@ -347,6 +347,7 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
     constexpr int kOutPitch = kD + 8;
     __shared__ __attribute__((aligned(16))) T ost[kTile * kOutPitch];
     __shared__ uint32_t lists[2][kPipeList];
+    __shared__ int32_t out_rows[2][kTile];       // token rows of this and the next item's 64 query slots (row table given)
     __shared__ __attribute__((aligned(16))) char qstage[kTileBytes];      // Q of the next item, in register order
     uint32_t* const big = reinterpret_cast<uint32_t*>(ost);
 
@@ -709,6 +710,7 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
             const int32_t* list = idx + ((int64_t)bh * nbq + qblock) * idx_stride;
             int lane_now = lane;                                     // see the epilogue
             asm volatile("" : "+v"(lane_now));
+            if (L.q_rows != nullptr) out_rows[list_buf][lane_now] = L.q_rows[qrow0 + lane_now];
             for (int e = lane_now; e < nent; e += 64) big[e] = (uint32_t)list[e];
             ents = big;
             __syncthreads();
@@ -819,7 +821,10 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
 #pragma unroll
                 for (int e = 0; e < kPipeList / 64; ++e)
                     if (64 * e < next_nent)
-                        load_to_lds_4(nlist, (uint32_t)min(lane + 64 * e, next_nent - 1) * 4u, lds_address(&lists[list_buf ^ 1][64 * e]));
+                        load_to_lds_4(nlist, (uint32_t)min(lane + 64 * e, next_nent - 1) * 4u, (uint32_t)uni((int)lds_address(&lists[list_buf ^ 1][64 * e])));
+                // and the token rows of its 64 query slots, which its epilogue stores through
+                if (L.q_rows != nullptr)
+                    load_to_lds_4(L.q_rows + nqrow0, (uint32_t)lane * 4u, (uint32_t)uni((int)lds_address(&out_rows[list_buf ^ 1][0])));
                 const int64_t nq_bh = (int64_t)(nbh / Hn) * L.q_st[0] + (int64_t)(nbh % Hn) * L.q_st[1];
                 const char* qsrc = reinterpret_cast<const char*>(q + nq_bh);
 #pragma unroll
@@ -876,7 +881,7 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
             inv[qq] = l > 0.f ? 1.0f / l : 0.f;
             if (lse != nullptr && lh == 0) {
                 int64_t row = qrow0 + 32 * qq + lr;
-                if (L.q_rows != nullptr) row = L.q_rows[row];
+                if (L.q_rows != nullptr) row = out_rows[list_buf][32 * qq + lr];
                 if (row >= 0) lse[(int64_t)bh * lse_S + row] = l > 0.f ? (m_i[qq] + __builtin_log2f(l)) * kLn2 : -INFINITY;
             }
         }
@@ -906,7 +911,7 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
             for (int i = 0; i < 16; ++i) {
                 const int r = kr + 4 * i;
                 int64_t row = qrow0 + r;
-                if (L.q_rows != nullptr) row = L.q_rows[row];
+                if (L.q_rows != nullptr) row = out_rows[list_buf][r];
                 if (row >= 0)
                     *reinterpret_cast<uint4*>(o + o_bh + row * L.o_st[2] + kc * 8) =
                         *reinterpret_cast<const uint4*>(ost + r * kOutPitch + kc * 8);
