@@ -309,7 +309,8 @@ int bsa_bwd_3d(const bsa_3d_params* p,
  *     covers, in bf16 with 4x4x4 chunks, the 720p grid at up to 6 heads or the 480p grid at up to 17 heads:
  *     one GPU's share of a head-sharded layer).
  *   - The call itself makes no hipMalloc / hipFree and calls no allocating library routine.  The first call
- *     on a device looks up the buffer's address (hipGetSymbolAddress); make that call outside graph capture.
+ *     on a device is also the set-up for that device: it looks up the buffer's address (hipGetSymbolAddress) and
+ *     creates the one event that later calls record; make that call outside graph capture.
  *   - All calls on one GPU share the one buffer, which keeps the previous call's contents; nothing in it
  *     needs to start at zero.  Calls that overlap in time on one GPU would race on it: serialise them, or use
  *     bsa_fwd_3d with one workspace per stream.  A call made while the previous call on the same GPU, enqueued

@@ -684,8 +684,15 @@ int static_scratch(void** out) {
     if (dev < 0 || dev >= kMaxDevices) return set_error(BSA_ERR_UNSUPPORTED, "fwd_3d_static: device %d beyond the %d supported", dev, kMaxDevices);
     void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
     if (ptr == nullptr) {
+        // set-up, once per device: the buffer's address on this device and the event that later calls record
         e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
         if (e != hipSuccess || ptr == nullptr) return hip_fail(e, "fwd_3d_static: hipGetSymbolAddress(scratch)");
+        StaticUse& use = g_static_use[dev];
+        std::lock_guard<std::mutex> lock(use.mu);
+        if (use.done == nullptr && (e = hipEventCreateWithFlags(&use.done, hipEventDisableTiming)) != hipSuccess) {
+            use.done = nullptr;
+            return hip_fail(e, "fwd_3d_static: hipEventCreateWithFlags");
+        }
         // two threads racing here look up the same address for the same device
         g_scratch_ptr[dev].store(ptr, std::memory_order_release);
     }
@@ -760,10 +767,6 @@ int bsa_fwd_3d_static(const bsa_3d_params* p, const void* q, const int64_t q_str
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     const bool capturing = hipStreamIsCapturing((hipStream_t)stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone;
     if (!capturing) {
-        if (use.done == nullptr && hipEventCreateWithFlags(&use.done, hipEventDisableTiming) != hipSuccess) {
-            use.done = nullptr;
-            return set_error(BSA_ERR_HIP, "fwd_3d_static: hipEventCreateWithFlags");
-        }
         if (use.pending && use.stream != (hipStream_t)stream) {
             const hipError_t q_state = hipEventQuery(use.done);
             (void)hipGetLastError();                   // "not ready" is an answer, not a failure to be found later
