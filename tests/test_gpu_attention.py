@@ -277,6 +277,53 @@ def test_random_lists_lengths_and_masks(seed):
     assert torch.all(torch.isinf(lse[~fin]) & (lse[~fin] < 0)) and torch.all(o[~fin] == 0)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_items_with_and_without_a_norm_bound_side_by_side(dtype):
+    """The fragment-order kernel runs a launch's work items several per workgroup, each prepared by the one before it,
+    without row maxima where |q| |k| bounds the logits; an item without such a bound is left to a last launch of the
+    exact kernel, and the item after it starts from scratch.  6 400 work items (every workgroup runs six or seven), of
+    which every third query block has rows 40 times the usual size, some lists are empty and some are short: against
+    the LDS-tiled kernel on every row (a different summation order: 1.6e-2 / 1e-3) and against the oracle on sampled
+    query blocks of both kinds."""
+    bi = I()
+    H, nbq, nbk, width = 5, 1280, 96, 6
+    g = torch.Generator().manual_seed(61)
+    q = torch.randn(1, H, nbq * 64, 128, generator=g)
+    k = torch.randn(1, H, nbk * 64, 128, generator=g)
+    v = torch.randn(1, H, nbk * 64, 128, generator=g)
+    big = (torch.arange(nbq) % 3 == 1).repeat_interleave(64).view(1, 1, -1, 1)
+    q = torch.where(big, q * 40.0, q).to(dtype)
+    k, v = k.to(dtype), v.to(dtype)
+    idx = torch.stack([torch.randperm(nbk, generator=g)[:width].sort().values for _ in range(H * nbq)]).view(1, H, nbq, width).int()
+    lens = torch.full((1, H, nbq), width, dtype=torch.int32)
+    lens[:, :, 5::17] = 0
+    lens[:, :, 7::23] = 2
+    outs = {}
+    for kern in ("fragment", "lds"):
+        o, lse = bi.attn_fwd_bsa_varlen(q.cuda(), k.cuda(), v.cuda(), 1 / math.sqrt(128), idx.cuda(), lens.cuda(), 64, 64, kernel=kern)
+        torch.cuda.synchronize()
+        outs[kern] = (o.cpu(), lse.cpu())
+    o, lse = outs["fragment"]
+    o2, lse2 = outs["lds"]
+    assert torch.isfinite(o.float()).all()
+    d = (o.float() - o2.float()).abs()
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10       # a nearly one-hot row gives one row of v: one ulp of its size
+    assert bool((d <= 1.6e-2 + ulp * o2.float().abs()).all()) and float(d.mean()) <= 1e-3, (float(d.max()), float(d.mean()))
+    fin = torch.isfinite(lse2)
+    assert torch.equal(torch.isfinite(lse), fin) and torch.allclose(lse[fin], lse2[fin], rtol=1e-4, atol=2e-3)
+    empty = (lens == 0).repeat_interleave(64, dim=-1)
+    assert torch.all(o[empty] == 0)
+    # the oracle on a few query blocks of each kind, first and last work items included
+    for h, m in ((0, 0), (0, 1), (1, 4), (2, 640), (3, 1024), (4, 1278), (4, 1279), (2, 7), (1, 5)):
+        rows = slice(64 * m, 64 * m + 64)
+        want, want_lse = O.masked_dense_attention(q[:, h:h + 1, rows], k[:, h:h + 1], v[:, h:h + 1],
+                                                  O.block_mask_from_indices(idx[:, h:h + 1, m:m + 1].long(), lens[:, h:h + 1, m:m + 1], nbk),
+                                                  64, 64, 1 / math.sqrt(128))
+        close(o[:, h:h + 1, rows], want, dtype)
+        f = torch.isfinite(want_lse)
+        assert torch.allclose(lse[:, h:h + 1, rows][f], want_lse[f], rtol=1e-4, atol=2e-3)
+
+
 @pytest.mark.parametrize("case", ["scaled", "late", "late_within_bound", "nan_free_zero_keys"])
 def test_thw_kernel_keeps_its_exponentials_finite(case):
     """The (T,H,W)-order kernel raises its running maximum lazily and rescales its accumulators a quarter of a step
