@@ -907,15 +907,27 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
             int lane_now = lane;
             asm volatile("" : "+v"(lane_now));
             const int kc = lane_now & 15, kr = lane_now >> 4;
+            // in three sweeps - the sixteen token rows, the sixteen pieces, the stores - so that the LDS reads are all
+            // on their way before the first is waited for (row by row, every store sat behind two LDS round trips)
+            int32_t rows[16];                         // relative to qrow0 without a row table
+            u32x4 pieces[16];
+            if (L.q_rows != nullptr) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int r = kr + 4 * i;
-                int64_t row = qrow0 + r;
-                if (L.q_rows != nullptr) row = out_rows[list_buf][r];
-                if (row >= 0)
-                    *reinterpret_cast<uint4*>(o + o_bh + row * L.o_st[2] + kc * 8) =
-                        *reinterpret_cast<const uint4*>(ost + r * kOutPitch + kc * 8);
+                for (int i = 0; i < 16; ++i) rows[i] = out_rows[list_buf][kr + 4 * i];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) rows[i] = kr + 4 * i;
             }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(rows[i]));
+            const int64_t row_base = L.q_rows != nullptr ? 0 : qrow0;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) pieces[i] = *reinterpret_cast<const u32x4*>(ost + (kr + 4 * i) * kOutPitch + kc * 8);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(pieces[i]));      // read here, not inside the branches below
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                if (rows[i] >= 0) *reinterpret_cast<u32x4*>(o + o_bh + (row_base + rows[i]) * L.o_st[2] + kc * 8) = pieces[i];
         }
         }   // run
         // ---- on to the next item
