@@ -483,18 +483,21 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
         if (kNsub1) return tile_base + (uint32_t)blk;
         return tile_base + (uint32_t)(blk * nsub + tp % nsub);
     };
-    auto entry_mask = [&](int tp, uint32_t tile) -> uint64_t {
-        uint32_t lo = ~0u, hi = ~0u;
-        if (tile_valid != nullptr) {
-            // the same word in every lane; made a scalar by hand (behind the stores of an earlier item's output the
-            // compiler reads it with a vector load)
-            const uint64_t word = tile_valid[tp >= ntiles ? 0u : tile - tile_base];     // behind the list: another head's tile
-            lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)word);
-            hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(word >> 32));
-        }
+    // the validity word of a tile (all keys valid without padding), in two steps so that a caller can ask for several
+    // words before it waits for the first
+    auto entry_word = [&](int tp, uint32_t tile) -> uint64_t {
+        if (tile_valid == nullptr) return ~0ull;
+        return tile_valid[tp >= ntiles ? 0u : tile - tile_base];                        // behind the list: another head's tile
+    };
+    auto mask_of = [&](int tp, uint64_t word) -> uint64_t {
+        // the same word in every lane; made a scalar by hand (behind the stores of an earlier item's output the
+        // compiler reads it with a vector load)
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)word);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(word >> 32));
         const uint32_t keep = tp >= ntiles ? 0u : ~0u;
         return (uint64_t)(lo & keep) | ((uint64_t)(hi & keep) << 32);
     };
+    auto entry_mask = [&](int tp, uint32_t tile) -> uint64_t { return mask_of(tp, entry_word(tp, tile)); };
     // accumulator i <-> key 8 (i / 4) + 4 lh + i % 4 of the step's 32 keys, query lr (+32)
     auto mask_pair = [&](f32x16 (&sv)[2], uint32_t half) {
         if (__builtin_expect(half != ~0u, 0)) {
@@ -735,10 +738,18 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
 
         bool run = true;                     // this kernel computes the item (see the bound on q . k below)
         if (ntiles > 0) {
+            {
+                // the three entries, then the three words, each kind in one sweep: one wait per kind instead of three
+                uint32_t raw3[3];
+                uint64_t word3[3];
 #pragma unroll
-            for (int r = 0; r < 3; ++r) {
-                w_tile[r] = entry_tile(r, entry_raw(r));
-                w_mask[r] = entry_mask(r, w_tile[r]);
+                for (int r = 0; r < 3; ++r) raw3[r] = entry_raw(r);
+#pragma unroll
+                for (int r = 0; r < 3; ++r) w_tile[r] = entry_tile(r, raw3[r]);
+#pragma unroll
+                for (int r = 0; r < 3; ++r) word3[r] = entry_word(r, w_tile[r]);
+#pragma unroll
+                for (int r = 0; r < 3; ++r) w_mask[r] = mask_of(r, word3[r]);
             }
             // ---- prologue.  In flight when the loop starts: K(1), K(2), V_A(0), V_B(0), V_A(1); the ring slot of
             // V_B(1) holds zeros, which the first step multiplies with P = 0 (there is no step -1).  A prepared item
@@ -771,7 +782,7 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
 #pragma unroll
                 for (int qq = 0; qq < 2; ++qq) {
                     const int64_t row = nqrow0 + 32 * qq + lr;
-                    next_rows[qq] = L.q_rows != nullptr ? max(L.q_rows[row], 0) : (int32_t)row;
+                    next_rows[qq] = L.q_rows != nullptr ? L.q_rows[row] : (int32_t)row;      // used (and clamped) behind S(0): no wait here
                 }
             }
 #pragma unroll
@@ -829,7 +840,7 @@ __global__ __launch_bounds__(64) void fwd_frag_kernel(
                 const char* qsrc = reinterpret_cast<const char*>(q + nq_bh);
 #pragma unroll
                 for (int qq = 0; qq < 2; ++qq) {
-                    const uint32_t voff = (uint32_t)next_rows[qq] * (uint32_t)(L.q_st[2] * 2) + (uint32_t)(16 * lh);
+                    const uint32_t voff = (uint32_t)max(next_rows[qq], 0) * (uint32_t)(L.q_st[2] * 2) + (uint32_t)(16 * lh);   // padded slots read token 0
 #pragma unroll
                     for (int c = 0; c < 8; ++c) load_to_lds_16(qsrc + 32 * c, voff, lds_address(qstage + (qq * 8 + c) * 1024));
                 }
