@@ -230,6 +230,36 @@ def test_the_token_order_backward_equals_the_rearranging_route(dtype, lq, lk, ch
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_random_grids_through_both_backward_routes(seed):
+    """Random grids, chunk shapes, batch and head counts, selection rules and storage types: bsa_bwd_3d against the
+    rearranging route, bit for bit, and both finite."""
+    bi = I()
+    rnd = np.random.default_rng(100 + seed)
+    chunk_q = [(4, 4, 4), (2, 4, 8), (4, 4, 8), (1, 8, 8)][rnd.integers(0, 4)]
+    chunk_k = [(4, 4, 4), (2, 4, 8), (4, 4, 8)][rnd.integers(0, 3)]
+    lq = tuple(int(rnd.integers(c, 4 * c + 2)) for c in chunk_q)
+    lk = lq if rnd.integers(0, 2) else tuple(int(rnd.integers(c, 4 * c + 2)) for c in chunk_k)
+    B, H = int(rnd.integers(1, 3)), int(rnd.integers(1, 4))
+    dtype = [torch.bfloat16, torch.float16][rnd.integers(0, 2)]
+    sparsity = [0.0, 0.5, 0.8][rnd.integers(0, 3)]
+    cdf = None if rnd.integers(0, 3) else 0.7
+    g = torch.Generator().manual_seed(200 + seed)
+    Sq, Sk = int(np.prod(lq)), int(np.prod(lk))
+    q = torch.randn(B, H, Sq, 128, generator=g).to(dtype).cuda()
+    k, v = (torch.randn(B, H, Sk, 128, generator=g).to(dtype).cuda() for _ in range(2))
+    do = torch.randn(B, H, Sq, 128, generator=g).to(dtype).cuda()
+    o, walk, lens, lse = bi._bsa_3d(q, k, v, lq, lk, sparsity, chunk_q, chunk_k, cdf_threshold=cdf, for_backward=True)
+    if walk.shape[3] == 0:
+        pytest.skip("no block selected at this size")
+    args = (do, q, k, v, o, lse, walk, lens, lq, lk, chunk_q, chunk_k, 1 / math.sqrt(128))
+    got = bi._bsa_3d_backward(*args)
+    want = bi._bsa_3d_backward_by_rearranging(*args)
+    for a, b, name in zip(got, want, ("dq", "dk", "dv")):
+        assert torch.isfinite(a.float()).all(), (name, lq, lk, chunk_q, chunk_k)
+        assert torch.equal(a, b), (name, lq, lk, chunk_q, chunk_k, float((a.float() - b.float()).abs().max()))
+
+
 def test_argument_checks():
     from longcat_video_amd import _capi
     lib = _capi.load()
