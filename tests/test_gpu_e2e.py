@@ -106,6 +106,27 @@ def test_chunk_shapes_on_ragged_grids(latent, chunk):
     assert torch.isfinite(o.float()).all()
 
 
+@pytest.mark.parametrize("latent,chunk", [
+    ((8, 16, 16), (4, 8, 8)),    # 256 tokens per chunk: the case the reference gives to its second kernel
+    ((9, 10, 11), (8, 8, 4)),    # the same on a grid that is ragged in every direction
+    ((8, 16, 16), (8, 8, 8)),    # 512 tokens per chunk
+    ((5, 12, 20), (2, 12, 8)),   # 192 tokens: a multiple of 64 that is no power of two
+])
+def test_chunks_above_128_tokens(latent, chunk):
+    """The reference switches to another kernel when a KV chunk holds more than 128 tokens
+    (bsa_interface.py:311-313, flash_attn_bsa_varlen_mask.py:35-153: the chunk in steps of BLOCK_N keys, same
+    arithmetic).  Here the same kernels take every chunk that is a multiple of 64 tokens."""
+    S = int(np.prod(latent))
+    q, k, v = seeded_qkv(38, 1, 2, S, S, 128, torch.bfloat16)
+    o, idx, lens, score = I()._bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, 0.5, chunk, chunk, True)
+    nb = int(np.prod(O.block_grid(latent, chunk)))
+    check_against_oracle(q, k, v, latent, latent, 0.5, o, idx, lens, score, q_blocks=range(nb), chunk=chunk)
+    assert torch.isfinite(o.float()).all()
+    pub = I().flash_attn_bsa_3d(q.cuda(), k.cuda(), v.cuda(), latent, latent, sparsity=0.5,
+                                chunk_3d_shape_q=list(chunk), chunk_3d_shape_k=list(chunk))
+    assert torch.equal(pub, o)
+
+
 def test_strided_inputs_on_a_ragged_grid():
     """q, k, v as views of one [B, S, 3, H, D] projection output and o written into a [B, S, H, D]
     buffer, on a grid with padded chunks in every direction."""
